@@ -1,0 +1,198 @@
+/* C ABI of libsubstation_amd.so: the fused BERT encoder layer (forward and
+ * backward) on AMD MI355X (gfx950).
+ *
+ * Drop-in for the four symbols the reference's JIT-compiled encoder.so exports
+ * (pytorch_module/encoder.cu:304-318) and that pytorch_module/encoder.py:395-403
+ * binds with ctypes.  The reference bakes sizes, layouts, dtype and dropout
+ * probabilities into the library at compile time (encoder.py:213-376); this
+ * library is prebuilt, so the same information arrives through sub_config.
+ *
+ * All tensors are dense fp16 device buffers owned by the caller, laid out
+ * row-major in the dimension order given by their layout string.  Functions
+ * returning int give 0 on success and a negative value on error, with the
+ * message available from sub_last_error(); nothing aborts the process (the
+ * reference's CHECK macro does, pytorch_module/all.cuh:7-13).  A handle must
+ * not be used from two threads at once (it carries the RNG step, like the
+ * reference's GlobalRandomState, pytorch_module/blocks.cuh:48-51).  Kernels are
+ * enqueued on the stream set with sub_set_stream (default: the null stream) and
+ * are not synchronised (as pytorch_module/encoder.cu:156,298).
+ */
+#ifndef SUBSTATION_AMD_H
+#define SUBSTATION_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SUB_ABI_VERSION 1
+#define SUB_N_PARAMS 12   /* WKQV BKQV WO BO S1 B1 LINB1 LINW1 S2 B2 LINB2 LINW2 */
+#define SUB_N_FWD 23      /* forward intermediates, pytorch_module/encoder.py:81 */
+#define SUB_N_BWD 14      /* backward intermediates, pytorch_module/encoder.py:111 */
+
+#define SUB_DTYPE_F16 0
+#define SUB_ACT_RELU 0
+#define SUB_ACT_GELU 1    /* tanh form, substation/transformer.py:11-14 */
+
+/* Dropout sites (word 2 of the Philox counter). */
+#define SUB_SITE_SOFTMAX 0
+#define SUB_SITE_RESID1 1
+#define SUB_SITE_ACT 2
+#define SUB_SITE_RESID2 3
+
+/* What pytorch_module/encoder.py:213-376 writes into encoder_parameters.cuh.
+ * Names and layouts are listed in the order in which the caller will pass the
+ * pointers (the order of the lists in the layouts pickle, encoder.py:229-264).
+ * Dimension letters: B batch, J/K query/key position, H heads, P head size,
+ * I embedding, U feed-forward width, Q stack index (0=K, 1=Q, 2=V). */
+typedef struct sub_config {
+    int32_t abi_version;            /* SUB_ABI_VERSION */
+    int32_t batch, seq, heads, embed;
+    int32_t intermediate;           /* 0 means 4*embed (encoder.py:33) */
+    int32_t dtype;                  /* SUB_DTYPE_F16 */
+    int32_t activation;             /* SUB_ACT_* */
+    float p_softmax, p_resid1, p_act, p_resid2;
+    float ln_eps;                   /* 0 means 1e-5 (block_bdrln.cuh:258) */
+    uint64_t seed;
+    const char* input_layout;       /* of X, a permutation of "BJI" */
+    const char* output_layout;      /* of SB2 */
+    const char* param_names[SUB_N_PARAMS];
+    const char* param_layouts[SUB_N_PARAMS];
+    const char* fwd_names[SUB_N_FWD];
+    const char* fwd_layouts[SUB_N_FWD];
+    const char* bwd_names[SUB_N_BWD];
+    const char* bwd_layouts[SUB_N_BWD];
+} sub_config;
+
+/* ---- the reference's four exports (pytorch_module/encoder.cu:304-318) ------ */
+
+/* encoder.cu:304 `Encoder* init()`.  Returns an unconfigured handle (NULL on
+ * failure); call sub_configure before use, or use init_cfg. */
+void* init(void);
+
+/* encoder.cu:316 `void destroy(Encoder*)`. */
+void destroy(void* handle);
+
+/* encoder.cu:308 `void encoder_forward(Encoder*, ENCODER_FORWARD_DEF)`:
+ * X, the 12 parameters, the 23 forward intermediates, Y (encoder.py:88-93). */
+int encoder_forward(void* handle, void* X,
+                    void* w0, void* w1, void* w2, void* w3, void* w4, void* w5,
+                    void* w6, void* w7, void* w8, void* w9, void* w10, void* w11,
+                    void* f0, void* f1, void* f2, void* f3, void* f4, void* f5, void* f6, void* f7,
+                    void* f8, void* f9, void* f10, void* f11, void* f12, void* f13, void* f14,
+                    void* f15, void* f16, void* f17, void* f18, void* f19, void* f20, void* f21,
+                    void* f22, void* Y);
+
+/* encoder.cu:312 `void encoder_backward(Encoder*, ENCODER_BACKWARD_DEF)`:
+ * DY, 12 parameter gradients, 14 backward intermediates, 12 parameters,
+ * 23 forward intermediates, X, DX (encoder.py:124-130). */
+int encoder_backward(void* handle, void* DY,
+                     void* dw0, void* dw1, void* dw2, void* dw3, void* dw4, void* dw5,
+                     void* dw6, void* dw7, void* dw8, void* dw9, void* dw10, void* dw11,
+                     void* b0, void* b1, void* b2, void* b3, void* b4, void* b5, void* b6,
+                     void* b7, void* b8, void* b9, void* b10, void* b11, void* b12, void* b13,
+                     void* w0, void* w1, void* w2, void* w3, void* w4, void* w5,
+                     void* w6, void* w7, void* w8, void* w9, void* w10, void* w11,
+                     void* f0, void* f1, void* f2, void* f3, void* f4, void* f5, void* f6, void* f7,
+                     void* f8, void* f9, void* f10, void* f11, void* f12, void* f13, void* f14,
+                     void* f15, void* f16, void* f17, void* f18, void* f19, void* f20, void* f21,
+                     void* f22, void* X, void* DX);
+
+/* ---- configuration (replaces the generated encoder_parameters.cuh) --------- */
+
+void* init_cfg(const sub_config* cfg);               /* init() + sub_configure() */
+int sub_configure(void* handle, const sub_config* cfg);
+int sub_set_stream(void* handle, void* hip_stream);  /* hipStream_t */
+/* Dropout masks are a pure function of (seed, site, step, element); step is
+ * incremented by every encoder_forward (blocks.cuh:48-51 advances an offset). */
+int sub_set_rng(void* handle, uint64_t seed, uint32_t step);
+const char* sub_last_error(void);
+
+/* Array forms of the two calls above: ptrs holds the same pointers in the same
+ * order, without the handle (n must be 37 resp. 64). */
+int sub_encoder_forward(void* handle, void* const* ptrs, int n);
+int sub_encoder_backward(void* handle, void* const* ptrs, int n);
+
+/* Per-operator timing with HIP events on the handle's stream; the counterpart
+ * of the NVTX ranges of encoder.cu:32-53.  sub_profile_read waits for the
+ * stream and returns the number of operators of the last forward/backward call
+ * (at most cap are written). */
+int sub_profile_enable(void* handle, int on);
+int sub_profile_read(void* handle, int cap, const char** names, float* ms);
+
+/* ---- single operators (the units pytorch_module/benchmark.py times) -------- */
+/* Sizes come from the handle's configuration; every tensor takes its own layout
+ * string.  Vectors of parameters ([I], [U]) are dense. */
+
+/* block_softmax.cuh:127-188; `scale` multiplies the input (1 in the layer, where
+ * the factor is the GEMM's alpha, encoder.cu:116). */
+int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alpha,
+                   const char* l_alpha, void* mask, const char* l_mask, void* drop,
+                   const char* l_drop, float scale, float p, uint32_t site);
+/* block_bs.cuh:107-156 */
+int sub_op_bs(void* handle, const void* alpha, const char* l_alpha, const void* mask,
+              const char* l_mask, const void* ddrop, const char* l_ddrop, void* dbeta,
+              const char* l_dbeta, float scale);
+/* block_bdrln.cuh:287-352; lin may alias in (encoder.cu:134-135) */
+int sub_op_bdrln(void* handle, const void* in, const char* l_in, const void* resid,
+                 const char* l_resid, const void* linear_bias, const void* scale, const void* bias,
+                 void* lin, const char* l_lin, void* mask, const char* l_mask, void* diff,
+                 const char* l_diff, void* normed, const char* l_normed, void* out,
+                 const char* l_out, void* istd, const char* l_istd, float p, uint32_t site);
+/* block_blnrd.cuh:203-259 */
+int sub_op_blnrd(void* handle, const void* dout, const char* l_dout, const void* istd,
+                 const char* l_istd, const void* diff, const char* l_diff, const void* mask,
+                 const char* l_mask, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                 const char* l_d_drop_in);
+/* block_bad.cuh:87-145 */
+int sub_op_bad(void* handle, const void* in, const char* l_in, const void* bias, void* lin,
+               const char* l_lin, void* mask, const char* l_mask, void* out, const char* l_out,
+               float p, uint32_t site);
+/* block_bsb_ebsb.cuh:178-216 */
+int sub_op_bsb(void* handle, const void* in, const char* l_in, const void* scale, const void* dout,
+               const char* l_dout, void* din, const char* l_din, void* dscale, void* dbias);
+/* block_bsb_ebsb.cuh:376-420 */
+int sub_op_ebsb(void* handle, const void* in, const char* l_in, const void* scale,
+                const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                const void* dlinear, const char* l_dlinear, void* din, const char* l_din,
+                void* dscale, void* dbias, void* dlinear_bias);
+/* block_bdrlb.cuh:105-146 */
+int sub_op_bdrlb(void* handle, const void* ddrop, const char* l_ddrop, const void* mask,
+                 const char* l_mask, const void* lin, const char* l_lin, void* dlinear,
+                 const char* l_dlinear, void* dbias);
+/* block_baob.cuh:79-97 */
+int sub_op_baob(void* handle, const void* datt, const char* l_datt, void* dbo);
+/* block_aib.cuh:64-155, on the Q-stacked tensors */
+int sub_op_aib(void* handle, const void* in, const char* l_in, const void* bias, const char* l_bias,
+               void* out, const char* l_out);
+/* block_baib.cuh:161-211, on the Q-stacked tensors */
+int sub_op_baib(void* handle, const void* d, const char* l_d, void* dbias, const char* l_dbias);
+/* block_bei.cuh:58-106 */
+int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void* dresid1,
+               const char* l_dresid1, void* dx, const char* l_dx);
+/* gemm.cuh:134-147 `Einsum<Real, lA, lB, lC>::run`: C = alpha * einsum(A, B),
+ * dimension roles derived from the three layout strings (einsumparser.h:9-55). */
+int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
+                  void* C, const char* l_C, float alpha);
+
+/* ---- host-only helpers (no GPU needed) ------------------------------------- */
+
+/* metahelpers.h:61-78: element strides of `layout` for dims "BJKHPIUQ"
+ * (0 for absent dims) under the handle's sizes. */
+int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]);
+/* einsumparser.h:9-55.  out = {batch, M, N, K, sAM, sAK, sAB0, sBN, sBK, sBB0,
+ * sCM, sCN, sCB0, nbatchdims, K0, sAK0, sBK0, kernel_kind} */
+int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const char* l_C,
+                        int64_t out[18]);
+/* The 16-bit random fields of canonical elements start .. start+n-1, computed
+ * on the host by the same code the kernels run. */
+int sub_philox_fields_host(uint64_t seed, uint32_t site, uint32_t step, uint64_t start,
+                           uint64_t n, uint16_t* out);
+/* Drop threshold used for probability p: keep iff field >= threshold. */
+uint32_t sub_dropout_threshold(float p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SUBSTATION_AMD_H */

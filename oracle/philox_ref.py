@@ -56,8 +56,9 @@ def philox4x32_10(counter, key):
 
 
 def threshold16(p):
-    """Drop threshold on the 16-bit field: round(p*65536) clamped to [0, 65536]."""
-    return int(min(65536, max(0, int(np.floor(float(p) * 65536.0 + 0.5)))))
+    """Drop threshold on the 16-bit field: round(p*65536) clamped to [0, 65536].
+    p is taken at float32 precision, the type the C ABI passes it in."""
+    return int(min(65536, max(0, int(np.floor(float(np.float32(p)) * 65536.0 + 0.5)))))
 
 
 def random16(n, seed, site, step=0, start=0):

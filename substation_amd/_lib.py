@@ -1,0 +1,189 @@
+"""ctypes binding of libsubstation_amd.so (declared in include/substation_amd.h).
+
+Takes the place of the ``ctypes.CDLL`` block at pytorch_module/encoder.py:395-403.
+There is no CPU fallback: if the library is missing, loading raises."""
+import ctypes
+import os
+
+from . import layouts as _lay
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, 'lib', 'libsubstation_amd.so')
+
+N_PARAMS, N_FWD, N_BWD = 12, 23, 14
+ABI_VERSION = 1
+ACTIVATIONS = {'relu': 0, 'gelu': 1}
+
+
+class SubConfig(ctypes.Structure):
+    _fields_ = [
+        ('abi_version', ctypes.c_int32),
+        ('batch', ctypes.c_int32), ('seq', ctypes.c_int32), ('heads', ctypes.c_int32),
+        ('embed', ctypes.c_int32), ('intermediate', ctypes.c_int32),
+        ('dtype', ctypes.c_int32), ('activation', ctypes.c_int32),
+        ('p_softmax', ctypes.c_float), ('p_resid1', ctypes.c_float),
+        ('p_act', ctypes.c_float), ('p_resid2', ctypes.c_float),
+        ('ln_eps', ctypes.c_float),
+        ('seed', ctypes.c_uint64),
+        ('input_layout', ctypes.c_char_p), ('output_layout', ctypes.c_char_p),
+        ('param_names', ctypes.c_char_p * N_PARAMS), ('param_layouts', ctypes.c_char_p * N_PARAMS),
+        ('fwd_names', ctypes.c_char_p * N_FWD), ('fwd_layouts', ctypes.c_char_p * N_FWD),
+        ('bwd_names', ctypes.c_char_p * N_BWD), ('bwd_layouts', ctypes.c_char_p * N_BWD),
+    ]
+
+
+_lib = None
+
+_VP, _CP, _F, _U32, _U64, _I = (ctypes.c_void_p, ctypes.c_char_p, ctypes.c_float, ctypes.c_uint32,
+                                ctypes.c_uint64, ctypes.c_int)
+
+#: every symbol include/substation_amd.h declares: name -> (restype, argtypes)
+SIGNATURES = {
+    'init': (_VP, []),
+    'destroy': (None, [_VP]),
+    'encoder_forward': (_I, [_VP] * (1 + 1 + N_PARAMS + N_FWD + 1)),
+    'encoder_backward': (_I, [_VP] * (1 + 1 + N_PARAMS + N_BWD + N_PARAMS + N_FWD + 1 + 1)),
+    'init_cfg': (_VP, [ctypes.POINTER(SubConfig)]),
+    'sub_configure': (_I, [_VP, ctypes.POINTER(SubConfig)]),
+    'sub_set_stream': (_I, [_VP, _VP]),
+    'sub_set_rng': (_I, [_VP, _U64, _U32]),
+    'sub_last_error': (_CP, []),
+    'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
+    'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
+    'sub_profile_enable': (_I, [_VP, _I]),
+    'sub_profile_read': (_I, [_VP, _I, ctypes.POINTER(_CP), ctypes.POINTER(_F)]),
+    'sub_op_softmax': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _U32]),
+    'sub_op_bs': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
+    'sub_op_bdrln': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP, _CP, _VP, _CP, _VP, _CP,
+                          _VP, _CP, _VP, _CP, _VP, _CP, _F, _U32]),
+    'sub_op_blnrd': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP]),
+    'sub_op_bad': (_I, [_VP, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _U32]),
+    'sub_op_bsb': (_I, [_VP, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _VP]),
+    'sub_op_ebsb': (_I, [_VP, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP]),
+    'sub_op_bdrlb': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP]),
+    'sub_op_baob': (_I, [_VP, _VP, _CP, _VP]),
+    'sub_op_aib': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
+    'sub_op_baib': (_I, [_VP, _VP, _CP, _VP, _CP]),
+    'sub_op_bei': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
+    'sub_op_einsum': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
+    'sub_layout_strides': (_I, [_VP, _CP, ctypes.POINTER(ctypes.c_int64)]),
+    'sub_einsum_classify': (_I, [_VP, _CP, _CP, _CP, ctypes.POINTER(ctypes.c_int64)]),
+    'sub_philox_fields_host': (_I, [_U64, _U32, _U32, _U64, _U64, ctypes.POINTER(ctypes.c_uint16)]),
+    'sub_dropout_threshold': (_U32, [_F]),
+}
+
+
+def load():
+    """Loads the prebuilt library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f'{LIB_PATH} is missing: build it with `python -m substation_amd.build` '
+            '(there is no fallback implementation)')
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+class SubstationError(RuntimeError):
+    pass
+
+
+def check(rc, what=''):
+    if rc is not None and rc < 0:
+        msg = load().sub_last_error()
+        raise SubstationError((what + ': ' if what else '') + (msg.decode() if msg else 'unknown error'))
+    return rc
+
+
+def make_config(batch_size, max_seq_len, num_heads, embedding_size, layouts, p_softmax=0.0,
+                p_resid1=0.0, p_act=0.0, p_resid2=0.0, activation='relu', seed=0,
+                intermediate_size=0, ln_eps=0.0):
+    """Builds a sub_config from a layouts dict (names/layouts in the dict's own
+    order, which is also the order the pointers are passed in)."""
+    _lay.validate(layouts)
+    if activation not in ACTIVATIONS:
+        raise ValueError('Unknown activation ' + str(activation))
+    c = SubConfig()
+    c.abi_version = ABI_VERSION
+    c.batch, c.seq, c.heads, c.embed = batch_size, max_seq_len, num_heads, embedding_size
+    c.intermediate = intermediate_size or 0
+    c.dtype = 0
+    c.activation = ACTIVATIONS[activation]
+    c.p_softmax, c.p_resid1, c.p_act, c.p_resid2 = p_softmax, p_resid1, p_act, p_resid2
+    c.ln_eps = ln_eps
+    c.seed = seed
+    c.input_layout = layouts['input'][1].encode()
+    c.output_layout = layouts['output'][1].encode()
+    for key, names, lays in (('params', c.param_names, c.param_layouts),
+                             ('forward_interm', c.fwd_names, c.fwd_layouts),
+                             ('backward_interm', c.bwd_names, c.bwd_layouts)):
+        for i, (n, l) in enumerate(layouts[key]):
+            names[i] = n.encode()
+            lays[i] = l.encode()
+    return c
+
+
+class Handle:
+    """Owns one native encoder handle."""
+
+    def __init__(self, config):
+        self.lib = load()
+        self._config = config       # keeps the char buffers alive
+        self.ptr = self.lib.init_cfg(ctypes.byref(config))
+        if not self.ptr:
+            msg = self.lib.sub_last_error()
+            raise SubstationError('init_cfg: ' + (msg.decode() if msg else 'failed'))
+
+    def close(self):
+        if getattr(self, 'ptr', None):
+            self.lib.destroy(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def set_stream(self, stream):
+        check(self.lib.sub_set_stream(self.ptr, ctypes.c_void_p(stream)), 'sub_set_stream')
+
+    def set_rng(self, seed, step=0):
+        check(self.lib.sub_set_rng(self.ptr, seed, step), 'sub_set_rng')
+
+    def profile_enable(self, on=True):
+        check(self.lib.sub_profile_enable(self.ptr, 1 if on else 0), 'sub_profile_enable')
+
+    def profile_read(self, cap=64):
+        names = (ctypes.c_char_p * cap)()
+        ms = (ctypes.c_float * cap)()
+        n = check(self.lib.sub_profile_read(self.ptr, cap, names, ms), 'sub_profile_read')
+        return [(names[i].decode(), float(ms[i])) for i in range(min(n, cap))]
+
+    def strides(self, layout):
+        out = (ctypes.c_int64 * 8)()
+        check(self.lib.sub_layout_strides(self.ptr, layout.encode(), out), 'sub_layout_strides')
+        return dict(zip('BJKHPIUQ', out))
+
+    def classify(self, la, lb, lc):
+        out = (ctypes.c_int64 * 18)()
+        check(self.lib.sub_einsum_classify(self.ptr, la.encode(), lb.encode(), lc.encode(), out),
+              'sub_einsum_classify')
+        keys = ('batch', 'M', 'N', 'K', 'sAM', 'sAK', 'sAB', 'sBN', 'sBK', 'sBB', 'sCM', 'sCN', 'sCB',
+                'nbatch', 'K0', 'sAK0', 'sBK0', 'kernel')
+        return dict(zip(keys, out))
+
+
+def philox_fields_host(seed, site, step, start, n):
+    import numpy as np
+    out = np.empty(n, dtype=np.uint16)
+    check(load().sub_philox_fields_host(seed, site, step, start, n,
+                                        out.ctypes.data_as(ctypes.POINTER(ctypes.c_uint16))))
+    return out

@@ -1,0 +1,821 @@
+// Encoder-layer orchestration and the C ABI of libsubstation_amd.so.
+// Counterpart of pytorch_module/encoder.cu (struct Encoder, the two operator
+// sequences and the four extern "C" exports); the compile-time configuration of
+// the generated encoder_parameters.cuh (pytorch_module/encoder.py:213-376) is
+// a run-time sub_config here.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/substation_amd.h"
+#include "sub_common.hpp"
+#include "sub_ops.hpp"
+
+namespace sub {
+
+namespace {
+
+thread_local std::string g_last_error;
+
+// ---------------------------------------------------------------------------
+// Tensor tables: names in the reference's pickle order and canonical dims.
+// ---------------------------------------------------------------------------
+struct TensorDef { const char* name; const char* dims; };
+
+const TensorDef kParams[SUB_N_PARAMS] = {
+    {"WKQV", "QPHI"}, {"BKQV", "QPH"}, {"WO", "IPH"}, {"BO", "I"}, {"S1", "I"}, {"B1", "I"},
+    {"LINB1", "U"}, {"LINW1", "IU"}, {"S2", "I"}, {"B2", "I"}, {"LINB2", "I"}, {"LINW2", "UI"}};
+const TensorDef kFwd[SUB_N_FWD] = {
+    {"KKQQVV", "QPHBJ"}, {"WKKWQQWVV", "QPHBJ"}, {"BETA", "HBJK"}, {"ALPHA", "HBJK"},
+    {"ATTN_DROP_MASK", "HBJK"}, {"ATTN_DROP", "HBJK"}, {"GAMMA", "PHBJ"}, {"ATT", "BJI"},
+    {"DROP1MASK", "BJI"}, {"SB1", "BJI"}, {"SB1_LINW1", "BJU"}, {"DROP2", "BJU"}, {"LIN1", "BJU"},
+    {"DROP2_LINW2", "BJI"}, {"LIN2", "BJI"}, {"LN2", "BJI"}, {"LN2STD", "BJ"}, {"LN2DIFF", "BJI"},
+    {"DROP2MASK", "BJU"}, {"DROP3MASK", "BJI"}, {"LN1", "BJI"}, {"LN1STD", "BJ"}, {"LN1DIFF", "BJI"}};
+const TensorDef kBwd[SUB_N_BWD] = {
+    {"DLN2", "BJI"}, {"DRESID2", "BJI"}, {"DLIN2", "BJI"}, {"DDROP2", "BJU"}, {"DLIN1", "BJU"},
+    {"DLIN1_LINW1", "BJI"}, {"DLN1", "BJI"}, {"DRESID1", "BJI"}, {"DATT", "BJI"}, {"DXATT", "BJI"},
+    {"DGAMMA", "PHBJ"}, {"DATTN_DROP", "HBJK"}, {"DBETA", "HBJK"}, {"DKKQQVV", "QPHBJ"}};
+
+enum P { WKQV, BKQV, WO, BO, S1, B1, LINB1, LINW1, S2, B2, LINB2, LINW2 };
+enum F { KKQQVV, WKKWQQWVV, BETA, ALPHA, ATTN_DROP_MASK, ATTN_DROP, GAMMA, ATT, DROP1MASK, SB1,
+         SB1_LINW1, DROP2, LIN1, DROP2_LINW2, LIN2, LN2, LN2STD, LN2DIFF, DROP2MASK, DROP3MASK,
+         LN1, LN1STD, LN1DIFF };
+enum Bw { DLN2, DRESID2, DLIN2, DDROP2, DLIN1, DLIN1_LINW1, DLN1, DRESID1, DATT, DXATT, DGAMMA,
+          DATTN_DROP, DBETA, DKKQQVV };
+
+bool same_dims(const Layout& l, const char* dims) {
+    size_t n = std::strlen(dims);
+    if ((size_t)l.rank != n) return false;
+    for (size_t i = 0; i < n; ++i) if (!l.has[dim_of(dims[i])]) return false;
+    return true;
+}
+
+// ---------------------------------------------------------------------------
+// Views
+// ---------------------------------------------------------------------------
+struct Space {
+    RowSpace rs;
+    int outer[4];   // logical dims of the four outer slots (-1: unused)
+    int rdim;       // logical dim of the row
+};
+
+Space make_space(const Sizes& sz, std::initializer_list<int> outer, int rdim) {
+    Space s;
+    int n[4] = {1, 1, 1, 1};
+    int k = 4 - (int)outer.size();
+    for (int i = 0; i < 4; ++i) s.outer[i] = -1;
+    for (int d : outer) { s.outer[k] = d; n[k] = (int)sz.n[d]; ++k; }
+    s.rdim = rdim;
+    s.rs.n0 = n[0]; s.rs.n1 = n[1]; s.rs.n2 = n[2]; s.rs.n3 = n[3];
+    s.rs.R = (int)sz.n[rdim];
+    return s;
+}
+
+View make_view(const void* p, const Layout& l, const Space& sp) {
+    View v;
+    v.p = (half_t*)p;
+    long so[4];
+    for (int i = 0; i < 4; ++i) so[i] = sp.outer[i] >= 0 && l.has[sp.outer[i]] ? l.stride[sp.outer[i]] : 0;
+    v.s0 = so[0]; v.s1 = so[1]; v.s2 = so[2]; v.s3 = so[3];
+    v.sr = l.has[sp.rdim] ? l.stride[sp.rdim] : 0;
+    bool vec = v.sr == 1 && (sp.rs.R % 8 == 0) && ((reinterpret_cast<uintptr_t>(p) & 15) == 0);
+    for (int i = 0; i < 4; ++i) vec = vec && (so[i] % 8 == 0);
+    v.vec = vec ? 1 : 0;
+    return v;
+}
+
+// A dense vector indexed by the row dim only ([I] or [U] parameters).
+View vector_view(const void* p, int R) {
+    View v;
+    v.p = (half_t*)p;
+    v.s0 = v.s1 = v.s2 = v.s3 = 0;
+    v.sr = 1;
+    v.vec = (R % 8 == 0) && ((reinterpret_cast<uintptr_t>(p) & 15) == 0) ? 1 : 0;
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// Handle
+// ---------------------------------------------------------------------------
+struct GemmPlan {
+    GemmShape shape;
+    float alpha = 1.f;
+};
+
+enum G { G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
+         G_DWOUT, G_DXOUT, G_DX1GAMMA, G_DX2GAMMA, G_DX1QKT, G_DX2QKT, G_DXQKV, G_DWQKV, G_COUNT };
+
+struct ProfEntry { const char* name; hipEvent_t a, b; };
+
+struct Handle {
+    bool configured = false;
+    Sizes sz;
+    int act = ACT_RELU;
+    float p_softmax = 0, p_resid1 = 0, p_act = 0, p_resid2 = 0, eps = 1e-5f;
+    uint64_t seed = 0;
+    uint32_t step = 0;
+    hipStream_t stream = nullptr;
+    Layout lX, lY;
+    Layout lp[SUB_N_PARAMS], lf[SUB_N_FWD], lb[SUB_N_BWD];
+    int pos_p[SUB_N_PARAMS], pos_f[SUB_N_FWD], pos_b[SUB_N_BWD];   // internal id -> caller position
+    Layout lKK, lQQ, lDKK, lDQQ, lWsub, lBsub;
+    GemmPlan gemm[G_COUNT];
+    float* ws = nullptr;
+    size_t ws_floats = 0;
+    bool profiling = false;
+    std::vector<ProfEntry> prof;
+    size_t prof_used = 0;
+
+    ~Handle() {
+        if (ws) (void)hipFree(ws);
+        for (auto& e : prof) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+    }
+};
+
+void hip_check(hipError_t e, const char* what) {
+    if (e != hipSuccess) fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+PhiloxKey make_key(const Handle& h, uint32_t site, float p) {
+    PhiloxKey k;
+    k.k0 = (uint32_t)h.seed; k.k1 = (uint32_t)(h.seed >> 32);
+    k.site = site; k.step = h.step; k.thr = threshold16(p);
+    return k;
+}
+
+struct ProfScope {
+    Handle& h; ProfEntry* e = nullptr;
+    ProfScope(Handle& h_, const char* name) : h(h_) {
+        if (!h.profiling) return;
+        if (h.prof_used == h.prof.size()) {
+            ProfEntry n{name, nullptr, nullptr};
+            hip_check(hipEventCreate(&n.a), "hipEventCreate");
+            hip_check(hipEventCreate(&n.b), "hipEventCreate");
+            h.prof.push_back(n);
+        }
+        e = &h.prof[h.prof_used++];
+        e->name = name;
+        hip_check(hipEventRecord(e->a, h.stream), "hipEventRecord");
+    }
+    ~ProfScope() { if (e) (void)hipEventRecord(e->b, h.stream); }
+};
+
+void ensure_ws(Handle& h, size_t floats) {
+    if (floats <= h.ws_floats) return;
+    if (h.ws) hip_check(hipFree(h.ws), "hipFree");
+    h.ws = nullptr; h.ws_floats = 0;
+    hip_check(hipMalloc((void**)&h.ws, floats * sizeof(float)), "hipMalloc(workspace)");
+    h.ws_floats = floats;
+}
+
+// ---------------------------------------------------------------------------
+// Configuration
+// ---------------------------------------------------------------------------
+template <int N>
+void bind_tensors(const TensorDef (&defs)[N], const char* const* names, const char* const* layouts,
+                  const Sizes& sz, Layout* out, int* pos, const char* what) {
+    bool seen[N] = {false};
+    for (int i = 0; i < N; ++i) {
+        if (!names[i] || !layouts[i]) fail(std::string(what) + ": null name or layout");
+        int id = -1;
+        for (int j = 0; j < N; ++j) if (std::strcmp(names[i], defs[j].name) == 0) id = j;
+        if (id < 0) fail(std::string(what) + ": unknown tensor name " + names[i]);
+        if (seen[id]) fail(std::string(what) + ": tensor listed twice: " + names[i]);
+        seen[id] = true;
+        out[id] = make_layout(layouts[i], sz);
+        if (!same_dims(out[id], defs[id].dims))
+            fail(std::string("layout of ") + names[i] + " must be a permutation of " + defs[id].dims +
+                 ", got " + layouts[i]);
+        pos[id] = i;
+    }
+}
+
+void plan_gemm(Handle& h, int id, const Layout& a, const Layout& b, const Layout& c, float alpha,
+               const char* name) {
+    try {
+        h.gemm[id].shape = classify_einsum(a, b, c);
+    } catch (const Error& e) {
+        fail(std::string(name) + " (" + a.str() + "," + b.str() + "->" + c.str() + "): " + e.what());
+    }
+    h.gemm[id].alpha = alpha;
+}
+
+void configure(Handle& h, const sub_config* c) {
+    if (!c) fail("sub_configure: null config");
+    if (c->abi_version != SUB_ABI_VERSION) fail("sub_configure: ABI version mismatch");
+    if (c->dtype != SUB_DTYPE_F16) fail("sub_configure: only fp16 tensors are supported");
+    if (c->batch <= 0 || c->seq <= 0 || c->heads <= 0 || c->embed <= 0) fail("sub_configure: sizes must be positive");
+    if (c->embed % c->heads != 0) fail("sub_configure: embed must be a multiple of heads");
+    if (c->activation != SUB_ACT_RELU && c->activation != SUB_ACT_GELU) fail("sub_configure: unknown activation");
+    const float ps[4] = {c->p_softmax, c->p_resid1, c->p_act, c->p_resid2};
+    for (float p : ps) if (!(p >= 0.f && p <= 1.f)) fail("sub_configure: dropout probability outside [0,1]");
+    h.configured = false;
+    Sizes sz;
+    sz.n[dB] = c->batch; sz.n[dJ] = c->seq; sz.n[dK] = c->seq; sz.n[dH] = c->heads;
+    sz.n[dP] = c->embed / c->heads; sz.n[dI] = c->embed;
+    sz.n[dU] = c->intermediate > 0 ? c->intermediate : 4 * (int64_t)c->embed; sz.n[dQ] = 3;
+    h.sz = sz;
+    h.act = c->activation;
+    h.p_softmax = c->p_softmax; h.p_resid1 = c->p_resid1; h.p_act = c->p_act; h.p_resid2 = c->p_resid2;
+    h.eps = c->ln_eps > 0.f ? c->ln_eps : 1e-5f;
+    h.seed = c->seed; h.step = 0;
+    h.lX = make_layout(c->input_layout, sz);
+    h.lY = make_layout(c->output_layout, sz);
+    if (!same_dims(h.lX, "BJI") || !same_dims(h.lY, "BJI")) fail("input/output layout must be a permutation of BJI");
+    bind_tensors(kParams, c->param_names, c->param_layouts, sz, h.lp, h.pos_p, "params");
+    bind_tensors(kFwd, c->fwd_names, c->fwd_layouts, sz, h.lf, h.pos_f, "forward_interm");
+    bind_tensors(kBwd, c->bwd_names, c->bwd_layouts, sz, h.lb, h.pos_b, "backward_interm");
+
+    // Sub-tensors of the Q-stacked tensors (pytorch_module/encoder.py:318-362).
+    Layout kq = drop_front(h.lf[KKQQVV], dQ);
+    h.lQQ = kq; h.lKK = rename_dim(kq, dJ, dK);
+    Layout dkq = drop_front(h.lb[DKKQQVV], dQ);
+    h.lDQQ = dkq; h.lDKK = rename_dim(dkq, dJ, dK);
+    (void)drop_front(h.lf[WKKWQQWVV], dQ);
+    (void)drop_front(h.lp[WKQV], dQ);
+    (void)drop_front(h.lp[BKQV], dQ);
+
+    const float a = 1.0f / std::sqrt((float)sz.n[dP]);
+    // forward (pytorch_module/encoder.cu:87-157)
+    plan_gemm(h, G_QKV, h.lX, h.lp[WKQV], h.lf[WKKWQQWVV], 1.f, "QKV-fused");
+    plan_gemm(h, G_QKT, h.lKK, h.lQQ, h.lf[BETA], a, "QKT");
+    plan_gemm(h, G_GAMMA, h.lKK, h.lf[ATTN_DROP], h.lf[GAMMA], 1.f, "gamma");
+    plan_gemm(h, G_OUT, h.lp[WO], h.lf[GAMMA], h.lf[ATT], 1.f, "out");
+    plan_gemm(h, G_LIN1, h.lf[SB1], h.lp[LINW1], h.lf[SB1_LINW1], 1.f, "lin1");
+    plan_gemm(h, G_LIN2, h.lf[DROP2], h.lp[LINW2], h.lf[DROP2_LINW2], 1.f, "lin2");
+    // backward (pytorch_module/encoder.cu:158-299)
+    plan_gemm(h, G_DXLIN2, h.lb[DLIN2], h.lp[LINW2], h.lb[DDROP2], 1.f, "dXlin2");
+    plan_gemm(h, G_DWLIN2, h.lb[DLIN2], h.lf[DROP2], h.lp[LINW2], 1.f, "dWlin2");
+    plan_gemm(h, G_DXLIN1, h.lb[DLIN1], h.lp[LINW1], h.lb[DLIN1_LINW1], 1.f, "dXlin1");
+    plan_gemm(h, G_DWLIN1, h.lb[DLIN1], h.lf[SB1], h.lp[LINW1], 1.f, "dWlin1");
+    plan_gemm(h, G_DWOUT, h.lf[GAMMA], h.lb[DATT], h.lp[WO], 1.f, "dWout");
+    plan_gemm(h, G_DXOUT, h.lp[WO], h.lb[DATT], h.lb[DGAMMA], 1.f, "dXout");
+    plan_gemm(h, G_DX1GAMMA, h.lKK, h.lb[DGAMMA], h.lb[DATTN_DROP], 1.f, "dX1gamma");
+    plan_gemm(h, G_DX2GAMMA, h.lb[DGAMMA], h.lf[ATTN_DROP], h.lDKK, 1.f, "dX2gamma");
+    plan_gemm(h, G_DX1QKT, h.lKK, h.lb[DBETA], h.lDQQ, a, "dX1QKT");
+    plan_gemm(h, G_DX2QKT, h.lQQ, h.lb[DBETA], h.lDKK, a, "dX2QKT");
+    plan_gemm(h, G_DXQKV, h.lp[WKQV], h.lb[DKKQQVV], h.lb[DXATT], 1.f, "dXQKV-fused");
+    plan_gemm(h, G_DWQKV, h.lX, h.lb[DKKQQVV], h.lp[WKQV], 1.f, "dWQKV-fused");
+
+    // The fp32 scratch of the column reductions is allocated by the first
+    // operator that needs it, so that configuring needs no GPU.
+    h.configured = true;
+}
+
+// ---------------------------------------------------------------------------
+// Operators on a handle
+// ---------------------------------------------------------------------------
+void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const char* name) {
+    ProfScope ps(h, name);
+    GemmEpilogue ep;
+    launch_gemm(h.gemm[id].shape, (const half_t*)A, (const half_t*)B, (half_t*)C, h.gemm[id].alpha, ep, h.stream);
+}
+
+void op_softmax(Handle& h, const void* beta, const Layout& lb, void* alpha, const Layout& la,
+                void* mask, const Layout& lm, void* drop, const Layout& ld, float scale, float p,
+                uint32_t site) {
+    Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
+    launch_softmax(sp.rs, make_view(beta, lb, sp), make_view(alpha, la, sp), make_view(mask, lm, sp),
+                   make_view(drop, ld, sp), scale, make_key(h, site, p), h.stream);
+}
+
+void op_bs(Handle& h, const void* alpha, const Layout& la, const void* mask, const Layout& lm,
+           const void* ddrop, const Layout& ld, void* dbeta, const Layout& lo, float scale) {
+    Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
+    launch_bs(sp.rs, make_view(alpha, la, sp), make_view(mask, lm, sp), make_view(ddrop, ld, sp),
+              make_view(dbeta, lo, sp), scale, h.stream);
+}
+
+void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, const Layout& lres,
+              const void* linear_bias, const void* scale, const void* bias, void* lin,
+              const Layout& llin, void* mask, const Layout& lmask, void* diff, const Layout& ldiff,
+              void* normed, const Layout& lnorm, void* out, const Layout& lout, void* istd,
+              const Layout& listd, float p, uint32_t site) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    int R = sp.rs.R;
+    launch_bdrln(sp.rs, make_view(in, lin_, sp), make_view(resid, lres, sp), vector_view(linear_bias, R),
+                 vector_view(scale, R), vector_view(bias, R), make_view(lin, llin, sp),
+                 make_view(mask, lmask, sp), make_view(diff, ldiff, sp), make_view(normed, lnorm, sp),
+                 make_view(out, lout, sp), make_view(istd, listd, sp), make_key(h, site, p), h.eps,
+                 h.stream);
+}
+
+void op_blnrd(Handle& h, const void* dout, const Layout& ldout, const void* istd, const Layout& listd,
+              const void* diff, const Layout& ldiff, const void* mask, const Layout& lmask,
+              void* d_ln_in, const Layout& l1, void* d_drop_in, const Layout& l2) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    launch_blnrd(sp.rs, make_view(dout, ldout, sp), make_view(istd, listd, sp), make_view(diff, ldiff, sp),
+                 make_view(mask, lmask, sp), make_view(d_ln_in, l1, sp), make_view(d_drop_in, l2, sp),
+                 h.stream);
+}
+
+void op_bad(Handle& h, const void* in, const Layout& lin_, const void* bias, void* lin,
+            const Layout& llin, void* mask, const Layout& lmask, void* out, const Layout& lout,
+            float p, uint32_t site) {
+    Space sp = make_space(h.sz, {dB, dJ}, dU);
+    launch_bad(sp.rs, make_view(in, lin_, sp), vector_view(bias, sp.rs.R), make_view(lin, llin, sp),
+               make_view(mask, lmask, sp), make_view(out, lout, sp), h.act, make_key(h, site, p),
+               h.stream);
+}
+
+void op_bsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* dout,
+            const Layout& ldout, void* din, const Layout& ldin, void* dscale, void* dbias) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    ensure_ws(h, colreduce_ws_floats(sp.rs, 2));
+    launch_bsb(sp.rs, make_view(in, lin_, sp), make_view(dout, ldout, sp), vector_view(scale, sp.rs.R),
+               make_view(din, ldin, sp), ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, h.ws, h.stream);
+}
+
+void op_ebsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* d1,
+             const Layout& l1, const void* d2, const Layout& l2, const void* dlinear,
+             const Layout& ldl, void* din, const Layout& ldin, void* dscale, void* dbias,
+             void* dlinear_bias) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    ensure_ws(h, colreduce_ws_floats(sp.rs, 3));
+    launch_ebsb(sp.rs, make_view(in, lin_, sp), make_view(d1, l1, sp), make_view(d2, l2, sp),
+                make_view(dlinear, ldl, sp), vector_view(scale, sp.rs.R), make_view(din, ldin, sp),
+                ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, ColOut{(half_t*)dlinear_bias}, h.ws,
+                h.stream);
+}
+
+void op_bdrlb(Handle& h, const void* ddrop, const Layout& ld, const void* mask, const Layout& lm,
+              const void* lin, const Layout& ll, void* dlinear, const Layout& lo, void* dbias) {
+    Space sp = make_space(h.sz, {dB, dJ}, dU);
+    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
+    launch_bdrlb(sp.rs, make_view(ddrop, ld, sp), make_view(mask, lm, sp), make_view(lin, ll, sp),
+                 make_view(dlinear, lo, sp), ColOut{(half_t*)dbias}, h.act, h.ws, h.stream);
+}
+
+void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
+    launch_baob(sp.rs, make_view(datt, l, sp), ColOut{(half_t*)dbo}, h.ws, h.stream);
+}
+
+// out[q,p,h,b,j] = in[q,p,h,b,j] + bias[q,p,h].  The row dim is the innermost
+// dim of the output when the input is contiguous along it too, else J.
+void op_aib(Handle& h, const void* in, const Layout& lin_, const void* bias, const Layout& lbias,
+            void* out, const Layout& lout) {
+    int r = lout.dims[lout.rank - 1];
+    if (lin_.stride[r] != 1) r = dJ;
+    int outer[4]; int k = 0;
+    const int canon[5] = {dQ, dP, dH, dB, dJ};
+    for (int d : canon) if (d != r) outer[k++] = d;
+    Space sp = make_space(h.sz, {outer[0], outer[1], outer[2], outer[3]}, r);
+    launch_add(sp.rs, make_view(in, lin_, sp), make_view(bias, lbias, sp), make_view(out, lout, sp), h.stream);
+}
+
+// dbias[q,p,h] = sum_{b,j} d[q,p,h,b,j]
+void op_baib(Handle& h, const void* d, const Layout& ld, void* dbias, const Layout& lbias) {
+    Space sp = make_space(h.sz, {dQ, dP, dH, dB}, dJ);
+    launch_baib(sp.rs, make_view(d, ld, sp), make_view(dbias, lbias, sp), h.stream);
+}
+
+void op_bei(Handle& h, const void* a, const Layout& la, const void* b, const Layout& lb_, void* o,
+            const Layout& lo) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    launch_add(sp.rs, make_view(a, la, sp), make_view(b, lb_, sp), make_view(o, lo, sp), h.stream);
+}
+
+// ---------------------------------------------------------------------------
+// The two operator sequences
+// ---------------------------------------------------------------------------
+struct FwdPtrs {
+    void* X; void* W[SUB_N_PARAMS]; void* F[SUB_N_FWD]; void* Y;
+};
+struct BwdPtrs {
+    void* DY; void* DW[SUB_N_PARAMS]; void* Bk[SUB_N_BWD]; void* W[SUB_N_PARAMS]; void* F[SUB_N_FWD];
+    void* X; void* DX;
+};
+
+half_t* sub_q(void* base, const Handle& h, int q) {
+    int64_t n = h.sz.n[dP] * h.sz.n[dH] * h.sz.n[dB] * h.sz.n[dJ];
+    return (half_t*)base + (int64_t)q * n;
+}
+
+void forward(Handle& h, const FwdPtrs& t) {
+    if (!h.configured) fail("encoder_forward: handle is not configured");
+    h.prof_used = 0;
+    void* const* W = t.W; void* const* F = t.F;
+    run_gemm(h, G_QKV, t.X, W[WKQV], F[WKKWQQWVV], "QKV-fused");
+    {
+        ProfScope ps(h, "aib");
+        op_aib(h, F[WKKWQQWVV], h.lf[WKKWQQWVV], W[BKQV], h.lp[BKQV], F[KKQQVV], h.lf[KKQQVV]);
+    }
+    half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
+    run_gemm(h, G_QKT, KK, QQ, F[BETA], "QKT");
+    {
+        ProfScope ps(h, "softmax");
+        op_softmax(h, F[BETA], h.lf[BETA], F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK],
+                   F[ATTN_DROP], h.lf[ATTN_DROP], 1.0f, h.p_softmax, SUB_SITE_SOFTMAX);
+    }
+    run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
+    run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
+    {
+        ProfScope ps(h, "bdrln1");   // adds BO to ATT in place (encoder.cu:134-135)
+        op_bdrln(h, F[ATT], h.lf[ATT], t.X, h.lX, W[BO], W[S1], W[B1], F[ATT], h.lf[ATT],
+                 F[DROP1MASK], h.lf[DROP1MASK], F[LN1DIFF], h.lf[LN1DIFF], F[LN1], h.lf[LN1],
+                 F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1);
+    }
+    run_gemm(h, G_LIN1, F[SB1], W[LINW1], F[SB1_LINW1], "lin1");
+    {
+        ProfScope ps(h, "bad");
+        op_bad(h, F[SB1_LINW1], h.lf[SB1_LINW1], W[LINB1], F[LIN1], h.lf[LIN1], F[DROP2MASK],
+               h.lf[DROP2MASK], F[DROP2], h.lf[DROP2], h.p_act, SUB_SITE_ACT);
+    }
+    run_gemm(h, G_LIN2, F[DROP2], W[LINW2], F[DROP2_LINW2], "lin2");
+    {
+        ProfScope ps(h, "bdrln2");
+        op_bdrln(h, F[DROP2_LINW2], h.lf[DROP2_LINW2], F[SB1], h.lf[SB1], W[LINB2], W[S2], W[B2],
+                 F[LIN2], h.lf[LIN2], F[DROP3MASK], h.lf[DROP3MASK], F[LN2DIFF], h.lf[LN2DIFF],
+                 F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2);
+    }
+    h.step += 1;
+}
+
+void backward(Handle& h, const BwdPtrs& t) {
+    if (!h.configured) fail("encoder_backward: handle is not configured");
+    h.prof_used = 0;
+    void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
+    {
+        ProfScope ps(h, "bsb");
+        op_bsb(h, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, D[DLN2], h.lb[DLN2], DW[S2], DW[B2]);
+    }
+    {
+        ProfScope ps(h, "blnrd1");
+        op_blnrd(h, D[DLN2], h.lb[DLN2], F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF],
+                 F[DROP3MASK], h.lf[DROP3MASK], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2]);
+    }
+    run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
+    run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
+    {
+        ProfScope ps(h, "bdrlb");
+        op_bdrlb(h, D[DDROP2], h.lb[DDROP2], F[DROP2MASK], h.lf[DROP2MASK], F[LIN1], h.lf[LIN1],
+                 D[DLIN1], h.lb[DLIN1], DW[LINB1]);
+    }
+    run_gemm(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1");
+    run_gemm(h, G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1");
+    {
+        ProfScope ps(h, "ebsb");
+        op_ebsb(h, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
+                h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], D[DLN1], h.lb[DLN1], DW[S1], DW[B1], DW[LINB2]);
+    }
+    {
+        ProfScope ps(h, "blnrd2");
+        op_blnrd(h, D[DLN1], h.lb[DLN1], F[LN1STD], h.lf[LN1STD], F[LN1DIFF], h.lf[LN1DIFF],
+                 F[DROP1MASK], h.lf[DROP1MASK], D[DRESID1], h.lb[DRESID1], D[DATT], h.lb[DATT]);
+    }
+    {
+        ProfScope ps(h, "baob");
+        op_baob(h, D[DATT], h.lb[DATT], DW[BO]);
+    }
+    run_gemm(h, G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout");
+    run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
+    half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
+    half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
+    run_gemm(h, G_DX1GAMMA, VV, D[DGAMMA], D[DATTN_DROP], "dX1gamma");
+    run_gemm(h, G_DX2GAMMA, D[DGAMMA], F[ATTN_DROP], DVV, "dX2gamma");
+    {
+        ProfScope ps(h, "bs");
+        op_bs(h, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK], D[DATTN_DROP],
+              h.lb[DATTN_DROP], D[DBETA], h.lb[DBETA], 1.0f);
+    }
+    run_gemm(h, G_DX1QKT, KK, D[DBETA], DQQ, "dX1QKT");
+    run_gemm(h, G_DX2QKT, QQ, D[DBETA], DKK, "dX2QKT");
+    run_gemm(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused");
+    run_gemm(h, G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused");
+    {
+        ProfScope ps(h, "baib");
+        op_baib(h, D[DKKQQVV], h.lb[DKKQQVV], DW[BKQV], h.lp[BKQV]);
+    }
+    {
+        ProfScope ps(h, "bei");
+        op_bei(h, D[DXATT], h.lb[DXATT], D[DRESID1], h.lb[DRESID1], t.DX, h.lX);
+    }
+}
+
+void unpack_forward(const Handle& h, void* const* p, FwdPtrs& t) {
+    t.X = p[0];
+    for (int i = 0; i < SUB_N_PARAMS; ++i) t.W[i] = p[1 + h.pos_p[i]];
+    for (int i = 0; i < SUB_N_FWD; ++i) t.F[i] = p[1 + SUB_N_PARAMS + h.pos_f[i]];
+    t.Y = p[1 + SUB_N_PARAMS + SUB_N_FWD];
+}
+
+void unpack_backward(const Handle& h, void* const* p, BwdPtrs& t) {
+    int o = 0;
+    t.DY = p[o++];
+    for (int i = 0; i < SUB_N_PARAMS; ++i) t.DW[i] = p[o + h.pos_p[i]];
+    o += SUB_N_PARAMS;
+    for (int i = 0; i < SUB_N_BWD; ++i) t.Bk[i] = p[o + h.pos_b[i]];
+    o += SUB_N_BWD;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) t.W[i] = p[o + h.pos_p[i]];
+    o += SUB_N_PARAMS;
+    for (int i = 0; i < SUB_N_FWD; ++i) t.F[i] = p[o + h.pos_f[i]];
+    o += SUB_N_FWD;
+    t.X = p[o++];
+    t.DX = p[o++];
+}
+
+template <class Fn>
+int guarded(Fn&& fn) {
+    try {
+        fn();
+        return 0;
+    } catch (const std::exception& e) {
+        g_last_error = e.what();
+        return -1;
+    } catch (...) {
+        g_last_error = "unknown error";
+        return -1;
+    }
+}
+
+Handle& as_handle(void* h) {
+    if (!h) fail("null handle");
+    return *static_cast<Handle*>(h);
+}
+
+Layout L(Handle& h, const char* s) { return make_layout(s, h.sz); }
+
+void need_cfg(const Handle& h) {
+    if (!h.configured) fail("handle is not configured");
+}
+
+}  // namespace
+}  // namespace sub
+
+using namespace sub;
+
+extern "C" {
+
+const char* sub_last_error(void) { return g_last_error.c_str(); }
+
+void* init(void) {
+    void* r = nullptr;
+    guarded([&] { r = new Handle(); });
+    return r;
+}
+
+void destroy(void* handle) {
+    guarded([&] { delete static_cast<Handle*>(handle); });
+}
+
+int sub_configure(void* handle, const sub_config* cfg) {
+    return guarded([&] { configure(as_handle(handle), cfg); });
+}
+
+void* init_cfg(const sub_config* cfg) {
+    void* h = init();
+    if (!h) return nullptr;
+    if (sub_configure(h, cfg) != 0) {
+        std::string keep = g_last_error;
+        destroy(h);
+        g_last_error = keep;
+        return nullptr;
+    }
+    return h;
+}
+
+int sub_set_stream(void* handle, void* hip_stream) {
+    return guarded([&] { as_handle(handle).stream = (hipStream_t)hip_stream; });
+}
+
+int sub_set_rng(void* handle, uint64_t seed, uint32_t step) {
+    return guarded([&] { Handle& h = as_handle(handle); h.seed = seed; h.step = step; });
+}
+
+int sub_encoder_forward(void* handle, void* const* ptrs, int n) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        if (n != 1 + SUB_N_PARAMS + SUB_N_FWD + 1) fail("sub_encoder_forward: expected 37 pointers");
+        need_cfg(h);
+        for (int i = 0; i < n; ++i) if (!ptrs[i]) fail("sub_encoder_forward: null tensor pointer");
+        FwdPtrs t; unpack_forward(h, ptrs, t);
+        forward(h, t);
+    });
+}
+
+int sub_encoder_backward(void* handle, void* const* ptrs, int n) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        if (n != 2 + 2 * SUB_N_PARAMS + SUB_N_BWD + SUB_N_FWD + 2) fail("sub_encoder_backward: expected 64 pointers");
+        need_cfg(h);
+        for (int i = 0; i < n; ++i) if (!ptrs[i]) fail("sub_encoder_backward: null tensor pointer");
+        BwdPtrs t; unpack_backward(h, ptrs, t);
+        backward(h, t);
+    });
+}
+
+int encoder_forward(void* handle, void* X,
+                    void* w0, void* w1, void* w2, void* w3, void* w4, void* w5,
+                    void* w6, void* w7, void* w8, void* w9, void* w10, void* w11,
+                    void* f0, void* f1, void* f2, void* f3, void* f4, void* f5, void* f6, void* f7,
+                    void* f8, void* f9, void* f10, void* f11, void* f12, void* f13, void* f14,
+                    void* f15, void* f16, void* f17, void* f18, void* f19, void* f20, void* f21,
+                    void* f22, void* Y) {
+    void* p[] = {X, w0, w1, w2, w3, w4, w5, w6, w7, w8, w9, w10, w11,
+                 f0, f1, f2, f3, f4, f5, f6, f7, f8, f9, f10, f11, f12, f13, f14, f15, f16, f17,
+                 f18, f19, f20, f21, f22, Y};
+    return sub_encoder_forward(handle, p, (int)(sizeof(p) / sizeof(p[0])));
+}
+
+int encoder_backward(void* handle, void* DY,
+                     void* dw0, void* dw1, void* dw2, void* dw3, void* dw4, void* dw5,
+                     void* dw6, void* dw7, void* dw8, void* dw9, void* dw10, void* dw11,
+                     void* b0, void* b1, void* b2, void* b3, void* b4, void* b5, void* b6,
+                     void* b7, void* b8, void* b9, void* b10, void* b11, void* b12, void* b13,
+                     void* w0, void* w1, void* w2, void* w3, void* w4, void* w5,
+                     void* w6, void* w7, void* w8, void* w9, void* w10, void* w11,
+                     void* f0, void* f1, void* f2, void* f3, void* f4, void* f5, void* f6, void* f7,
+                     void* f8, void* f9, void* f10, void* f11, void* f12, void* f13, void* f14,
+                     void* f15, void* f16, void* f17, void* f18, void* f19, void* f20, void* f21,
+                     void* f22, void* X, void* DX) {
+    void* p[] = {DY, dw0, dw1, dw2, dw3, dw4, dw5, dw6, dw7, dw8, dw9, dw10, dw11,
+                 b0, b1, b2, b3, b4, b5, b6, b7, b8, b9, b10, b11, b12, b13,
+                 w0, w1, w2, w3, w4, w5, w6, w7, w8, w9, w10, w11,
+                 f0, f1, f2, f3, f4, f5, f6, f7, f8, f9, f10, f11, f12, f13, f14, f15, f16, f17,
+                 f18, f19, f20, f21, f22, X, DX};
+    return sub_encoder_backward(handle, p, (int)(sizeof(p) / sizeof(p[0])));
+}
+
+int sub_profile_enable(void* handle, int on) {
+    return guarded([&] { Handle& h = as_handle(handle); h.profiling = on != 0; h.prof_used = 0; });
+}
+
+int sub_profile_read(void* handle, int cap, const char** names, float* ms) {
+    int count = 0;
+    int rc = guarded([&] {
+        Handle& h = as_handle(handle);
+        hip_check(hipStreamSynchronize(h.stream), "hipStreamSynchronize");
+        count = (int)h.prof_used;
+        for (int i = 0; i < count && i < cap; ++i) {
+            float t = 0.f;
+            hip_check(hipEventElapsedTime(&t, h.prof[i].a, h.prof[i].b), "hipEventElapsedTime");
+            if (names) names[i] = h.prof[i].name;
+            if (ms) ms[i] = t;
+        }
+    });
+    return rc == 0 ? count : rc;
+}
+
+int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alpha,
+                   const char* l_alpha, void* mask, const char* l_mask, void* drop,
+                   const char* l_drop, float scale, float p, uint32_t site) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_softmax(h, beta, L(h, l_beta), alpha, L(h, l_alpha), mask, L(h, l_mask), drop, L(h, l_drop),
+                   scale, p, site);
+    });
+}
+
+int sub_op_bs(void* handle, const void* alpha, const char* l_alpha, const void* mask,
+              const char* l_mask, const void* ddrop, const char* l_ddrop, void* dbeta,
+              const char* l_dbeta, float scale) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bs(h, alpha, L(h, l_alpha), mask, L(h, l_mask), ddrop, L(h, l_ddrop), dbeta, L(h, l_dbeta), scale);
+    });
+}
+
+int sub_op_bdrln(void* handle, const void* in, const char* l_in, const void* resid,
+                 const char* l_resid, const void* linear_bias, const void* scale, const void* bias,
+                 void* lin, const char* l_lin, void* mask, const char* l_mask, void* diff,
+                 const char* l_diff, void* normed, const char* l_normed, void* out,
+                 const char* l_out, void* istd, const char* l_istd, float p, uint32_t site) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bdrln(h, in, L(h, l_in), resid, L(h, l_resid), linear_bias, scale, bias, lin, L(h, l_lin),
+                 mask, L(h, l_mask), diff, L(h, l_diff), normed, L(h, l_normed), out, L(h, l_out),
+                 istd, L(h, l_istd), p, site);
+    });
+}
+
+int sub_op_blnrd(void* handle, const void* dout, const char* l_dout, const void* istd,
+                 const char* l_istd, const void* diff, const char* l_diff, const void* mask,
+                 const char* l_mask, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                 const char* l_d_drop_in) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_blnrd(h, dout, L(h, l_dout), istd, L(h, l_istd), diff, L(h, l_diff), mask, L(h, l_mask),
+                 d_ln_in, L(h, l_d_ln_in), d_drop_in, L(h, l_d_drop_in));
+    });
+}
+
+int sub_op_bad(void* handle, const void* in, const char* l_in, const void* bias, void* lin,
+               const char* l_lin, void* mask, const char* l_mask, void* out, const char* l_out,
+               float p, uint32_t site) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bad(h, in, L(h, l_in), bias, lin, L(h, l_lin), mask, L(h, l_mask), out, L(h, l_out), p, site);
+    });
+}
+
+int sub_op_bsb(void* handle, const void* in, const char* l_in, const void* scale, const void* dout,
+               const char* l_dout, void* din, const char* l_din, void* dscale, void* dbias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bsb(h, in, L(h, l_in), scale, dout, L(h, l_dout), din, L(h, l_din), dscale, dbias);
+    });
+}
+
+int sub_op_ebsb(void* handle, const void* in, const char* l_in, const void* scale,
+                const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                const void* dlinear, const char* l_dlinear, void* din, const char* l_din,
+                void* dscale, void* dbias, void* dlinear_bias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_ebsb(h, in, L(h, l_in), scale, dout1, L(h, l_dout1), dout2, L(h, l_dout2), dlinear,
+                L(h, l_dlinear), din, L(h, l_din), dscale, dbias, dlinear_bias);
+    });
+}
+
+int sub_op_bdrlb(void* handle, const void* ddrop, const char* l_ddrop, const void* mask,
+                 const char* l_mask, const void* lin, const char* l_lin, void* dlinear,
+                 const char* l_dlinear, void* dbias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bdrlb(h, ddrop, L(h, l_ddrop), mask, L(h, l_mask), lin, L(h, l_lin), dlinear, L(h, l_dlinear), dbias);
+    });
+}
+
+int sub_op_baob(void* handle, const void* datt, const char* l_datt, void* dbo) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_baob(h, datt, L(h, l_datt), dbo);
+    });
+}
+
+int sub_op_aib(void* handle, const void* in, const char* l_in, const void* bias, const char* l_bias,
+               void* out, const char* l_out) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_aib(h, in, L(h, l_in), bias, L(h, l_bias), out, L(h, l_out));
+    });
+}
+
+int sub_op_baib(void* handle, const void* d, const char* l_d, void* dbias, const char* l_dbias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_baib(h, d, L(h, l_d), dbias, L(h, l_dbias));
+    });
+}
+
+int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void* dresid1,
+               const char* l_dresid1, void* dx, const char* l_dx) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        op_bei(h, dxatt, L(h, l_dxatt), dresid1, L(h, l_dresid1), dx, L(h, l_dx));
+    });
+}
+
+int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
+                  void* C, const char* l_C, float alpha) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), L(h, l_C));
+        GemmEpilogue ep;
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream);
+    });
+}
+
+int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        Layout l = L(h, layout);
+        for (int d = 0; d < NDIM; ++d) strides[d] = l.has[d] ? l.stride[d] : 0;
+    });
+}
+
+int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const char* l_C,
+                        int64_t out[18]) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), L(h, l_C));
+        out[0] = g.batch(); out[1] = g.M; out[2] = g.N; out[3] = g.K();
+        out[4] = g.sAM; out[5] = g.sAK1; out[6] = g.sAb[0];
+        out[7] = g.sBN; out[8] = g.sBK1; out[9] = g.sBb[0];
+        out[10] = g.sCM; out[11] = g.sCN; out[12] = g.sCb[0];
+        out[13] = g.nbatch; out[14] = g.K0; out[15] = g.sAK0; out[16] = g.sBK0;
+        // alignment of real buffers is unknown here: assume 16-byte aligned bases
+        out[17] = gemm_kernel_kind(g, (const void*)16, (const void*)16, (const void*)16);
+    });
+}
+
+int sub_philox_fields_host(uint64_t seed, uint32_t site, uint32_t step, uint64_t start, uint64_t n,
+                           uint16_t* out) {
+    return guarded([&] {
+        PhiloxKey k; k.k0 = (uint32_t)seed; k.k1 = (uint32_t)(seed >> 32); k.site = site; k.step = step; k.thr = 0;
+        for (uint64_t i = 0; i < n; ++i) {
+            uint64_t e = start + i;
+            U4 r = philox_group(k, e >> 3);
+            out[i] = (uint16_t)field16(r, (int)(e & 7));
+        }
+    });
+}
+
+uint32_t sub_dropout_threshold(float p) { return threshold16(p); }
+
+}  // extern "C"

@@ -1,0 +1,264 @@
+// Column reductions: gradients of per-feature vectors (LayerNorm scale/bias,
+// linear biases) fused with the elementwise work that shares their inputs.
+// Counterparts: pytorch_module/block_bsb_ebsb.cuh:12-420, block_bdrlb.cuh:13-146,
+// block_baob.cuh:10-97, block_baib.cuh:15-211.
+//
+// The reference gives each feature one 32-thread warp that walks every token.
+// Here tokens are split into chunks so that the grid fills 256 CUs: each block
+// reduces its token chunk for a strip of features into fp32 partials
+// (deterministically, no atomics), and a small second kernel adds the partials.
+#include "sub_ops.hpp"
+
+namespace sub {
+
+namespace {
+
+constexpr int BLOCK = 256;
+constexpr int WPB = BLOCK / WAVE;
+
+enum ColKind { COL_BSB, COL_EBSB, COL_BDRLB, COL_BAOB };
+
+struct ColArgs {
+    View v[7];
+    int act;
+};
+
+template <int KIND> struct ColTraits;
+template <> struct ColTraits<COL_BSB> { static constexpr int NS = 2; };
+template <> struct ColTraits<COL_EBSB> { static constexpr int NS = 3; };
+template <> struct ColTraits<COL_BDRLB> { static constexpr int NS = 1; };
+template <> struct ColTraits<COL_BAOB> { static constexpr int NS = 1; };
+
+__device__ __forceinline__ float gelu_grad(float x) {
+    const float c = 0.7978845608028654f;
+    float x3 = x * x * x;
+    float u = c * (x + 0.044715f * x3);
+    float t = 1.0f - 2.0f / (1.0f + __expf(2.0f * u));
+    float sech2 = 1.0f - t * t;
+    return 0.5f * t + (1.5f * 0.044715f * c * x3 + 0.5f * c * x) * sech2 + 0.5f;
+}
+
+template <int KIND>
+__device__ __forceinline__ void col_process(const RowSpace& rs, const ColArgs& a, const RowIdx& ix,
+                                            int e0, int nv, const F8& fscale,
+                                            float (&acc)[ColTraits<KIND>::NS][8]) {
+    if (KIND == COL_BSB) {
+        // v0 IN (normed), v1 DOUT, v3 DIN
+        F8 fi = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
+        F8 fd = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
+        F8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            o.v[i] = fd.v[i] * fscale.v[i];
+            acc[0][i] += fd.v[i] * fi.v[i];
+            acc[1][i] += fd.v[i];
+        }
+        store8(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
+    } else if (KIND == COL_EBSB) {
+        // v0 IN, v1 DOUT1, v2 DOUT2, v4 DLINEAR, v3 DIN
+        F8 fi = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
+        F8 f1 = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
+        F8 f2 = load8(a.v[2], view_offset(a.v[2], ix), e0, nv);
+        F8 fl = load8(a.v[4], view_offset(a.v[4], ix), e0, nv);
+        F8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float d = f1.v[i] + f2.v[i];
+            o.v[i] = d * fscale.v[i];
+            acc[0][i] += d * fi.v[i];
+            acc[1][i] += d;
+            acc[2][i] += fl.v[i];
+        }
+        store8(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
+    } else if (KIND == COL_BDRLB) {
+        // v0 DDROP, v1 MASK, v2 LIN, v3 DLINEAR
+        F8 fd = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
+        F8 fm = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
+        F8 fl = load8(a.v[2], view_offset(a.v[2], ix), e0, nv);
+        h8 oh;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float d = fd.v[i] * fm.v[i];
+            float g = a.act == ACT_GELU ? gelu_grad(fl.v[i]) * d : (fl.v[i] > 0.f ? d : 0.f);
+            oh[i] = (half_t)g;
+            acc[0][i] += i < nv ? (float)oh[i] : 0.f;
+        }
+        store8h(a.v[3], view_offset(a.v[3], ix), e0, nv, oh);
+    } else {
+        F8 fd = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[0][i] += fd.v[i];
+    }
+}
+
+// grid.x = feature strips of lpr*8 features, grid.y = token chunks.
+template <int KIND>
+__global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, float* ws, int lpr_log2,
+                                                     long rows_per_block, long nrows) {
+    constexpr int NS = ColTraits<KIND>::NS;
+    __shared__ float red[BLOCK][9];          // +1 pad: conflict-free column reads
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int lpr = 1 << lpr_log2, rpw = WAVE >> lpr_log2;
+    const int fl = lane & (lpr - 1), sub = lane >> lpr_log2;
+    const int e0 = (blockIdx.x * lpr + fl) * 8;
+    int nv = rs.R - e0; nv = nv < 0 ? 0 : (nv > 8 ? 8 : nv);
+    long row_begin = (long)blockIdx.y * rows_per_block;
+    long row_end = row_begin + rows_per_block; row_end = row_end < nrows ? row_end : nrows;
+    float acc[NS][8];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[s][i] = 0.f;
+    F8 fscale;
+    if (KIND == COL_BSB || KIND == COL_EBSB) fscale = load8(a.v[5], 0, e0, nv);
+    if (nv > 0) {
+        for (long row = row_begin + wave * rpw + sub; row < row_end; row += WPB * rpw) {
+            RowIdx ix = row_index(rs, row);
+            col_process<KIND>(rs, a, ix, e0, nv, fscale, acc);
+        }
+    }
+    const int ntc = gridDim.y;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) red[tid][i] = acc[s][i];
+        __syncthreads();
+        if (tid < lpr && nv > 0) {
+            float tot[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tot[i] = 0.f;
+            for (int t = tid; t < BLOCK; t += lpr)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) tot[i] += red[t][i];
+            float* dst = ws + ((long)s * ntc + blockIdx.y) * rs.R + e0;
+            for (int i = 0; i < nv; ++i) dst[i] = tot[i];
+        }
+    }
+}
+
+struct FinishArgs {
+    half_t* out[3];
+};
+
+__global__ __launch_bounds__(BLOCK) void k_colfinish(const float* ws, FinishArgs o, int ns, int ntc, int R) {
+    long idx = (long)blockIdx.x * BLOCK + threadIdx.x;
+    if (idx >= (long)ns * R) return;
+    int s = (int)(idx / R), f = (int)(idx - (long)s * R);
+    const float* p = ws + (long)s * ntc * R + f;
+    float t = 0.f;
+    for (int c = 0; c < ntc; ++c) t += p[(long)c * R];
+    o.out[s][f] = (half_t)t;
+}
+
+struct ColPlan {
+    int lpr_log2, nstrips, ntc;
+    long rows_per_block;
+};
+
+inline ColPlan col_plan(const RowSpace& rs) {
+    ColPlan p;
+    int chunks = (rs.R + 7) / 8;
+    p.lpr_log2 = 0;
+    while ((1 << p.lpr_log2) < chunks && p.lpr_log2 < 6) ++p.lpr_log2;
+    int lpr = 1 << p.lpr_log2;
+    p.nstrips = (chunks + lpr - 1) / lpr;
+    long nrows = rs.rows();
+    int rows_per_iter = WPB * (WAVE / lpr);
+    // aim for ~2048 blocks in total, at least two row-iterations per block
+    long want_tc = 2048 / p.nstrips; if (want_tc < 1) want_tc = 1;
+    long rpb = (nrows + want_tc - 1) / want_tc;
+    if (rpb < 2L * rows_per_iter) rpb = 2L * rows_per_iter;
+    rpb = (rpb + rows_per_iter - 1) / rows_per_iter * rows_per_iter;
+    p.rows_per_block = rpb;
+    p.ntc = (int)((nrows + rpb - 1) / rpb);
+    if (p.ntc < 1) p.ntc = 1;
+    return p;
+}
+
+template <int KIND>
+void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hipStream_t st,
+             const char* what) {
+    constexpr int NS = ColTraits<KIND>::NS;
+    if (rs.R <= 0) return;
+    if (!ws) fail(std::string(what) + ": no reduction workspace");
+    ColPlan p = col_plan(rs);
+    long nrows = rs.rows();
+    hipLaunchKernelGGL(k_colreduce<KIND>, dim3(p.nstrips, p.ntc), dim3(BLOCK), 0, st, rs, a, ws,
+                       p.lpr_log2, p.rows_per_block, nrows);
+    check_launch(what);
+    long n = (long)NS * rs.R;
+    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((n + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, st,
+                       (const float*)ws, fo, NS, p.ntc, rs.R);
+    check_launch(what);
+}
+
+// One wave per (i0,i1,i2): sum over i3 and the row.
+__global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, View out, long ngroups) {
+    const int lane = threadIdx.x & 63;
+    const long nwaves = (long)gridDim.x * WPB;
+    for (long g = (long)blockIdx.x * WPB + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
+        long i2 = g % rs.n2; long r = g / rs.n2;
+        long i1 = r % rs.n1; long i0 = r / rs.n1;
+        long base = i0 * d.s0 + i1 * d.s1 + i2 * d.s2;
+        float s = 0.f;
+        for (int i3 = 0; i3 < rs.n3; ++i3) {
+            long ob = base + (long)i3 * d.s3;
+            for (int e0 = lane * 8; e0 < rs.R; e0 += WAVE * 8) {
+                int nv = rs.R - e0; nv = nv > 8 ? 8 : nv;
+                F8 f = load8(d, ob, e0, nv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s += f.v[i];
+            }
+        }
+        s = wave_sum(s);
+        if (lane == 0) out.p[i0 * out.s0 + i1 * out.s1 + i2 * out.s2] = (half_t)s;
+    }
+}
+
+}  // namespace
+
+size_t colreduce_ws_floats(const RowSpace& rs, int nsums) {
+    ColPlan p = col_plan(rs);
+    return (size_t)nsums * p.ntc * rs.R;
+}
+
+void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
+                ColOut dbias, float* ws, hipStream_t st) {
+    ColArgs a{}; a.v[0] = in; a.v[1] = dout; a.v[3] = din; a.v[5] = scale; a.act = 0;
+    FinishArgs fo{{dscale.p, dbias.p, nullptr}};
+    run_col<COL_BSB>(rs, a, fo, ws, st, "backward scale-bias");
+}
+
+void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dlinear, View scale,
+                 View din, ColOut dscale, ColOut dbias, ColOut dlinear_bias, float* ws,
+                 hipStream_t st) {
+    ColArgs a{}; a.v[0] = in; a.v[1] = dout1; a.v[2] = dout2; a.v[3] = din; a.v[4] = dlinear;
+    a.v[5] = scale; a.act = 0;
+    FinishArgs fo{{dscale.p, dbias.p, dlinear_bias.p}};
+    run_col<COL_EBSB>(rs, a, fo, ws, st, "extended backward scale-bias");
+}
+
+void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
+                  int act, float* ws, hipStream_t st) {
+    ColArgs a{}; a.v[0] = ddrop; a.v[1] = mask; a.v[2] = lin; a.v[3] = dlinear; a.act = act;
+    FinishArgs fo{{dbias.p, nullptr, nullptr}};
+    run_col<COL_BDRLB>(rs, a, fo, ws, st, "backward dropout-activation-bias");
+}
+
+void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st) {
+    ColArgs a{}; a.v[0] = datt; a.act = 0;
+    FinishArgs fo{{dbo.p, nullptr, nullptr}};
+    run_col<COL_BAOB>(rs, a, fo, ws, st, "backward attention-output bias");
+}
+
+void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st) {
+    long ngroups = (long)rs.n0 * rs.n1 * rs.n2;
+    if (ngroups == 0) return;
+    long blocks = (ngroups + WPB - 1) / WPB;
+    if (blocks > 256L * 64) blocks = 256L * 64;
+    hipLaunchKernelGGL(k_rowgroup_sum, dim3((unsigned)blocks), dim3(BLOCK), 0, st, rs, d, out, ngroups);
+    check_launch("backward attention-input biases");
+}
+
+}  // namespace sub

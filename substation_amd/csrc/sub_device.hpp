@@ -1,0 +1,148 @@
+// Device-side building blocks for the fused (memory-bound) operators:
+// 128-bit fp16 packs with fp32 math, wave64 reductions on DPP, strided views.
+// Takes the place of pytorch_module/{half8,vector_types,warpreduce}.cuh.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+#include "sub_philox.hpp"
+
+namespace sub {
+
+typedef _Float16 half_t;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+
+constexpr int WAVE = 64;
+
+// Row space: up to four outer dimensions (canonical order) times a row of R
+// elements.  The canonical element index of (row r, column e) is r*R + e.
+struct RowSpace {
+    int n0, n1, n2, n3;
+    int R;
+    long rows() const { return (long)n0 * n1 * n2 * n3; }
+};
+
+// A tensor seen through the row space: strides of the four outer dims and of
+// the row dim, in elements.  vec != 0 promises that 8 consecutive row elements
+// starting at a multiple of 8 are one aligned 16-byte word.
+struct View {
+    half_t* p;
+    long s0, s1, s2, s3;
+    long sr;
+    int vec;
+};
+
+struct F8 {
+    float v[8];
+};
+
+__device__ __forceinline__ long row_offset(const RowSpace& rs, const View& t, long row) {
+    long i3 = row % rs.n3; long r = row / rs.n3;
+    long i2 = r % rs.n2; r /= rs.n2;
+    long i1 = r % rs.n1; long i0 = r / rs.n1;
+    return i0 * t.s0 + i1 * t.s1 + i2 * t.s2 + i3 * t.s3;
+}
+
+// Outer indices of a row, computed once and reused for every view.
+struct RowIdx {
+    long i0, i1, i2, i3;
+};
+__device__ __forceinline__ RowIdx row_index(const RowSpace& rs, long row) {
+    RowIdx x;
+    x.i3 = row % rs.n3; long r = row / rs.n3;
+    x.i2 = r % rs.n2; r /= rs.n2;
+    x.i1 = r % rs.n1; x.i0 = r / rs.n1;
+    return x;
+}
+__device__ __forceinline__ long view_offset(const View& t, const RowIdx& x) {
+    return x.i0 * t.s0 + x.i1 * t.s1 + x.i2 * t.s2 + x.i3 * t.s3;
+}
+
+// Load 8 row elements e0 .. e0+7 (nvalid of them inside the row) as fp32.
+__device__ __forceinline__ F8 load8(const View& t, long base, int e0, int nvalid, float fill = 0.f) {
+    F8 r;
+    const half_t* p = t.p + base;
+    if (t.vec && nvalid == 8) {
+        h8 v = *reinterpret_cast<const h8*>(p + e0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.v[i] = (float)v[i];
+    } else if (t.sr == 0) {
+        float x = nvalid > 0 ? (float)p[0] : fill;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.v[i] = i < nvalid ? x : fill;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r.v[i] = i < nvalid ? (float)p[(long)(e0 + i) * t.sr] : fill;
+    }
+    return r;
+}
+
+__device__ __forceinline__ h8 to_h8(const F8& x) {
+    h8 v;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (half_t)x.v[i];
+    return v;
+}
+
+__device__ __forceinline__ void store8h(const View& t, long base, int e0, int nvalid, h8 v) {
+    half_t* p = t.p + base;
+    if (t.vec && nvalid == 8) {
+        *reinterpret_cast<h8*>(p + e0) = v;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (i < nvalid) p[(long)(e0 + i) * t.sr] = v[i];
+    }
+}
+
+__device__ __forceinline__ void store8(const View& t, long base, int e0, int nvalid, const F8& x) {
+    store8h(t, base, e0, nvalid, to_h8(x));
+}
+
+// ---- wave64 reductions ------------------------------------------------------
+// Two quad permutes, two row mirrors (DPP), then the four row totals are read
+// with v_readlane and combined; the result is uniform across the wave.
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    int i = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true);
+    return __int_as_float(i);
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+    x += dpp<0xB1>(x);    // quad_perm [1,0,3,2]
+    x += dpp<0x4E>(x);    // quad_perm [2,3,0,1]
+    x += dpp<0x141>(x);   // row_half_mirror
+    x += dpp<0x140>(x);   // row_mirror
+    int xi = __float_as_int(x);
+    float a = __int_as_float(__builtin_amdgcn_readlane(xi, 0));
+    float b = __int_as_float(__builtin_amdgcn_readlane(xi, 16));
+    float c = __int_as_float(__builtin_amdgcn_readlane(xi, 32));
+    float d = __int_as_float(__builtin_amdgcn_readlane(xi, 48));
+    return (a + b) + (c + d);
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+    x = fmaxf(x, dpp<0xB1>(x));
+    x = fmaxf(x, dpp<0x4E>(x));
+    x = fmaxf(x, dpp<0x141>(x));
+    x = fmaxf(x, dpp<0x140>(x));
+    int xi = __float_as_int(x);
+    float a = __int_as_float(__builtin_amdgcn_readlane(xi, 0));
+    float b = __int_as_float(__builtin_amdgcn_readlane(xi, 16));
+    float c = __int_as_float(__builtin_amdgcn_readlane(xi, 32));
+    float d = __int_as_float(__builtin_amdgcn_readlane(xi, 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// {0,1} mask pack from keep bits
+__device__ __forceinline__ h8 mask_h8(uint32_t bits) {
+    h8 m;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) m[i] = ((bits >> i) & 1u) ? (half_t)1.0f : (half_t)0.0f;
+    return m;
+}
+
+}  // namespace sub

@@ -1,0 +1,64 @@
+// Launchers of the device kernels (one per fused operator + the GEMM).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "sub_common.hpp"
+#include "sub_device.hpp"
+
+namespace sub {
+
+enum Activation { ACT_RELU = 0, ACT_GELU = 1 };
+
+inline void check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// --- row operators (one wave per row, row held in registers) -----------------
+void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, float scale,
+                    PhiloxKey key, hipStream_t st);
+void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
+               hipStream_t st);
+void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
+                  View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
+                  float eps, hipStream_t st);
+void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
+                  View d_drop_in, hipStream_t st);
+
+// --- elementwise operators ---------------------------------------------------
+void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, View out, int act,
+                PhiloxKey key, hipStream_t st);
+// out = a + b (b may be a broadcast view): bei, aib
+void launch_add(const RowSpace& rs, View a, View b, View out, hipStream_t st);
+
+// --- column reductions -------------------------------------------------------
+// Sums over all rows of the row space, one result per row element.  `ws` is
+// fp32 scratch of at least colreduce_ws_floats() elements.
+struct ColOut {
+    half_t* p;   // dense [R]
+};
+size_t colreduce_ws_floats(const RowSpace& rs, int nsums);
+void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
+                ColOut dbias, float* ws, hipStream_t st);
+void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dlinear, View scale,
+                 View din, ColOut dscale, ColOut dbias, ColOut dlinear_bias, float* ws,
+                 hipStream_t st);
+void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
+                  int act, float* ws, hipStream_t st);
+void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st);
+// Row sums: out[row-group] = sum over (n3, R) for each (n0,n1,n2): baib.
+void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
+
+// --- tensor contraction ------------------------------------------------------
+struct GemmEpilogue {
+    const half_t* bias = nullptr;   // optional bias added after alpha scaling
+    int64_t sbM = 0, sbN = 0;       // bias strides along M and N
+    int64_t sbb[3] = {0, 0, 0};     // and along the batch dims
+};
+void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C, float alpha,
+                 const GemmEpilogue& ep, hipStream_t st);
+// Which kernel launch_gemm would pick: 0 = scalar fallback, 1 = MFMA.
+int gemm_kernel_kind(const GemmShape& g, const void* A, const void* B, const void* C);
+
+}  // namespace sub

@@ -1,0 +1,158 @@
+"""PyTorch interface to the MI355X encoder layer.
+
+Mirror of pytorch_module/encoder.py: same constructor, attributes, parameter
+naming/shapes (one ``nn.Parameter`` per ``layouts['params']`` entry, shaped in
+layout order), ``forward(X)`` and autograd backward returning ``(DX, *grads)``,
+``debug`` capture.  Differences: nothing is compiled at construction (the
+library is prebuilt, ``compilation_dir`` is accepted and unused), kernels run on
+the caller's current stream, and three keyword-only extras exist: ``activation``
+('relu' as in the CUDA module, or 'gelu'), ``seed`` for the dropout masks and
+``intermediate_size`` (default ``4 * embedding_size``, encoder.py:33).
+"""
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+from . import layouts as _lay
+
+_SUPPORTED_DTYPES = (torch.float16,)
+
+
+class Encoder(torch.nn.Module):
+    """Optimized BERT encoder layer (pytorch_module/encoder.py:19-162)."""
+
+    def __init__(self, compilation_dir, batch_size, max_seq_len, num_heads, embedding_size,
+                 layouts, torch_dtype,
+                 softmax_dropout_probability, residual1_dropout_probability,
+                 activation_dropout_probability, residual2_dropout_probability,
+                 enable_debug=False, profiling=False, *, activation='relu', seed=0,
+                 intermediate_size=None):
+        super().__init__()
+        if torch_dtype not in _SUPPORTED_DTYPES:
+            raise NotImplementedError(
+                f'{torch_dtype}: the MI355X kernels are fp16 storage / fp32 accumulate only')
+        self.batch_size = batch_size
+        self.max_seq_len = max_seq_len
+        self.num_heads = num_heads
+        self.embedding_size = embedding_size
+        self.proj_size = self.embedding_size // self.num_heads
+        self.intermediate_size = intermediate_size or self.embedding_size * 4
+        self.softmax_dropout_probability = softmax_dropout_probability
+        self.residual1_dropout_probability = residual1_dropout_probability
+        self.activation_dropout_probability = activation_dropout_probability
+        self.residual2_dropout_probability = residual2_dropout_probability
+        self.torch_dtype = torch_dtype
+        self.activation = activation
+        self.seed = seed
+        self.debug = {}  # captures intermediate tensors when enable_debug is set
+        self.layouts = _lay.validate(layouts)
+        self.enable_debug = enable_debug
+        self.profiling = profiling
+        self.compilation_dir = compilation_dir
+
+        sizes = _lay.sizes_map(batch_size, max_seq_len, num_heads, embedding_size,
+                               self.intermediate_size)
+        self.sizes = sizes
+
+        for param, layout in layouts['params']:
+            sz = tuple(sizes[s] for s in layout)
+            setattr(self, param, torch.nn.Parameter(torch.empty(*sz, dtype=self.torch_dtype)))
+        self.params = tuple(getattr(self, k) for k, _ in layouts['params'])
+        self.reset_parameters()
+
+        config = _lib.make_config(
+            batch_size, max_seq_len, num_heads, embedding_size, layouts,
+            softmax_dropout_probability, residual1_dropout_probability,
+            activation_dropout_probability, residual2_dropout_probability,
+            activation=activation, seed=seed, intermediate_size=self.intermediate_size)
+        self._handle = _lib.Handle(config)
+        if profiling:
+            self._handle.profile_enable(True)
+        handle = self._handle
+        lib = handle.lib
+        module = self
+        n_fwd = 1 + len(layouts['params']) + len(layouts['forward_interm']) + 1
+        n_bwd = 1 + len(layouts['params']) + len(layouts['backward_interm']) + (
+            len(layouts['params']) + len(layouts['forward_interm']) + 1) + 1
+        fwd_array = ctypes.c_void_p * n_fwd
+        bwd_array = ctypes.c_void_p * n_bwd
+
+        def _alloc(key, device):
+            return [torch.empty(*tuple(sizes[s] for s in layout), device=device,
+                                dtype=module.torch_dtype, requires_grad=False)
+                    for _, layout in layouts[key]]
+
+        class EncoderFunction(torch.autograd.Function):
+            @staticmethod
+            def forward(ctx, X, *weights):
+                if not X.is_cuda:
+                    raise RuntimeError('Encoder.forward needs a tensor on the GPU')
+                dev = X.device
+                X = X.contiguous()
+                Y = torch.empty_like(X)
+                forward_intermediate = _alloc('forward_interm', dev)
+                weights_c = [t.contiguous() for t in weights]
+                handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)
+                ptrs = fwd_array(X.data_ptr(), *(t.data_ptr() for t in weights_c),
+                                 *(t.data_ptr() for t in forward_intermediate), Y.data_ptr())
+                _lib.check(lib.sub_encoder_forward(handle.ptr, ptrs, n_fwd), 'encoder_forward')
+                ctx.save_for_backward(*weights_c, *forward_intermediate, X)
+
+                if module.enable_debug:
+                    torch.cuda.synchronize()
+                    for idx, (name, _) in enumerate(layouts['forward_interm']):
+                        module.debug[name] = forward_intermediate[idx].detach().cpu().numpy()
+                    for idx, (name, _) in enumerate(layouts['params']):
+                        module.debug[name] = weights[idx].detach().cpu().numpy()
+                return Y
+
+            @staticmethod
+            def backward(ctx, DY):
+                dev = DY.device
+                DY = DY.contiguous()
+                DX = torch.empty_like(DY)
+                backward_intermediate = _alloc('backward_interm', dev)
+                param_gradients = _alloc('params', dev)
+                handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)
+                ptrs = bwd_array(DY.data_ptr(), *(t.data_ptr() for t in param_gradients),
+                                 *(t.data_ptr() for t in backward_intermediate),
+                                 *(t.data_ptr() for t in ctx.saved_tensors), DX.data_ptr())
+                _lib.check(lib.sub_encoder_backward(handle.ptr, ptrs, n_bwd), 'encoder_backward')
+
+                if module.enable_debug:
+                    torch.cuda.synchronize()
+                    for idx, (name, _) in enumerate(layouts['backward_interm']):
+                        module.debug[name] = backward_intermediate[idx].detach().cpu().numpy()
+                    for idx, (name, _) in enumerate(layouts['params']):
+                        module.debug['D' + name] = param_gradients[idx].detach().cpu().numpy()
+                return (DX, *param_gradients)
+
+        self.encoder_func = EncoderFunction
+
+    def reset_parameters(self):
+        """U(-1/sqrt(2), 1/sqrt(2)) for every parameter, pytorch_module/encoder.py:144-158."""
+        stdev = 1.0 / math.sqrt(2)
+        for weight in self.parameters():
+            t = torch.empty_like(weight, dtype=torch.float32)
+            torch.nn.init.uniform_(t, -stdev, stdev)
+            with torch.no_grad():
+                weight[:] = t
+
+    def set_rng(self, seed, step=0):
+        """Dropout masks are a pure function of (seed, site, step, element index);
+        every forward call advances ``step`` by one."""
+        self.seed = seed
+        self._handle.set_rng(seed, step)
+
+    def profile(self):
+        """Per-operator times in ms of the last forward or backward call
+        (``profiling=True`` only); the counterpart of the NVTX ranges of
+        pytorch_module/encoder.cu:32-53."""
+        return self._handle.profile_read()
+
+    def forward(self, X):
+        """Run the encoder.  X is in ``layouts['input'][1]`` order; the result is
+        in ``layouts['output'][1]`` order."""
+        return self.encoder_func.apply(X, *self.params)

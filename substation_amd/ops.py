@@ -1,0 +1,110 @@
+"""Single fused operators and the einsum contraction on torch tensors.
+
+The units pytorch_module/benchmark.py generates, compiles and times one by one
+(`Kernel` subclasses at benchmark.py:318-1325); here they are entry points of the
+prebuilt library.  Every tensor argument is a contiguous fp16 CUDA tensor whose
+dimension order is given by the layout string that follows it.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from . import layouts as _lay
+
+
+def _p(t):
+    if t is None:
+        return None
+    if not (t.is_cuda and t.is_contiguous() and t.dtype == torch.float16):
+        raise ValueError('operators take contiguous fp16 CUDA tensors')
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _s(layout):
+    return layout.encode()
+
+
+class Ops:
+    """Operators bound to one problem size (B, L, H, E[, U])."""
+
+    def __init__(self, batch_size, max_seq_len, num_heads, embedding_size, activation='relu',
+                 seed=0, intermediate_size=None):
+        cfg = _lib.make_config(batch_size, max_seq_len, num_heads, embedding_size,
+                               _lay.mi355x_layouts(), activation=activation, seed=seed,
+                               intermediate_size=intermediate_size or 0)
+        self.handle = _lib.Handle(cfg)
+        self.lib = self.handle.lib
+        self.sizes = _lay.sizes_map(batch_size, max_seq_len, num_heads, embedding_size,
+                                    intermediate_size)
+
+    def _pre(self):
+        self.handle.set_stream(torch.cuda.current_stream().cuda_stream)
+        return self.handle.ptr
+
+    def empty(self, layout, device='cuda'):
+        return torch.empty(_lay.shape_of(layout, self.sizes), dtype=torch.float16, device=device)
+
+    def set_rng(self, seed, step=0):
+        self.handle.set_rng(seed, step)
+
+    def softmax(self, beta, l_beta, alpha, l_alpha, mask, l_mask, drop, l_drop, scale=1.0, p=0.0,
+                site=0):
+        _lib.check(self.lib.sub_op_softmax(self._pre(), _p(beta), _s(l_beta), _p(alpha), _s(l_alpha),
+                                           _p(mask), _s(l_mask), _p(drop), _s(l_drop), scale, p, site),
+                   'softmax')
+
+    def bs(self, alpha, l_alpha, mask, l_mask, ddrop, l_ddrop, dbeta, l_dbeta, scale=1.0):
+        _lib.check(self.lib.sub_op_bs(self._pre(), _p(alpha), _s(l_alpha), _p(mask), _s(l_mask),
+                                      _p(ddrop), _s(l_ddrop), _p(dbeta), _s(l_dbeta), scale), 'bs')
+
+    def bdrln(self, inp, l_in, resid, l_resid, linear_bias, scale, bias, lin, l_lin, mask, l_mask,
+              diff, l_diff, normed, l_normed, out, l_out, istd, l_istd, p=0.0, site=1):
+        _lib.check(self.lib.sub_op_bdrln(
+            self._pre(), _p(inp), _s(l_in), _p(resid), _s(l_resid), _p(linear_bias), _p(scale),
+            _p(bias), _p(lin), _s(l_lin), _p(mask), _s(l_mask), _p(diff), _s(l_diff), _p(normed),
+            _s(l_normed), _p(out), _s(l_out), _p(istd), _s(l_istd), p, site), 'bdrln')
+
+    def blnrd(self, dout, l_dout, istd, l_istd, diff, l_diff, mask, l_mask, d_ln_in, l_d_ln_in,
+              d_drop_in, l_d_drop_in):
+        _lib.check(self.lib.sub_op_blnrd(
+            self._pre(), _p(dout), _s(l_dout), _p(istd), _s(l_istd), _p(diff), _s(l_diff), _p(mask),
+            _s(l_mask), _p(d_ln_in), _s(l_d_ln_in), _p(d_drop_in), _s(l_d_drop_in)), 'blnrd')
+
+    def bad(self, inp, l_in, bias, lin, l_lin, mask, l_mask, out, l_out, p=0.0, site=2):
+        _lib.check(self.lib.sub_op_bad(self._pre(), _p(inp), _s(l_in), _p(bias), _p(lin), _s(l_lin),
+                                       _p(mask), _s(l_mask), _p(out), _s(l_out), p, site), 'bad')
+
+    def bsb(self, inp, l_in, scale, dout, l_dout, din, l_din, dscale, dbias):
+        _lib.check(self.lib.sub_op_bsb(self._pre(), _p(inp), _s(l_in), _p(scale), _p(dout), _s(l_dout),
+                                       _p(din), _s(l_din), _p(dscale), _p(dbias)), 'bsb')
+
+    def ebsb(self, inp, l_in, scale, dout1, l_dout1, dout2, l_dout2, dlinear, l_dlinear, din, l_din,
+             dscale, dbias, dlinear_bias):
+        _lib.check(self.lib.sub_op_ebsb(
+            self._pre(), _p(inp), _s(l_in), _p(scale), _p(dout1), _s(l_dout1), _p(dout2), _s(l_dout2),
+            _p(dlinear), _s(l_dlinear), _p(din), _s(l_din), _p(dscale), _p(dbias), _p(dlinear_bias)),
+            'ebsb')
+
+    def bdrlb(self, ddrop, l_ddrop, mask, l_mask, lin, l_lin, dlinear, l_dlinear, dbias):
+        _lib.check(self.lib.sub_op_bdrlb(self._pre(), _p(ddrop), _s(l_ddrop), _p(mask), _s(l_mask),
+                                         _p(lin), _s(l_lin), _p(dlinear), _s(l_dlinear), _p(dbias)),
+                   'bdrlb')
+
+    def baob(self, datt, l_datt, dbo):
+        _lib.check(self.lib.sub_op_baob(self._pre(), _p(datt), _s(l_datt), _p(dbo)), 'baob')
+
+    def aib(self, inp, l_in, bias, l_bias, out, l_out):
+        _lib.check(self.lib.sub_op_aib(self._pre(), _p(inp), _s(l_in), _p(bias), _s(l_bias), _p(out),
+                                       _s(l_out)), 'aib')
+
+    def baib(self, d, l_d, dbias, l_dbias):
+        _lib.check(self.lib.sub_op_baib(self._pre(), _p(d), _s(l_d), _p(dbias), _s(l_dbias)), 'baib')
+
+    def bei(self, dxatt, l_dxatt, dresid1, l_dresid1, dx, l_dx):
+        _lib.check(self.lib.sub_op_bei(self._pre(), _p(dxatt), _s(l_dxatt), _p(dresid1),
+                                       _s(l_dresid1), _p(dx), _s(l_dx)), 'bei')
+
+    def einsum(self, a, l_a, b, l_b, c, l_c, alpha=1.0):
+        _lib.check(self.lib.sub_op_einsum(self._pre(), _p(a), _s(l_a), _p(b), _s(l_b), _p(c), _s(l_c),
+                                          alpha), 'einsum')

@@ -1,0 +1,185 @@
+"""GPU parity of every fused operator against the oracle's closed forms
+(oracle/encoder_ref.py op_*, restating pytorch_module/benchmark.py), through the
+C ABI.  Inputs are rounded to fp16 first, so the only difference left is the
+device's fp32-internal arithmetic and one fp16 rounding per output: tolerance
+1e-2 relative (pytorch_module/benchmark.py:294-302 uses atol=rtol=1e-2).
+Dropout masks are compared bit-exactly with oracle/philox_ref.py."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import encoder_ref as ref
+from oracle import philox_ref as ph
+from tests.helpers import assert_close, from_layout, h16, to_layout
+
+pytestmark = pytest.mark.gpu
+
+SEED = 0x5EED
+
+
+def _ops(B, L, H, E, act='relu', U=None):
+    from substation_amd.ops import Ops
+    o = Ops(B, L, H, E, activation=act, seed=SEED, intermediate_size=U)
+    return o
+
+
+def _perms(canon, keep=None, limit=4):
+    """A few layouts of `canon`: the canonical one plus others (deterministic)."""
+    allp = [''.join(p) for p in itertools.permutations(canon)]
+    picks = [canon, allp[-1]] + allp[1:len(allp) - 1:max(1, len(allp) // limit)]
+    out = []
+    for p in picks:
+        if p not in out:
+            out.append(p)
+    return out[:limit + 1]
+
+
+SIZES = [(2, 16, 2, 32), (3, 24, 2, 48), (2, 128, 4, 512)]
+
+
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(1, 520, 1, 8)])
+@pytest.mark.parametrize('p', [0.0, 0.5])
+def test_softmax_and_backward(B, L, H, E, p):
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(1)
+    beta = h16(rng.normal(size=(H, B, L, L)) * 2)
+    ddrop = h16(rng.normal(size=(H, B, L, L)))
+    scale = 0.125
+    want_mask = ph.dropout_mask((H, B, L, L), p, SEED, ph.SITE_SOFTMAX, step=3)
+    alpha_w, drop_w = ref.op_softmax(beta, want_mask, scale)
+    for lin, lout in (('HBJK', 'HBJK'), ('BHJK', 'BHJK'), ('HBJK', 'JBHK'), ('KJBH', 'HBKJ')):
+        o.set_rng(SEED, 3)
+        t_beta = to_layout(beta, 'HBJK', lin)
+        a, m, d = o.empty(lout), o.empty(lout), o.empty(lin)
+        o.softmax(t_beta, lin, a, lout, m, lout, d, lin, scale=scale, p=p, site=0)
+        torch.cuda.synchronize()
+        got_mask = from_layout(m, 'HBJK', lout)
+        assert (got_mask == want_mask).all(), 'mask differs from the oracle'
+        assert_close(from_layout(a, 'HBJK', lout), alpha_w, name='ALPHA ' + lin)
+        assert_close(from_layout(d, 'HBJK', lin), drop_w, name='ATTN_DROP ' + lin)
+        # ATTN_DROP is exactly ALPHA * MASK in fp16
+        assert (from_layout(d, 'HBJK', lin) == from_layout(a, 'HBJK', lout) * got_mask).all()
+        # backward on the device's own fp16 alpha
+        alpha16 = from_layout(a, 'HBJK', lout)
+        dbeta = o.empty(lout)
+        o.bs(a, lout, m, lout, to_layout(ddrop, 'HBJK', lin), lin, dbeta, lout, scale=scale)
+        torch.cuda.synchronize()
+        assert_close(from_layout(dbeta, 'HBJK', lout), ref.op_bs(alpha16, want_mask, ddrop, scale),
+                     name='DBETA ' + lin)
+
+
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 8, 1, 1024), (1, 4, 1, 4096), (2, 3, 1, 20)])
+@pytest.mark.parametrize('p', [0.0, 0.3])
+def test_bdrln_and_blnrd(B, L, H, E, p):
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(2)
+    inp = h16(rng.normal(size=(B, L, E))); resid = h16(rng.normal(size=(B, L, E)))
+    lb = h16(rng.normal(size=E) * 0.1); s = h16(1 + 0.1 * rng.normal(size=E)); b = h16(0.1 * rng.normal(size=E))
+    dout = h16(rng.normal(size=(B, L, E)))
+    want_mask = ph.dropout_mask((B, L, E), p, SEED, ph.SITE_RESID1, step=0)
+    for lay, lay2, lstd in (('BJI', 'BJI', 'BJ'), ('JBI', 'BJI', 'JB'), ('IBJ', 'JBI', 'BJ')):
+        o.set_rng(SEED, 0)
+        t_in = to_layout(inp, 'BJI', lay)
+        lin = t_in if lay == 'BJI' else o.empty(lay)          # in-place bias add as in the layer
+        mask, diff, normed, out, istd = o.empty(lay2), o.empty(lay2), o.empty(lay), o.empty(lay), o.empty(lstd)
+        dev = lambda v: torch.from_numpy(v).to(torch.float16).cuda()
+        o.bdrln(t_in, lay, to_layout(resid, 'BJI', lay2), lay2, dev(lb), dev(s), dev(b), lin, lay,
+                mask, lay2, diff, lay2, normed, lay, out, lay, istd, lstd, p=p, site=1)
+        torch.cuda.synchronize()
+        assert (from_layout(mask, 'BJI', lay2) == want_mask).all()
+        lin_w = h16(inp + lb)               # the device rounds LIN before using it
+        _, istd_w, diff_w, normed_w, out_w = ref.op_bdrln(lin_w, resid, 0.0, s, b, want_mask)
+        assert (from_layout(lin, 'BJI', lay) == lin_w).all()
+        assert_close(from_layout(istd, 'BJ', lstd), istd_w, name='ISTD')
+        assert_close(from_layout(diff, 'BJI', lay2), diff_w, name='DIFF')
+        assert_close(from_layout(normed, 'BJI', lay), normed_w, name='NORMED')
+        assert_close(from_layout(out, 'BJI', lay), out_w, name='OUT')
+        # backward from the device's own fp16 DIFF / ISTD
+        d1, d2 = o.empty(lay), o.empty(lay2)
+        o.blnrd(to_layout(dout, 'BJI', lay2), lay2, istd, lstd, diff, lay2, mask, lay2, d1, lay, d2, lay2)
+        torch.cuda.synchronize()
+        w1, w2 = ref.op_blnrd(dout, from_layout(istd, 'BJ', lstd), from_layout(diff, 'BJI', lay2), want_mask)
+        assert_close(from_layout(d1, 'BJI', lay), w1, name='D_LN_IN')
+        assert_close(from_layout(d2, 'BJI', lay2), w2, name='D_DROP_IN')
+
+
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 5, 1, 8)])
+@pytest.mark.parametrize('act', ['relu', 'gelu'])
+def test_bad_and_bdrlb(B, L, H, E, act):
+    U = 4 * E if E != 8 else 20
+    o = _ops(B, L, H, E, act, U=U)
+    rng = np.random.default_rng(3)
+    inp = h16(rng.normal(size=(B, L, U))); bias = h16(rng.normal(size=U) * 0.5)
+    ddrop = h16(rng.normal(size=(B, L, U)))
+    p = 0.25
+    want_mask = ph.dropout_mask((B, L, U), p, SEED, ph.SITE_ACT, step=1)
+    dev = lambda v: torch.from_numpy(v).to(torch.float16).cuda()
+    for lay, lay2 in (('BJU', 'BJU'), ('UBJ', 'BJU'), ('JBU', 'JUB')):
+        o.set_rng(SEED, 1)
+        lin, mask, out = o.empty(lay2), o.empty(lay), o.empty(lay2)
+        o.bad(to_layout(inp, 'BJU', lay), lay, dev(bias), lin, lay2, mask, lay, out, lay2, p=p, site=2)
+        torch.cuda.synchronize()
+        assert (from_layout(mask, 'BJU', lay) == want_mask).all()
+        lin_w = h16(inp + bias)
+        assert (from_layout(lin, 'BJU', lay2) == lin_w).all()
+        assert_close(from_layout(out, 'BJU', lay2), ref.op_bad(lin_w, 0.0, want_mask, act)[1], name='DROP2')
+        dlin, dbias = o.empty(lay), torch.empty(U, dtype=torch.float16, device='cuda')
+        o.bdrlb(to_layout(ddrop, 'BJU', lay2), lay2, mask, lay, lin, lay2, dlin, lay, dbias)
+        torch.cuda.synchronize()
+        w_dlin, w_dbias = ref.op_bdrlb(ddrop, want_mask, lin_w, act)
+        assert_close(from_layout(dlin, 'BJU', lay), w_dlin, name='DLIN1')
+        assert_close(dbias.float().cpu().numpy(), w_dbias, name='DLINB1', tol=2e-2)
+
+
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 3, 1, 20), (4, 64, 1, 1024)])
+def test_bsb_ebsb_baob_bei(B, L, H, E):
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(4)
+    g = lambda: h16(rng.normal(size=(B, L, E)))
+    inp, dout, d2, dl = g(), g(), g(), g()
+    s = h16(1 + 0.1 * rng.normal(size=E))
+    dev = lambda v: torch.from_numpy(v).to(torch.float16).cuda()
+    vec = lambda: torch.empty(E, dtype=torch.float16, device='cuda')
+    for lay, lay2 in (('BJI', 'BJI'), ('IBJ', 'JBI'), ('JBI', 'BJI')):
+        din, ds, db = o.empty(lay2), vec(), vec()
+        o.bsb(to_layout(inp, 'BJI', lay), lay, dev(s), to_layout(dout, 'BJI', lay2), lay2, din, lay2, ds, db)
+        torch.cuda.synchronize()
+        w = ref.op_bsb(inp, s, dout)
+        assert_close(from_layout(din, 'BJI', lay2), w[0], name='DLN2')
+        assert_close(ds.float().cpu().numpy(), w[1], name='DS2', tol=2e-2)
+        assert_close(db.float().cpu().numpy(), w[2], name='DB2', tol=2e-2)
+        din, ds, db, dlb = o.empty(lay), vec(), vec(), vec()
+        o.ebsb(to_layout(inp, 'BJI', lay), lay, dev(s), to_layout(dout, 'BJI', lay2), lay2,
+               to_layout(d2, 'BJI', lay), lay, to_layout(dl, 'BJI', lay2), lay2, din, lay, ds, db, dlb)
+        torch.cuda.synchronize()
+        w = ref.op_ebsb(inp, s, dout, d2, dl)
+        assert_close(from_layout(din, 'BJI', lay), w[0], name='DLN1')
+        assert_close(ds.float().cpu().numpy(), w[1], name='DS1', tol=2e-2)
+        assert_close(db.float().cpu().numpy(), w[2], name='DB1', tol=2e-2)
+        assert_close(dlb.float().cpu().numpy(), w[3], name='DLINB2', tol=2e-2)
+        dbo = vec()
+        o.baob(to_layout(dout, 'BJI', lay), lay, dbo)
+        dx = o.empty(lay2)
+        o.bei(to_layout(inp, 'BJI', lay), lay, to_layout(d2, 'BJI', lay2), lay2, dx, lay2)
+        torch.cuda.synchronize()
+        assert_close(dbo.float().cpu().numpy(), ref.op_baob(dout), name='DBO', tol=2e-2)
+        assert_close(from_layout(dx, 'BJI', lay2), ref.op_bei(inp, d2), name='DX')
+
+
+@pytest.mark.parametrize('B,L,H,E', SIZES)
+def test_aib_baib(B, L, H, E):
+    o = _ops(B, L, H, E)
+    P = E // H
+    rng = np.random.default_rng(5)
+    w = h16(rng.normal(size=(3, P, H, B, L))); bias = h16(rng.normal(size=(3, P, H)))
+    for lin, lout, lb in (('QPHBJ', 'QPHBJ', 'QPH'), ('QPHBJ', 'QHBPJ', 'QPH'), ('QBJHP', 'QBJHP', 'QHP'),
+                          ('QJBPH', 'QBHJP', 'QHP')):
+        out = o.empty(lout)
+        o.aib(to_layout(w, 'QPHBJ', lin), lin, to_layout(bias, 'QPH', lb), lb, out, lout)
+        db = o.empty(lb)
+        o.baib(to_layout(w, 'QPHBJ', lin), lin, db, lb)
+        torch.cuda.synchronize()
+        assert_close(from_layout(out, 'QPHBJ', lout), ref.op_aib(w, bias), name='KKQQVV ' + lin)
+        assert_close(from_layout(db, 'QPH', lb), ref.op_baib(w), name='DBKQV ' + lin, tol=2e-2)
