@@ -275,8 +275,16 @@ def encoder(x, attn_wq, attn_wk, attn_wv, attn_wo, attn_in_b, attn_out_b, attn_s
 def encoder_backward(x, dy, fwd, attn_wq, attn_wk, attn_wv, attn_wo, attn_scale,
                      norm1_scale, norm2_scale, linear1_w, linear1_b, linear2_w, linear2_b,
                      softmax_mask=None, attn_dropout_mask=None, linear1_dropout_mask=None,
-                     ff_dropout_mask=None, activation='relu'):
+                     ff_dropout_mask=None, activation='relu', relu_gate=None):
     """Backward data + weights, transformer.py:212-285.  ``fwd`` = encoder()'s dict.
+
+    ``relu_gate`` ([B,L,U] of {0,1}) replaces ``ff1_linear > 0`` in the ReLU
+    derivative.  ReLU's derivative is discontinuous at 0, so a forward value that
+    an fp16 path rounds to the other side of 0 flips one gradient element by its
+    full size; parity tests of a reduced-precision device path therefore feed
+    the gate the device saved (its stored LIN1 > 0), exactly as they feed the
+    dropout masks.  The reference's kernel reads the gate from its stored LIN1 as
+    well (pytorch_module/block_bdrlb.cuh:72).
 
     Returns a dict: dx, dattn_wq/wk/wv/wo, dattn_in_b (q,k,v order), dattn_out_b,
     dnorm{1,2}_{scale,bias}, dlinear{1,2}_{w,b}, plus the intermediate gradients
@@ -291,7 +299,10 @@ def encoder_backward(x, dy, fwd, attn_wq, attn_wk, attn_wv, attn_wo, attn_scale,
     dff1 = linear_backward_data(f['ff1'], linear2_w, dff)                    # DDROP2
     dlinear2_w, dlinear2_b = linear_backward_weights(f['ff1'], linear2_w, dff, bias=linear2_b)
     dff1_act = dropout_backward_data(dff1, linear1_dropout_mask)
-    dff1_linear = act_bwd(f['ff1_linear'], dff1_act)                         # DLIN1
+    if relu_gate is not None and activation == 'relu':
+        dff1_linear = relu_gate * dff1_act
+    else:
+        dff1_linear = act_bwd(f['ff1_linear'], dff1_act)                     # DLIN1
     dnormed1_linear = linear_backward_data(f['normed1'], linear1_w, dff1_linear)  # DLIN1_LINW1
     dlinear1_w, dlinear1_b = linear_backward_weights(
         f['normed1'], linear1_w, dff1_linear, bias=linear1_b)
@@ -353,7 +364,7 @@ def module_params_to_numpy(p):
         linear2_w=np.ascontiguousarray(p['LINW2'].T), linear2_b=p['LINB2'])
 
 
-def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt'):
+def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', relu_gate=None):
     """Forward + backward with device-module naming.
 
     params: dict name -> array in canonical dim order (CANONICAL); X, DY [B,J,I];
@@ -376,7 +387,8 @@ def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt'):
                 activation=activation, ln_mode=ln_mode, **mk)
     g = encoder_backward(X, DY, f, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], scale,
                          a['norm1_scale'], a['norm2_scale'], a['linear1_w'], a['linear1_b'],
-                         a['linear2_w'], a['linear2_b'], activation=activation, **mk)
+                         a['linear2_w'], a['linear2_b'], activation=activation,
+                         relu_gate=relu_gate, **mk)
     B, J, I = X.shape
     out = {}
     pq = np.stack(f['attn_proj_q']); pk = np.stack(f['attn_proj_k']); pv = np.stack(f['attn_proj_v'])

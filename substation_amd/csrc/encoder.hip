@@ -601,7 +601,7 @@ int sub_encoder_forward(void* handle, void* const* ptrs, int n) {
 int sub_encoder_backward(void* handle, void* const* ptrs, int n) {
     return guarded([&] {
         Handle& h = as_handle(handle);
-        if (n != 2 + 2 * SUB_N_PARAMS + SUB_N_BWD + SUB_N_FWD + 2) fail("sub_encoder_backward: expected 64 pointers");
+        if (n != 1 + 2 * SUB_N_PARAMS + SUB_N_BWD + SUB_N_FWD + 2) fail("sub_encoder_backward: expected 64 pointers");
         need_cfg(h);
         for (int i = 0; i < n; ++i) if (!ptrs[i]) fail("sub_encoder_backward: null tensor pointer");
         BwdPtrs t; unpack_backward(h, ptrs, t);

@@ -77,7 +77,14 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
         want = ph.dropout_mask(shape, p, SEED, site, step=step, dtype=np.float64)
         assert (got[name] == want).all(), name + ' differs from the seeded oracle mask'
         masks[name] = want
-    want = ref.run_named(params_np, X_np, DY_np, masks, act)
+    # The ReLU gate is taken from the device's stored LIN1, like the masks: a
+    # pre-activation that fp16 rounds across 0 would otherwise flip whole
+    # gradient elements (see oracle.encoder_ref.encoder_backward).
+    gate = (got['LIN1'] > 0).astype(np.float64) if act == 'relu' else None
+    want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate)
+    if gate is not None:
+        flips = (gate != (want['LIN1'] > 0)).mean()
+        assert flips < 1e-3, f'{flips:.2e} of the ReLU gates differ from the oracle forward'
     return want, got
 
 
