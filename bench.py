@@ -1,0 +1,270 @@
+"""Benchmark of the fused encoder layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3|4|5] [--layouts mi355x|ref]
+
+A step is one forward + one backward pass of a single encoder layer over one
+batch of synthetic input (the protocol of pytorch_module/run_encoder.py:345-383).
+The default workload is BERT-large B=8 L=512 H=16 E=1024 fp16 with the four
+dropouts at p=0.1.  Prints ONE JSON line: ms per layer, the per-operator
+roofline measured live with HIP events on the launch stream, and the CPU
+baseline (the NumPy oracle on the reference's own CPU-sized case).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12        # B/s, MI355X HBM3E
+MFMA_PEAK_F16 = 2.5e15   # FLOP/s, MI355X dense fp16
+V100_MS = 6.71           # reference README.md:23, V100-SXM2, same layer and sizes
+
+CONFIGS = {
+    3: dict(B=8, L=512, H=16, E=1024, act='relu', w_std=0.02, b_std=0.02,
+            name='configs[2]: BERT-large encoder layer fwd+bwd B=8 L=512 H=16 E=1024 P=64 FF=4096 '
+                 'post-LN ReLU fp16, 4 dropouts p=0.1 seeded'),
+    4: dict(B=96, L=128, H=16, E=1024, act='relu', w_std=0.02, b_std=0.02,
+            name='configs[3]: BERT-large encoder layer fwd+bwd B=96 L=128 H=16 E=1024 fp16'),
+    5: dict(B=4, L=2048, H=32, E=4096, act='gelu', w_std=0.01, b_std=0.0,
+            name='configs[4]: wide encoder layer fwd+bwd B=4 L=2048 H=32 E=4096 P=128 FF=16384 GELU fp16'),
+}
+
+GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
+            'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
+
+
+def algorithmic_work(B, L, H, E):
+    """Per operator: ('hbm', bytes) or ('mfma', flops, bytes).  Bytes = each big
+    tensor read once + written once in fp16; flops = 2*batch*M*N*K."""
+    U, P = 4 * E, E // H
+    bji, bju, hbjk, q = B * L * E, B * L * U, H * B * L * L, 3 * B * L * E
+    w = {
+        'aib': ('hbm', 2 * q * 2), 'softmax': ('hbm', 4 * hbjk * 2), 'bs': ('hbm', 4 * hbjk * 2),
+        'bdrln1': ('hbm', 7 * bji * 2), 'bdrln2': ('hbm', 7 * bji * 2),
+        'blnrd1': ('hbm', 5 * bji * 2), 'blnrd2': ('hbm', 5 * bji * 2),
+        'bsb': ('hbm', 3 * bji * 2), 'ebsb': ('hbm', 5 * bji * 2), 'baob': ('hbm', bji * 2),
+        'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', 4 * bju * 2), 'bdrlb': ('hbm', 4 * bju * 2),
+        'baib': ('hbm', q * 2),
+    }
+    tok = B * L
+    proj = (2 * tok * 3 * E * E, 2 * (tok * E + 3 * E * E + 3 * tok * E))
+    attn = (2 * H * B * L * L * P, 2 * (2 * tok * E + hbjk))
+    outp = (2 * tok * E * E, 2 * (2 * tok * E + E * E))
+    ffn = (2 * tok * E * U, 2 * (tok * E + E * U + tok * U))
+    for n in ('QKV-fused', 'dXQKV-fused', 'dWQKV-fused'):
+        w[n] = ('mfma',) + proj
+    for n in ('QKT', 'gamma', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT'):
+        w[n] = ('mfma',) + attn
+    for n in ('out', 'dWout', 'dXout'):
+        w[n] = ('mfma',) + outp
+    for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):
+        w[n] = ('mfma',) + ffn
+    return w
+
+
+def make_encoder(cfg, layouts_name, profiling=False, seed=0x5EED):
+    import torch
+    from substation_amd import Encoder, layouts as L
+    lay = (L.mi355x_layouts() if layouts_name == 'mi355x'
+           else L.reference_layouts('bert-b8-l512-h16-e1024' if cfg['L'] >= 512 else 'bert-b96-l128-h16-e1024'))
+    enc = Encoder('unused', cfg['B'], cfg['L'], cfg['H'], cfg['E'], lay, torch.float16,
+                  0.1, 0.1, 0.1, 0.1, profiling=profiling, activation=cfg['act'], seed=seed)
+    g = torch.Generator().manual_seed(1000 + cfg['E'])
+    with torch.no_grad():
+        for name, _ in lay['params']:
+            p = getattr(enc, name)
+            t = torch.randn(p.shape, generator=g, dtype=torch.float32)
+            if name in ('S1', 'S2'):
+                t = torch.ones_like(t)
+            elif name in ('B1', 'B2'):
+                t = torch.zeros_like(t)
+            elif p.dim() == 1 or name == 'BKQV':
+                t = cfg['b_std'] * t
+            else:
+                t = cfg['w_std'] * t
+            p.copy_(t)
+    enc = enc.cuda()
+    sz = enc.sizes
+    shape = tuple(sz[d] for d in lay['input'][1])
+    X = torch.randn(shape, generator=g, dtype=torch.float32).half().cuda().requires_grad_(True)
+    DY = torch.randn(shape, generator=g, dtype=torch.float32).half().cuda()
+    return enc, X, DY
+
+
+def cpu_baseline(budget_s=20.0):
+    """The NumPy oracle (a port of substation/transformer.py + attention.py with
+    the reference's per-sample np.matmul structure) on the reference's own
+    CPU-runnable case: B=2 L=128 H=12 E=768 FF=3072 fp32 post-LN ReLU, p=0.1
+    masks fed, forward + backward."""
+    import numpy as np
+    from oracle import encoder_ref as ref
+    from oracle import philox_ref as ph
+    B, L, H, E = 2, 128, 12, 768
+    U, P = 4 * E, E // H
+    rng = np.random.default_rng(1001)
+    f32 = np.float32
+    params = dict(
+        WKQV=(0.02 * rng.normal(size=(3, P, H, E))).astype(f32), BKQV=np.zeros((3, P, H), f32),
+        WO=(0.02 * rng.normal(size=(E, P, H))).astype(f32), BO=np.zeros(E, f32),
+        S1=np.ones(E, f32), B1=np.zeros(E, f32), LINB1=np.zeros(U, f32),
+        LINW1=(0.02 * rng.normal(size=(E, U))).astype(f32), S2=np.ones(E, f32), B2=np.zeros(E, f32),
+        LINB2=np.zeros(E, f32), LINW2=(0.02 * rng.normal(size=(U, E))).astype(f32))
+    X = rng.normal(size=(B, L, E)).astype(f32); DY = rng.normal(size=(B, L, E)).astype(f32)
+    masks = dict(ATTN_DROP_MASK=ph.dropout_mask((H, B, L, L), 0.1, 1001, 0, dtype=f32),
+                 DROP1MASK=ph.dropout_mask((B, L, E), 0.1, 1001, 1, dtype=f32),
+                 DROP2MASK=ph.dropout_mask((B, L, U), 0.1, 1001, 2, dtype=f32),
+                 DROP3MASK=ph.dropout_mask((B, L, E), 0.1, 1001, 3, dtype=f32))
+    a = ref.module_params_to_numpy(params)
+    scale = f32(1.0 / np.sqrt(P))
+    sm = np.ascontiguousarray(np.einsum('HBJK->BHJK', masks['ATTN_DROP_MASK']))
+    mk = dict(softmax_mask=sm, attn_dropout_mask=masks['DROP1MASK'],
+              linear1_dropout_mask=masks['DROP2MASK'], ff_dropout_mask=masks['DROP3MASK'])
+
+    def one():
+        f = ref.encoder(X, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], a['attn_in_b'],
+                        a['attn_out_b'], scale, a['norm1_scale'], a['norm1_bias'], a['norm2_scale'],
+                        a['norm2_bias'], a['linear1_w'], a['linear1_b'], a['linear2_w'], a['linear2_b'],
+                        activation='relu', **mk)
+        ref.encoder_backward(X, DY, f, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], scale,
+                             a['norm1_scale'], a['norm2_scale'], a['linear1_w'], a['linear1_b'],
+                             a['linear2_w'], a['linear2_b'], activation='relu', **mk)
+
+    for _ in range(2):
+        one()
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 10 or (time.perf_counter() - t_start < budget_s and len(times) < 200):
+        t0 = time.perf_counter(); one(); times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > 2 * budget_s:
+            break
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get('num_threads', 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = int(os.environ.get('OMP_NUM_THREADS', '1'))
+    return {
+        'value': round(statistics.median(times) * 1e3, 3), 'unit': 'ms/layer', 'cores': threads,
+        'kind': 'port',
+        'sample': f'NumPy oracle, configs[0] shape B=2 L=128 H=12 E=768 FF=3072 fp32 fwd+bwd, p=0.1 masks fed, '
+                  f'median of {len(times)} runs; host has {os.cpu_count()} logical CPUs',
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--warmup', type=int, default=30)
+    ap.add_argument('--config', type=int, default=3, choices=sorted(CONFIGS))
+    ap.add_argument('--layouts', default='mi355x', choices=['mi355x', 'ref'])
+    ap.add_argument('--profile-steps', type=int, default=20)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--per-op', action='store_true', help='print the per-operator table to stderr')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this build runs the encoder layer on ONE GPU only (no collectives exist on '
+              'this path); run with --gpus 1', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print('bench.py: no GPU visible', file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    cfg = CONFIGS[args.config]
+    enc, X, DY = make_encoder(cfg, args.layouts)
+
+    params = list(enc.parameters())
+
+    def step():
+        X.grad = None
+        for q in params:       # as optimizer.zero_grad(set_to_none=True): no accumulate kernels
+            q.grad = None
+        Y = enc(X)
+        Y.backward(DY)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # Per-operator durations: HIP events recorded by the library around every
+    # launch, on the stream the kernels run on.
+    enc._handle.profile_enable(True)
+    per_op = {}
+    for _ in range(args.profile_steps):
+        X.grad = None
+        for q in params:
+            q.grad = None
+        Y = enc(X)
+        for n, ms in enc.profile():
+            per_op.setdefault(n, []).append(ms)
+        Y.backward(DY)
+        for n, ms in enc.profile():
+            per_op.setdefault(n, []).append(ms)
+    enc._handle.profile_enable(False)
+    work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'])
+    ops = []
+    for n, ts in per_op.items():
+        t = statistics.mean(ts) * 1e-3
+        kind = work[n]
+        if kind[0] == 'hbm':
+            ops.append(dict(op=n, bound='hbm', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e9, 1),
+                            peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(kind[1] / t / HBM_PEAK, 4),
+                            bytes=kind[1]))
+        else:
+            ops.append(dict(op=n, bound='mfma', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e12, 1),
+                            peak=MFMA_PEAK_F16 / 1e12, unit='TFLOP/s', frac=round(kind[1] / t / MFMA_PEAK_F16, 4),
+                            flops=kind[1], hbm_gbps=round(kind[2] / t / 1e9, 1)))
+    ops.sort(key=lambda o: -o['us'])
+    if not ops:        # --profile-steps 0: timing only
+        print(json.dumps({'metric': 'fwd+bwd ms/layer', 'value': round(ms_per_step, 4), 'unit': 'ms',
+                          'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                          'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False}))
+        return
+    dom = ops[0]
+    total_us = sum(o['us'] for o in ops)
+    fused = [o for o in ops if o['bound'] == 'hbm']
+    gemms = [o for o in ops if o['bound'] == 'mfma']
+    if args.per_op:
+        for o in ops:
+            print(json.dumps(o), file=sys.stderr)
+
+    out = {
+        'metric': 'fwd+bwd ms/layer BERT-large B8 L512 fp16' if args.config == 3 else 'fwd+bwd ms/layer',
+        'value': round(ms_per_step, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False,
+        'scaling': 'weak', 'vs_baseline': round(ms_per_step / V100_MS, 4) if args.config == 3 else None,
+        'dtype': 'fp16', 'data': 'synthetic',
+        'config': {'workload': cfg['name'], 'layouts': args.layouts,
+                   'baseline': 'reference README.md:23: 6.71 ms on V100-SXM2 (other hardware)'},
+        'roofline': {
+            'kernel': dom['op'], 'bound': dom['bound'], 'achieved': dom['achieved'], 'peak': dom['peak'],
+            'unit': dom['unit'], 'frac': dom['frac'], 'traffic': None,
+            'launch_us': dom['us'], 'launches_per_step': 1,
+        },
+        'op_time_us': round(total_us, 1),
+        'fused_ops': {'us': round(sum(o['us'] for o in fused), 1),
+                      'gbps': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / 1e9, 1),
+                      'frac_of_hbm_peak': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4)},
+        'contractions': {'us': round(sum(o['us'] for o in gemms), 1),
+                         'tflops': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / 1e12, 1),
+                         'frac_of_mfma_peak': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / MFMA_PEAK_F16, 4)},
+        'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac')} for o in ops],
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

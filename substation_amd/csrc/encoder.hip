@@ -370,8 +370,32 @@ void op_aib(Handle& h, const void* in, const Layout& lin_, const void* bias, con
 
 // dbias[q,p,h] = sum_{b,j} d[q,p,h,b,j]
 void op_baib(Handle& h, const void* d, const Layout& ld, void* dbias, const Layout& lbias) {
-    Space sp = make_space(h.sz, {dQ, dP, dH, dB}, dJ);
-    launch_baib(sp.rs, make_view(d, ld, sp), make_view(dbias, lbias, sp), h.stream);
+    const int64_t P = h.sz.n[dP], H = h.sz.n[dH];
+    if (ld.stride[dJ] == 1) {
+        // J contiguous: one wave sums the (b, j) block of each (q,p,h)
+        Space sp = make_space(h.sz, {dQ, dP, dH, dB}, dJ);
+        launch_baib(sp.rs, make_view(d, ld, sp), make_view(dbias, lbias, sp), h.stream);
+        return;
+    }
+    const bool hp_merged = ld.stride[dP] == 1 && ld.stride[dH] == P && lbias.stride[dP] == 1 &&
+                           lbias.stride[dH] == P;
+    if (hp_merged) {
+        // (h,p) is one contiguous run of H*P features in both tensors: a column
+        // reduction over (b, j) per q with full-width rows.
+        RowSpace rs{1, (int)h.sz.n[dQ], (int)h.sz.n[dB], (int)h.sz.n[dJ], (int)(H * P)};
+        View v; v.p = (half_t*)d; v.s0 = 0; v.s1 = ld.stride[dQ]; v.s2 = ld.stride[dB]; v.s3 = ld.stride[dJ];
+        v.sr = 1;
+        v.vec = ((H * P) % 8 == 0 && v.s1 % 8 == 0 && v.s2 % 8 == 0 && v.s3 % 8 == 0 &&
+                 (reinterpret_cast<uintptr_t>(d) & 15) == 0) ? 1 : 0;
+        ensure_ws(h, colreduce_ws_floats(rs, 1));
+        launch_colsum(rs, v, (half_t*)dbias, 0, lbias.stride[dQ], 1, h.ws, h.stream);
+        return;
+    }
+    // general: rows of P features, kept (q,h), summed over (b,j)
+    Space sp = make_space(h.sz, {dQ, dH, dB, dJ}, dP);
+    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
+    launch_colsum(sp.rs, make_view(d, ld, sp), (half_t*)dbias, lbias.stride[dQ], lbias.stride[dH],
+                  lbias.stride[dP], h.ws, h.stream);
 }
 
 void op_bei(Handle& h, const void* a, const Layout& la, const void* b, const Layout& lb_, void* o,

@@ -91,7 +91,8 @@ __device__ __forceinline__ void col_process(const RowSpace& rs, const ColArgs& a
     }
 }
 
-// grid.x = feature strips of lpr*8 features, grid.y = token chunks.
+// grid.x = feature strips of lpr*8 features, grid.y = token chunks, grid.z = kept
+// outer index (i0,i1).  The sums run over the two inner outer dims (i2,i3).
 template <int KIND>
 __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, float* ws, int lpr_log2,
                                                      long rows_per_block, long nrows) {
@@ -112,8 +113,10 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
     F8 fscale;
     if (KIND == COL_BSB || KIND == COL_EBSB) fscale = load8(a.v[5], 0, e0, nv);
     if (nv > 0) {
+        RowIdx ix;
+        ix.i1 = blockIdx.z % rs.n1; ix.i0 = blockIdx.z / rs.n1;
         for (long row = row_begin + wave * rpw + sub; row < row_end; row += WPB * rpw) {
-            RowIdx ix = row_index(rs, row);
+            ix.i3 = row % rs.n3; ix.i2 = row / rs.n3;
             col_process<KIND>(rs, a, ix, e0, nv, fscale, acc);
         }
     }
@@ -131,7 +134,7 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
             for (int t = tid; t < BLOCK; t += lpr)
 #pragma unroll
                 for (int i = 0; i < 8; ++i) tot[i] += red[t][i];
-            float* dst = ws + ((long)s * ntc + blockIdx.y) * rs.R + e0;
+            float* dst = ws + (((long)s * gridDim.z + blockIdx.z) * ntc + blockIdx.y) * rs.R + e0;
             for (int i = 0; i < nv; ++i) dst[i] = tot[i];
         }
     }
@@ -139,16 +142,34 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
 
 struct FinishArgs {
     half_t* out[3];
+    long ob0, ob1, of;      // output strides of the kept dims (i0, i1) and of the feature
+    int n1;
 };
 
-__global__ __launch_bounds__(BLOCK) void k_colfinish(const float* ws, FinishArgs o, int ns, int ntc, int R) {
-    long idx = (long)blockIdx.x * BLOCK + threadIdx.x;
-    if (idx >= (long)ns * R) return;
-    int s = (int)(idx / R), f = (int)(idx - (long)s * R);
-    const float* p = ws + (long)s * ntc * R + f;
+// Adds the ntc partials of every (sum, kept index, feature): 32 features x 8
+// slices per block, the slices combined through LDS.
+__global__ __launch_bounds__(BLOCK) void k_colfinish(const float* ws, FinishArgs o, int ns, int nbatch,
+                                                     int ntc, int R) {
+    __shared__ float red[8][33];
+    const int fl = threadIdx.x & 31, sl = threadIdx.x >> 5;
+    long idx = (long)blockIdx.x * 32 + fl;
+    const bool ok = idx < (long)ns * nbatch * R;
+    int s = 0, f = 0, z = 0;
     float t = 0.f;
-    for (int c = 0; c < ntc; ++c) t += p[(long)c * R];
-    o.out[s][f] = (half_t)t;
+    if (ok) {
+        long sz = idx / R; f = (int)(idx - sz * R);
+        s = (int)(sz / nbatch); z = (int)(sz - (long)s * nbatch);
+        const float* p = ws + sz * ntc * R + f;
+        for (int c = sl; c < ntc; c += 8) t += p[(long)c * R];
+    }
+    red[sl][fl] = t;
+    __syncthreads();
+    if (sl == 0 && ok) {
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) tot += red[i][fl];
+        o.out[s][(long)(z / o.n1) * o.ob0 + (long)(z % o.n1) * o.ob1 + (long)f * o.of] = (half_t)tot;
+    }
 }
 
 struct ColPlan {
@@ -157,16 +178,19 @@ struct ColPlan {
 };
 
 inline ColPlan col_plan(const RowSpace& rs) {
+    const long nbatch = (long)rs.n0 * rs.n1;
     ColPlan p;
     int chunks = (rs.R + 7) / 8;
     p.lpr_log2 = 0;
-    while ((1 << p.lpr_log2) < chunks && p.lpr_log2 < 6) ++p.lpr_log2;
+    // at most 16 lanes (128 features, 256 contiguous bytes) per row: more strips,
+    // fewer token chunks for the finishing kernel to add up
+    while ((1 << p.lpr_log2) < chunks && p.lpr_log2 < 4) ++p.lpr_log2;
     int lpr = 1 << p.lpr_log2;
     p.nstrips = (chunks + lpr - 1) / lpr;
-    long nrows = rs.rows();
+    long nrows = (long)rs.n2 * rs.n3;
     int rows_per_iter = WPB * (WAVE / lpr);
-    // aim for ~2048 blocks in total, at least two row-iterations per block
-    long want_tc = 2048 / p.nstrips; if (want_tc < 1) want_tc = 1;
+    // aim for ~1024 blocks in total, at least two row-iterations per block
+    long want_tc = 1024 / (p.nstrips * nbatch); if (want_tc < 1) want_tc = 1;
     long rpb = (nrows + want_tc - 1) / want_tc;
     if (rpb < 2L * rows_per_iter) rpb = 2L * rows_per_iter;
     rpb = (rpb + rows_per_iter - 1) / rows_per_iter * rows_per_iter;
@@ -183,13 +207,17 @@ void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hip
     if (rs.R <= 0) return;
     if (!ws) fail(std::string(what) + ": no reduction workspace");
     ColPlan p = col_plan(rs);
-    long nrows = rs.rows();
-    hipLaunchKernelGGL(k_colreduce<KIND>, dim3(p.nstrips, p.ntc), dim3(BLOCK), 0, st, rs, a, ws,
+    long nrows = (long)rs.n2 * rs.n3;
+    int nbatch = rs.n0 * rs.n1;
+    if (nrows == 0 || nbatch == 0) return;
+    if (nbatch > 65535) fail(std::string(what) + ": too many kept rows");
+    fo.n1 = rs.n1;
+    hipLaunchKernelGGL(k_colreduce<KIND>, dim3(p.nstrips, p.ntc, nbatch), dim3(BLOCK), 0, st, rs, a, ws,
                        p.lpr_log2, p.rows_per_block, nrows);
     check_launch(what);
-    long n = (long)NS * rs.R;
-    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((n + BLOCK - 1) / BLOCK)), dim3(BLOCK), 0, st,
-                       (const float*)ws, fo, NS, p.ntc, rs.R);
+    long n = (long)NS * nbatch * rs.R;
+    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((n + 31) / 32)), dim3(BLOCK), 0, st,
+                       (const float*)ws, fo, NS, nbatch, p.ntc, rs.R);
     check_launch(what);
 }
 
@@ -220,13 +248,13 @@ __global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, Vie
 
 size_t colreduce_ws_floats(const RowSpace& rs, int nsums) {
     ColPlan p = col_plan(rs);
-    return (size_t)nsums * p.ntc * rs.R;
+    return (size_t)nsums * rs.n0 * rs.n1 * p.ntc * rs.R;
 }
 
 void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
                 ColOut dbias, float* ws, hipStream_t st) {
     ColArgs a{}; a.v[0] = in; a.v[1] = dout; a.v[3] = din; a.v[5] = scale; a.act = 0;
-    FinishArgs fo{{dscale.p, dbias.p, nullptr}};
+    FinishArgs fo{{dscale.p, dbias.p, nullptr}, 0, 0, 1, 1};
     run_col<COL_BSB>(rs, a, fo, ws, st, "backward scale-bias");
 }
 
@@ -235,21 +263,28 @@ void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dline
                  hipStream_t st) {
     ColArgs a{}; a.v[0] = in; a.v[1] = dout1; a.v[2] = dout2; a.v[3] = din; a.v[4] = dlinear;
     a.v[5] = scale; a.act = 0;
-    FinishArgs fo{{dscale.p, dbias.p, dlinear_bias.p}};
+    FinishArgs fo{{dscale.p, dbias.p, dlinear_bias.p}, 0, 0, 1, 1};
     run_col<COL_EBSB>(rs, a, fo, ws, st, "extended backward scale-bias");
 }
 
 void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
                   int act, float* ws, hipStream_t st) {
     ColArgs a{}; a.v[0] = ddrop; a.v[1] = mask; a.v[2] = lin; a.v[3] = dlinear; a.act = act;
-    FinishArgs fo{{dbias.p, nullptr, nullptr}};
+    FinishArgs fo{{dbias.p, nullptr, nullptr}, 0, 0, 1, 1};
     run_col<COL_BDRLB>(rs, a, fo, ws, st, "backward dropout-activation-bias");
 }
 
 void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st) {
     ColArgs a{}; a.v[0] = datt; a.act = 0;
-    FinishArgs fo{{dbo.p, nullptr, nullptr}};
+    FinishArgs fo{{dbo.p, nullptr, nullptr}, 0, 0, 1, 1};
     run_col<COL_BAOB>(rs, a, fo, ws, st, "backward attention-output bias");
+}
+
+void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, long of, float* ws,
+                   hipStream_t st) {
+    ColArgs a{}; a.v[0] = d; a.act = 0;
+    FinishArgs fo{{out, nullptr, nullptr}, ob0, ob1, of, 1};
+    run_col<COL_BAOB>(rs, a, fo, ws, st, "column sum");
 }
 
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st) {

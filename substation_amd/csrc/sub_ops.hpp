@@ -33,8 +33,9 @@ void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, Vie
 void launch_add(const RowSpace& rs, View a, View b, View out, hipStream_t st);
 
 // --- column reductions -------------------------------------------------------
-// Sums over all rows of the row space, one result per row element.  `ws` is
-// fp32 scratch of at least colreduce_ws_floats() elements.
+// Sums over the two inner outer dims (n2, n3) of the row space, one result per
+// (n0, n1, row element).  `ws` is fp32 scratch of at least colreduce_ws_floats()
+// elements.
 struct ColOut {
     half_t* p;   // dense [R]
 };
@@ -47,6 +48,9 @@ void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dline
 void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
                   int act, float* ws, hipStream_t st);
 void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st);
+// out[i0,i1,e] = sum over (i2,i3) of d; out strides ob0, ob1 (kept dims) and of.
+void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, long of, float* ws,
+                   hipStream_t st);
 // Row sums: out[row-group] = sum over (n3, R) for each (n0,n1,n2): baib.
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
 
