@@ -11,6 +11,8 @@
 // are always 8 consecutive k per lane.  The output is produced transposed in the
 // accumulators (4 consecutive n per lane), staged through LDS and written as
 // full 128-bit rows.
+#include <cstdlib>
+
 #include "sub_ops.hpp"
 
 namespace sub {
@@ -58,98 +60,154 @@ __global__ __launch_bounds__(256) void k_gemm_scalar(GemmArgs g, long total) {
 // ---------------------------------------------------------------------------
 // MFMA kernel.  256 threads = 2x2 waves; each wave owns TM x TN tiles of 32x32.
 // ---------------------------------------------------------------------------
-constexpr int BK = 64;            // k per LDS tile: one 128-byte line per row
+constexpr int BK = 64;            // k per LDS tile
 
-// LDS tile: rows of 64 halves (eight 16-byte slots); the slot index is xor-ed
-// with a function of the row so that both the fragment reads (32 consecutive
-// rows, one slot) and the transposing writes (rows 8 apart) spread over banks.
-__device__ __forceinline__ int lds_off(int row, int slot) {
-    return row * BK + ((slot ^ (row ^ (row >> 3))) & 7) * 8;
-}
+#ifdef SUB_GEMM_ABLATE
+// Performance experiments only (results are wrong): bit 0 skips the global
+// loads and LDS writes after the first tile, bit 1 skips the fragment reads.
+__device__ int g_ablate = 0;
+#define SUB_ABLATE(bit) (g_ablate & (bit))
+#else
+#define SUB_ABLATE(bit) 0
+#endif
+constexpr int MC_PAD = 32;        // halves of padding per k-row of a free-dim-contiguous tile
 
+typedef short s4v __attribute__((ext_vector_type(4)));
+
+// One operand tile in LDS: ROWS (free dim) x BK (k).
+//
+// KC (k contiguous in memory): rows of 64 halves = eight 16-byte slots, the slot
+// index xor-ed with a function of the row so that the fragment reads (32
+// consecutive rows, one slot) spread over the banks.  A fragment is one
+// ds_read_b128: 8 consecutive k of one row.
+//
+// !KC (free dim contiguous in memory): the tile is stored as it lies in memory,
+// [k][free] with a padded pitch, and fragments are gathered with the LDS
+// transpose read ds_read_b64_tr_b16.  Within each group of 16 lanes, lane i of
+// that instruction receives, as element e, the (i%4)-th half of the 8
+// bytes addressed by lane 4e + i/4.  With lane l addressing
+// T[k0 + l/4][m0 + 4*(l%4) ..+3], lane i ends up with T[k0 + 0..3][m0 + i]:
+// four consecutive k of its own row, which is what the matrix core wants.
 template <int ROWS, bool KC>
-struct TileLoader {
-    // ROWS rows (free dim) x BK k.  KC: k contiguous in memory, else the free dim.
-    static constexpr int NV = ROWS / 32;          // 16-byte loads per thread
-    static_assert(KC || NV % 4 == 0, "transposing loader needs at least 128 rows");
+struct Tile {
+    static constexpr int PITCH = KC ? BK : ROWS + MC_PAD;            // halves
+    static constexpr int HALVES = KC ? ROWS * BK : BK * (ROWS + MC_PAD);
+    static constexpr int NV = ROWS / 32;                              // 16-byte loads per thread
+    static constexpr int VPR = ROWS / 8;                              // vectors per k-row (!KC)
+
+    static __device__ __forceinline__ int kc_off(int row, int slot) {
+        return row * BK + ((slot ^ (row ^ (row >> 3))) & 7) * 8;
+    }
 
     // base points at (free0, k-tile start) of the current batch; sF / sK are the
-    // strides of the free dim and of k; nfree / nk are the extents left.
-    static __device__ __forceinline__ void load(h8 (&v)[NV], const half_t* base, long sF, long sK,
-                                                int nfree, int nk, int tid) {
-        if (KC) {
+    // strides of the free dim and of k; nfree / nk the extents left.
+    // Per-thread element offsets of its NV vectors within a tile (constant over
+    // the k loop) and, for edge tiles, which of them lie inside the free extent.
+    static __device__ __forceinline__ void offsets(unsigned (&off)[NV], unsigned& okmask, long sF, long sK,
+                                                   int nfree, int tid) {
+        okmask = 0;
 #pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                int id = tid + i * 256;
+        for (int i = 0; i < NV; ++i) {
+            int id = tid + i * 256;
+            if (KC) {
                 int row = id >> 3, slot = id & 7;
-                bool ok = row < nfree && slot * 8 + 8 <= nk;
-                if (ok) v[i] = *reinterpret_cast<const h8*>(base + (long)row * sF + slot * 8);
-                else v[i] = (h8)(half_t)0.0f;
+                off[i] = (unsigned)((long)row * sF + slot * 8);
+                okmask |= (row < nfree ? 1u : 0u) << i;
+            } else {
+                int k = id / VPR, mv = id % VPR;
+                off[i] = (unsigned)((long)k * sK + mv * 8);
+                okmask |= (mv * 8 + 8 <= nfree ? 1u : 0u) << i;
             }
-        } else {
-            constexpr int FB = ROWS / 8;          // 8-wide blocks along the free dim
-            constexpr int KQ = 256 / FB;          // k-quads covered per pass
-            int fb = tid % FB, kq = tid / FB;
+        }
+    }
+
+    // CHECK = false: the whole tile is inside the matrix, no predication.
+    // `tile` is wave-uniform; nk = k extent left at the start of this tile.
+    template <bool CHECK>
+    static __device__ __forceinline__ void load(h8 (&v)[NV], const half_t* tile, const unsigned (&off)[NV],
+                                                unsigned okmask, int nk, int tid) {
 #pragma unroll
-            for (int p = 0; p < NV / 4; ++p)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    int k = (p * KQ + kq) * 4 + i;
-                    bool ok = fb * 8 + 8 <= nfree && k < nk;
-                    if (ok) v[p * 4 + i] = *reinterpret_cast<const h8*>(base + (long)k * sK + fb * 8);
-                    else v[p * 4 + i] = (h8)(half_t)0.0f;
-                }
+        for (int i = 0; i < NV; ++i) {
+            const h8* p = reinterpret_cast<const h8*>(tile + off[i]);
+            if (!CHECK) {
+                v[i] = *p;
+            } else {
+                int id = tid + i * 256;
+                bool kok = KC ? ((id & 7) * 8 + 8 <= nk) : (id / VPR < nk);
+                v[i] = (h8)(half_t)0.0f;
+                if (kok && ((okmask >> i) & 1u)) v[i] = *p;
+            }
         }
     }
 
     static __device__ __forceinline__ void store(const h8 (&v)[NV], half_t* lds, int tid) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            int id = tid + i * 256;
+            if (KC) {
+                *reinterpret_cast<h8*>(lds + kc_off(id >> 3, id & 7)) = v[i];
+            } else {
+                *reinterpret_cast<h8*>(lds + (id / VPR) * PITCH + (id % VPR) * 8) = v[i];
+            }
+        }
+    }
+
+    // Fragment of the 32-row block starting at row0 for k-step ks (16 k): lane
+    // (l32 = lane%32, hi = lane/32) gets k = ks*16 + 8*hi + 0..7 of row row0+l32.
+    static __device__ __forceinline__ h8 frag(const half_t* lds, int row0, int ks, int lane) {
         if (KC) {
-#pragma unroll
-            for (int i = 0; i < NV; ++i) {
-                int id = tid + i * 256;
-                int row = id >> 3, slot = id & 7;
-                *reinterpret_cast<h8*>(lds + lds_off(row, slot)) = v[i];
-            }
+            return *reinterpret_cast<const h8*>(lds + kc_off(row0 + (lane & 31), ks * 2 + (lane >> 5)));
         } else {
-            constexpr int FB = ROWS / 8;
-            constexpr int KQ = 256 / FB;
-            int fb = tid % FB, kq = tid / FB;
-#pragma unroll
-            for (int p = 0; p < NV / 4; ++p) {
-                int kcol = (p * KQ + kq) * 4;     // first of 4 consecutive k
-#pragma unroll
-                for (int r = 0; r < 8; ++r) {
-                    h4 w;
-                    w[0] = v[p * 4 + 0][r]; w[1] = v[p * 4 + 1][r];
-                    w[2] = v[p * 4 + 2][r]; w[3] = v[p * 4 + 3][r];
-                    int row = fb * 8 + r;
-                    *reinterpret_cast<h4*>(lds + lds_off(row, kcol >> 3) + (kcol & 7)) = w;
-                }
-            }
+            const int g = lane >> 4, l = lane & 15;
+            const int k = ks * 16 + 8 * (g >> 1) + (l >> 2);
+            const int m = row0 + 16 * (g & 1) + 4 * (l & 3);
+            const half_t* p = lds + k * PITCH + m;
+            typedef s4v __attribute__((address_space(3))) * lds_s4;
+            s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p));
+            s4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p + 4 * PITCH));
+            typedef short s8 __attribute__((ext_vector_type(8)));
+            s8 r = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(h8, r);
         }
     }
 };
 
-template <int TM, int TN, bool AKC, bool BKC>
+template <int TM, int TN, bool AKC, bool BKC, bool FULL>
 __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
     constexpr int BM = 64 * TM, BN = 64 * TN;
-    constexpr int TILE_A = BM * BK, TILE_B = BN * BK;             // halves
-    constexpr int STAGE_PITCH = 32 * TN + 8;                       // halves
-    constexpr int STAGE_WAVE = 32 * STAGE_PITCH;                   // one 32-row slab per wave
-    constexpr int LDS_TILES = 2 * (TILE_A + TILE_B);
-    constexpr int LDS_STAGE = 4 * STAGE_WAVE;
-    constexpr int LDS_HALVES = LDS_TILES > LDS_STAGE ? LDS_TILES : LDS_STAGE;
+    using TA = Tile<BM, AKC>;
+    using TB = Tile<BN, BKC>;
+    constexpr int STAGE = TA::HALVES + TB::HALVES;                   // one pipeline stage
+    constexpr int STAGE_PITCH = 32 * TN + 8;                          // halves
+    constexpr int STAGE_WAVE = 32 * STAGE_PITCH;                      // one 32-row slab per wave
+    constexpr int LDS_HALVES = 2 * STAGE > 4 * STAGE_WAVE ? 2 * STAGE : 4 * STAGE_WAVE;
     __shared__ __attribute__((aligned(16))) half_t lds[LDS_HALVES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, hi = lane >> 5;
 
-    // batch offsets
-    long bz = blockIdx.z;
+    // Workgroup -> tile.  Workgroups are dealt round-robin to the 8 XCDs (each
+    // with its own L2), so consecutive logical tiles are given to one XCD, and
+    // within a batch tiles are walked in groups of 8 tile-rows so that the
+    // workgroups resident together share A and B tiles in that L2.
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    long lid = blockIdx.x;
+    {
+        const long nblocks = gridDim.x;
+        if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
+    }
+    const int per_batch = tiles_m * tiles_n;
+    long bz = lid / per_batch;
+    int r = (int)(lid - bz * per_batch);
+    constexpr int GM = 8;
+    const int grp = r / (GM * tiles_n), first_m = grp * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int rr = r - grp * GM * tiles_n;
+    const int tile_m = first_m + rr % gsz, tile_n = rr / gsz;
     long b2 = bz % g.nb2; long t = bz / g.nb2;
     long b1 = t % g.nb1; long b0 = t / g.nb1;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
     const half_t* Ab = g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM;
     const half_t* Bb = g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN;
     const int mleft = g.M - m0, nleft = g.N - n0;
@@ -165,54 +223,93 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    using LA = TileLoader<BM, AKC>;
-    using LB = TileLoader<BN, BKC>;
-    h8 ra[LA::NV], rb[LB::NV];
+    // Software pipeline: two register sets hold the global loads of the next two
+    // k-tiles (issued one and two iterations ahead), two LDS stages hold the
+    // current tile and the one being written.
+    h8 ra0[TA::NV], rb0[TB::NV], ra1[TA::NV], rb1[TB::NV];
+    unsigned offa[TA::NV], offb[TB::NV], oka, okb;
+    TA::offsets(offa, oka, g.sAM, g.sAK1, mleft, tid);
+    TB::offsets(offb, okb, g.sBN, g.sBK1, nleft, tid);
 
-#define SUB_GEMM_ISSUE(kt_)                                                                       \
+    // Running (wave-uniform) pointers to the next k-tile to fetch.  Past the last
+    // tile they stay on it: the surplus prefetches re-read valid memory and are
+    // never consumed, which keeps the loop body free of branches.
+    const half_t* pa = Ab;
+    const half_t* pb = Bb;
+    int kin = 0, fetched = 0;
+    const long stepA = (long)BK * g.sAK1, stepB = (long)BK * g.sBK1;
+    const long wrapA = g.sAK0 - (long)(tiles_per_k1 - 1) * stepA;
+    const long wrapB = g.sBK0 - (long)(tiles_per_k1 - 1) * stepB;
+
+#define SUB_GEMM_ISSUE(RA, RB)                                                                    \
     do {                                                                                          \
-        int k0_ = (kt_) / tiles_per_k1, kk_ = ((kt_) - k0_ * tiles_per_k1) * BK;                  \
-        LA::load(ra, Ab + (long)k0_ * g.sAK0 + (long)kk_ * g.sAK1, g.sAM, g.sAK1, mleft,          \
-                 g.K1 - kk_, tid);                                                                \
-        LB::load(rb, Bb + (long)k0_ * g.sBK0 + (long)kk_ * g.sBK1, g.sBN, g.sBK1, nleft,          \
-                 g.K1 - kk_, tid);                                                                \
+        TA::template load<!FULL>(RA, pa, offa, oka, g.K1 - kin * BK, tid);                        \
+        TB::template load<!FULL>(RB, pb, offb, okb, g.K1 - kin * BK, tid);                        \
+        const bool more_ = fetched + 1 < nkt;                                                     \
+        const bool wrap_ = kin + 1 == tiles_per_k1;                                               \
+        pa += more_ ? (wrap_ ? wrapA : stepA) : 0;                                                \
+        pb += more_ ? (wrap_ ? wrapB : stepB) : 0;                                                \
+        kin = more_ ? (wrap_ ? 0 : kin + 1) : kin;                                                \
+        fetched += more_ ? 1 : 0;                                                                 \
     } while (0)
 
-    SUB_GEMM_ISSUE(0);
-    LA::store(ra, lds, tid);
-    LB::store(rb, lds + TILE_A, tid);
+#define SUB_GEMM_COMPUTE(stage_)                                                                  \
+    do {                                                                                          \
+        const half_t* sA = lds + (stage_) * STAGE;                                                \
+        const half_t* sB = sA + TA::HALVES;                                                       \
+        h8 fa[2][TM], fb[2][TN];                                                                  \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                            \
+            fa[0][i] = TA::frag(sA, (wm * TM + i) * 32, 0, lane);                                 \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
+            fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
+        _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
+            if (ks + 1 < BK / 16 && !SUB_ABLATE(2)) {                                             \
+                _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
+                    fa[(ks + 1) & 1][i] = TA::frag(sA, (wm * TM + i) * 32, ks + 1, lane);         \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
+                    fb[(ks + 1) & 1][j] = TB::frag(sB, (wn * TN + j) * 32, ks + 1, lane);         \
+            }                                                                                     \
+            /* D^T tiles: rows of the MFMA result run along n, columns along m. */                \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                        \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][j], fa[ks & 1][i], \
+                                                                       acc[i][j], 0, 0, 0);       \
+        }                                                                                         \
+    } while (0)
+
+#define SUB_GEMM_STORE(stage_, RA, RB)                                                            \
+    do {                                                                                          \
+        half_t* dA = lds + (stage_) * STAGE;                                                      \
+        TA::store(RA, dA, tid);                                                                   \
+        TB::store(RB, dA + TA::HALVES, tid);                                                      \
+    } while (0)
+
+    SUB_GEMM_ISSUE(ra0, rb0);          // tile 0
+    SUB_GEMM_ISSUE(ra1, rb1);          // tile 1 (or tile 0 again)
+    SUB_GEMM_STORE(0, ra0, rb0);
     __syncthreads();
 
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int cur = kt & 1;
-        const half_t* sA = lds + cur * (TILE_A + TILE_B);
-        const half_t* sB = sA + TILE_A;
-        if (kt + 1 < nkt) SUB_GEMM_ISSUE(kt + 1);
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            h8 fa[TM], fb[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-                fa[i] = *reinterpret_cast<const h8*>(sA + lds_off(wm * 32 * TM + i * 32 + l32, ks * 2 + hi));
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-                fb[j] = *reinterpret_cast<const h8*>(sB + lds_off(wn * 32 * TN + j * 32 + l32, ks * 2 + hi));
-            // D^T tiles: rows of the MFMA result run along n, columns along m.
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < nkt) {
-            half_t* dA = lds + (cur ^ 1) * (TILE_A + TILE_B);
-            LA::store(ra, dA, tid);
-            LB::store(rb, dA + TILE_A, tid);
-        }
+    // Step 2p: stage 0 holds tile 2p, set 1 holds tile 2p+1 in flight, set 0 is free.
+    const int npairs = nkt >> 1;
+    const bool mem = !SUB_ABLATE(1);
+    for (int p = 0; p < npairs; ++p) {
+        if (mem) SUB_GEMM_ISSUE(ra0, rb0);        // tile 2p+2
+        SUB_GEMM_COMPUTE(0);
+        if (mem) SUB_GEMM_STORE(1, ra1, rb1);     // tile 2p+1
+        __syncthreads();
+        if (mem) SUB_GEMM_ISSUE(ra1, rb1);        // tile 2p+3
+        SUB_GEMM_COMPUTE(1);
+        if (mem) SUB_GEMM_STORE(0, ra0, rb0);     // tile 2p+2 (a surplus copy when 2p+2 == nkt)
         __syncthreads();
     }
-
+    if (nkt & 1) {
+        SUB_GEMM_COMPUTE(0);
+        __syncthreads();                          // the epilogue reuses the tile memory
+    }
+#undef SUB_GEMM_COMPUTE
+#undef SUB_GEMM_STORE
 #undef SUB_GEMM_ISSUE
+
     // Epilogue: per 32-row slab, accumulators -> LDS (8-byte packs of 4
     // consecutive n) -> 16-byte row segments -> global.
     half_t* stage = lds + wave * STAGE_WAVE;
@@ -308,13 +405,28 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     return ok ? 1 : 0;
 }
 
+// Block tile for a problem: 22 = 128x128, 42 = 256x128, 44 = 256x256.
+int pick_tile(const GemmArgs& a, long batch) {
+    (void)a; (void)batch;
+    return 22;
+}
+
+template <int TM, int TN, bool FULL>
+void launch_mfma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
+    if (akc && bkc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, true, true, FULL>), grid, dim3(256), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, true, false, FULL>), grid, dim3(256), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, true, FULL>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, false, FULL>), grid, dim3(256), 0, st, a);
+}
+
 template <int TM, int TN>
 void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, hipStream_t st) {
-    dim3 grid((a.N + 64 * TN - 1) / (64 * TN), (a.M + 64 * TM - 1) / (64 * TM), (unsigned)batch);
-    if (akc && bkc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, true, true>), grid, dim3(256), 0, st, a);
-    else if (akc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, true, false>), grid, dim3(256), 0, st, a);
-    else if (bkc) hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, true>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, false>), grid, dim3(256), 0, st, a);
+    long nblocks = (long)((a.N + 64 * TN - 1) / (64 * TN)) * ((a.M + 64 * TM - 1) / (64 * TM)) * batch;
+    if (nblocks > 0x7fffffffL) fail("gemm: too many tiles");
+    dim3 grid((unsigned)nblocks);
+    const bool full = a.M % (64 * TM) == 0 && a.N % (64 * TN) == 0 && a.K1 % BK == 0;
+    if (full) launch_mfma2<TM, TN, true>(a, akc, bkc, grid, st);
+    else launch_mfma2<TM, TN, false>(a, akc, bkc, grid, st);
 }
 
 }  // namespace
@@ -330,12 +442,15 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
                  const GemmEpilogue& ep, hipStream_t st) {
     long batch = s.batch();
     if (batch == 0 || s.M == 0 || s.N == 0) return;
-    if (batch > 65535) fail("gemm: more than 65535 batches");
     Canon c = canonicalise(s, A, B, C, alpha, ep);
     bool akc = false, bkc = false;
     int kind = pick_kind(c, akc, bkc);
     if (kind == 1) {
-        launch_mfma<2, 2>(c.a, akc, bkc, batch, st);
+        static const int force = [] { const char* e = getenv("SUB_GEMM_TILE"); return e ? atoi(e) : 0; }();
+        int tile = force ? force : pick_tile(c.a, batch);
+        if (tile == 44) launch_mfma<4, 4>(c.a, akc, bkc, batch, st);
+        else if (tile == 42) launch_mfma<4, 2>(c.a, akc, bkc, batch, st);
+        else launch_mfma<2, 2>(c.a, akc, bkc, batch, st);
     } else {
         long total = batch * (long)c.a.M * c.a.N;
         long blocks = (total + 255) / 256;
