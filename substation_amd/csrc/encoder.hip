@@ -71,7 +71,47 @@ Space make_space(const Sizes& sz, std::initializer_list<int> outer, int rdim) {
     s.rdim = rdim;
     s.rs.n0 = n[0]; s.rs.n1 = n[1]; s.rs.n2 = n[2]; s.rs.n3 = n[3];
     s.rs.R = (int)sz.n[rdim];
+    s.rs.flat = (n[0] == 1 && n[1] == 1 && n[2] == 1) ? 1 : 0;
     return s;
+}
+
+// Merges adjacent outer dims that every view walks with one stride
+// (s[i] == n[i+1] * s[i+1]), so that the kernels skip the row -> index
+// divisions; the canonical row numbering (and with it the dropout mask) is
+// unchanged.  `keep` leading outer dims are left alone (kept dims of the column
+// reductions).
+void flatten(RowSpace& rs, std::initializer_list<View*> views, int keep = 0) {
+    int n[4] = {rs.n0, rs.n1, rs.n2, rs.n3};
+    auto stride = [](View* v, int i) -> long& {
+        return i == 0 ? v->s0 : i == 1 ? v->s1 : i == 2 ? v->s2 : v->s3;
+    };
+    bool changed = true;
+    while (changed) {
+        changed = false;
+        for (int i = 2; i >= keep && !changed; --i) {
+            bool ok = n[i] == 1;
+            if (ok) {
+                // an extent-1 dim is only worth dropping if a real dim lies outside it
+                bool outer = false;
+                for (int j = keep; j < i; ++j) outer = outer || n[j] != 1;
+                if (!outer) continue;
+            } else {
+                ok = true;
+                for (View* v : views) ok = ok && stride(v, i) == (long)n[i + 1] * stride(v, i + 1);
+                if (!ok) continue;
+            }
+            n[i + 1] *= n[i];
+            for (int j = i; j > keep; --j) {
+                n[j] = n[j - 1];
+                for (View* v : views) stride(v, j) = stride(v, j - 1);
+            }
+            n[keep] = 1;
+            for (View* v : views) stride(v, keep) = 0;
+            changed = true;
+        }
+    }
+    rs.n0 = n[0]; rs.n1 = n[1]; rs.n2 = n[2]; rs.n3 = n[3];
+    rs.flat = (n[0] == 1 && n[1] == 1 && n[2] == 1) ? 1 : 0;
 }
 
 View make_view(const void* p, const Layout& l, const Space& sp) {
@@ -278,15 +318,19 @@ void op_softmax(Handle& h, const void* beta, const Layout& lb, void* alpha, cons
                 void* mask, const Layout& lm, void* drop, const Layout& ld, float scale, float p,
                 uint32_t site) {
     Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
-    launch_softmax(sp.rs, make_view(beta, lb, sp), make_view(alpha, la, sp), make_view(mask, lm, sp),
-                   make_view(drop, ld, sp), scale, make_key(h, site, p), h.stream);
+    View vb = make_view(beta, lb, sp), va = make_view(alpha, la, sp), vm = make_view(mask, lm, sp),
+         vd = make_view(drop, ld, sp);
+    flatten(sp.rs, {&vb, &va, &vm, &vd});
+    launch_softmax(sp.rs, vb, va, vm, vd, scale, make_key(h, site, p), h.stream);
 }
 
 void op_bs(Handle& h, const void* alpha, const Layout& la, const void* mask, const Layout& lm,
            const void* ddrop, const Layout& ld, void* dbeta, const Layout& lo, float scale) {
     Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
-    launch_bs(sp.rs, make_view(alpha, la, sp), make_view(mask, lm, sp), make_view(ddrop, ld, sp),
-              make_view(dbeta, lo, sp), scale, h.stream);
+    View va = make_view(alpha, la, sp), vm = make_view(mask, lm, sp), vd = make_view(ddrop, ld, sp),
+         vo = make_view(dbeta, lo, sp);
+    flatten(sp.rs, {&va, &vm, &vd, &vo});
+    launch_bs(sp.rs, va, vm, vd, vo, scale, h.stream);
 }
 
 void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, const Layout& lres,
@@ -296,29 +340,32 @@ void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, 
               const Layout& listd, float p, uint32_t site) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     int R = sp.rs.R;
-    launch_bdrln(sp.rs, make_view(in, lin_, sp), make_view(resid, lres, sp), vector_view(linear_bias, R),
-                 vector_view(scale, R), vector_view(bias, R), make_view(lin, llin, sp),
-                 make_view(mask, lmask, sp), make_view(diff, ldiff, sp), make_view(normed, lnorm, sp),
-                 make_view(out, lout, sp), make_view(istd, listd, sp), make_key(h, site, p), h.eps,
-                 h.stream);
+    View vi = make_view(in, lin_, sp), vr = make_view(resid, lres, sp), vl = make_view(lin, llin, sp),
+         vm = make_view(mask, lmask, sp), vd = make_view(diff, ldiff, sp), vn = make_view(normed, lnorm, sp),
+         vo = make_view(out, lout, sp), vs = make_view(istd, listd, sp);
+    flatten(sp.rs, {&vi, &vr, &vl, &vm, &vd, &vn, &vo, &vs});
+    launch_bdrln(sp.rs, vi, vr, vector_view(linear_bias, R), vector_view(scale, R), vector_view(bias, R),
+                 vl, vm, vd, vn, vo, vs, make_key(h, site, p), h.eps, h.stream);
 }
 
 void op_blnrd(Handle& h, const void* dout, const Layout& ldout, const void* istd, const Layout& listd,
               const void* diff, const Layout& ldiff, const void* mask, const Layout& lmask,
               void* d_ln_in, const Layout& l1, void* d_drop_in, const Layout& l2) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
-    launch_blnrd(sp.rs, make_view(dout, ldout, sp), make_view(istd, listd, sp), make_view(diff, ldiff, sp),
-                 make_view(mask, lmask, sp), make_view(d_ln_in, l1, sp), make_view(d_drop_in, l2, sp),
-                 h.stream);
+    View vg = make_view(dout, ldout, sp), vs = make_view(istd, listd, sp), vd = make_view(diff, ldiff, sp),
+         vm = make_view(mask, lmask, sp), v1 = make_view(d_ln_in, l1, sp), v2 = make_view(d_drop_in, l2, sp);
+    flatten(sp.rs, {&vg, &vs, &vd, &vm, &v1, &v2});
+    launch_blnrd(sp.rs, vg, vs, vd, vm, v1, v2, h.stream);
 }
 
 void op_bad(Handle& h, const void* in, const Layout& lin_, const void* bias, void* lin,
             const Layout& llin, void* mask, const Layout& lmask, void* out, const Layout& lout,
             float p, uint32_t site) {
     Space sp = make_space(h.sz, {dB, dJ}, dU);
-    launch_bad(sp.rs, make_view(in, lin_, sp), vector_view(bias, sp.rs.R), make_view(lin, llin, sp),
-               make_view(mask, lmask, sp), make_view(out, lout, sp), h.act, make_key(h, site, p),
-               h.stream);
+    View vi = make_view(in, lin_, sp), vl = make_view(lin, llin, sp), vm = make_view(mask, lmask, sp),
+         vo = make_view(out, lout, sp);
+    flatten(sp.rs, {&vi, &vl, &vm, &vo});
+    launch_bad(sp.rs, vi, vector_view(bias, sp.rs.R), vl, vm, vo, h.act, make_key(h, site, p), h.stream);
 }
 
 void op_bsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* dout,
@@ -365,7 +412,9 @@ void op_aib(Handle& h, const void* in, const Layout& lin_, const void* bias, con
     const int canon[5] = {dQ, dP, dH, dB, dJ};
     for (int d : canon) if (d != r) outer[k++] = d;
     Space sp = make_space(h.sz, {outer[0], outer[1], outer[2], outer[3]}, r);
-    launch_add(sp.rs, make_view(in, lin_, sp), make_view(bias, lbias, sp), make_view(out, lout, sp), h.stream);
+    View vi = make_view(in, lin_, sp), vb = make_view(bias, lbias, sp), vo = make_view(out, lout, sp);
+    flatten(sp.rs, {&vi, &vb, &vo});
+    launch_add(sp.rs, vi, vb, vo, h.stream);
 }
 
 // dbias[q,p,h] = sum_{b,j} d[q,p,h,b,j]
@@ -401,7 +450,9 @@ void op_baib(Handle& h, const void* d, const Layout& ld, void* dbias, const Layo
 void op_bei(Handle& h, const void* a, const Layout& la, const void* b, const Layout& lb_, void* o,
             const Layout& lo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
-    launch_add(sp.rs, make_view(a, la, sp), make_view(b, lb_, sp), make_view(o, lo, sp), h.stream);
+    View va = make_view(a, la, sp), vb = make_view(b, lb_, sp), vo = make_view(o, lo, sp);
+    flatten(sp.rs, {&va, &vb, &vo});
+    launch_add(sp.rs, va, vb, vo, h.stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -114,9 +114,9 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
     if (KIND == COL_BSB || KIND == COL_EBSB) fscale = load8(a.v[5], 0, e0, nv);
     if (nv > 0) {
         RowIdx ix;
-        ix.i1 = blockIdx.z % rs.n1; ix.i0 = blockIdx.z / rs.n1;
-        for (long row = row_begin + wave * rpw + sub; row < row_end; row += WPB * rpw) {
-            ix.i3 = row % rs.n3; ix.i2 = row / rs.n3;
+        ix.i1 = blockIdx.z % (unsigned)rs.n1; ix.i0 = blockIdx.z / (unsigned)rs.n1;
+        for (unsigned row = (unsigned)row_begin + wave * rpw + sub; row < (unsigned)row_end; row += WPB * rpw) {
+            ix.i2 = row / (unsigned)rs.n3; ix.i3 = row - ix.i2 * (unsigned)rs.n3;
             col_process<KIND>(rs, a, ix, e0, nv, fscale, acc);
         }
     }
@@ -226,9 +226,10 @@ __global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, Vie
     const int lane = threadIdx.x & 63;
     const long nwaves = (long)gridDim.x * WPB;
     for (long g = (long)blockIdx.x * WPB + (threadIdx.x >> 6); g < ngroups; g += nwaves) {
-        long i2 = g % rs.n2; long r = g / rs.n2;
-        long i1 = r % rs.n1; long i0 = r / rs.n1;
-        long base = i0 * d.s0 + i1 * d.s1 + i2 * d.s2;
+        unsigned gg = (unsigned)g;
+        unsigned r = gg / (unsigned)rs.n2; unsigned i2 = gg - r * (unsigned)rs.n2;
+        unsigned i0 = r / (unsigned)rs.n1; unsigned i1 = r - i0 * (unsigned)rs.n1;
+        long base = (long)i0 * d.s0 + (long)i1 * d.s1 + (long)i2 * d.s2;
         float s = 0.f;
         for (int i3 = 0; i3 < rs.n3; ++i3) {
             long ob = base + (long)i3 * d.s3;
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, Vie
             }
         }
         s = wave_sum(s);
-        if (lane == 0) out.p[i0 * out.s0 + i1 * out.s1 + i2 * out.s2] = (half_t)s;
+        if (lane == 0) out.p[(long)i0 * out.s0 + (long)i1 * out.s1 + (long)i2 * out.s2] = (half_t)s;
     }
 }
 

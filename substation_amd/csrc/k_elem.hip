@@ -1,7 +1,7 @@
 // Elementwise operators: bias + activation + dropout (forward), and the plain
 // add used for the attention input biases and the encoder-input gradient.
 // Counterparts: pytorch_module/block_bad.cuh:28-145, block_aib.cuh:17-155,
-// block_bei.cuh:12-106.  Each lane moves one 128-bit pack per tensor per step.
+// block_bei.cuh:12-106.  Each lane moves 128-bit packs, two per tensor per step.
 #include "sub_ops.hpp"
 
 namespace sub {
@@ -9,6 +9,7 @@ namespace sub {
 namespace {
 
 constexpr int BLOCK = 256;
+constexpr int UNROLL = 2;
 
 __device__ __forceinline__ float gelu_fwd(float x) {
     const float c = 0.7978845608028654f;
@@ -17,71 +18,122 @@ __device__ __forceinline__ float gelu_fwd(float x) {
     return 0.5f * x * (1.0f + t);
 }
 
+struct Chunk {
+    unsigned row;
+    int e0, nv;
+    RowIdx ix;
+};
+
+__device__ __forceinline__ Chunk chunk_of(const RowSpace& rs, unsigned idx, unsigned nchunks, unsigned cpr) {
+    Chunk c;
+    const bool live = idx < nchunks;
+    unsigned id = live ? idx : 0;
+    c.row = id / cpr;
+    c.e0 = (int)(id - c.row * cpr) * 8;
+    int nv = rs.R - c.e0;
+    c.nv = live ? (nv > 8 ? 8 : nv) : 0;
+    c.ix = row_index(rs, c.row);
+    return c;
+}
+
+template <bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, View lin, View mask,
-                                               View out, int act, PhiloxKey key, long nchunks, int cpr) {
-    const long stride = (long)gridDim.x * BLOCK;
-    for (long idx = (long)blockIdx.x * BLOCK + threadIdx.x; idx < nchunks; idx += stride) {
-        long row = idx / cpr;
-        int e0 = (int)(idx - row * cpr) * 8;
-        int nv = rs.R - e0; nv = nv > 8 ? 8 : nv;
-        RowIdx ix = row_index(rs, row);
-        F8 fi = load8(in, view_offset(in, ix), e0, nv);
-        F8 fb = load8(bias, 0, e0, nv);
-        uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0);
-        h8 lh, oh;
+                                               View out, int act, PhiloxKey key, unsigned nchunks,
+                                               unsigned cpr) {
+    const unsigned stride = gridDim.x * BLOCK;
+    for (unsigned base = blockIdx.x * BLOCK + threadIdx.x; base < nchunks; base += stride * UNROLL) {
+        Chunk c[UNROLL];
+        F8 fi[UNROLL], fb[UNROLL];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            lh[i] = (half_t)(fi.v[i] + fb.v[i]);
-            float l = (float)lh[i];
-            float a = act == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
-            oh[i] = ((bits >> i) & 1u) ? (half_t)a : (half_t)0.0f;
+        for (int u = 0; u < UNROLL; ++u) {
+            c[u] = chunk_of(rs, base + u * stride, nchunks, cpr);
+            fi[u] = ld8<FAST>(in, view_offset(in, c[u].ix), c[u].e0, c[u].nv);
+            fb[u] = ld8<FAST>(bias, 0, c[u].e0, c[u].nv);
         }
-        store8h(lin, view_offset(lin, ix), e0, nv, lh);
-        store8h(mask, view_offset(mask, ix), e0, nv, mask_h8(bits));
-        store8h(out, view_offset(out, ix), e0, nv, oh);
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (c[u].nv == 0) continue;
+            uint32_t bits = keep_bits8(key, (uint64_t)c[u].row * (uint64_t)rs.R + (uint64_t)c[u].e0);
+            h8 lh, oh;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) lh[i] = (half_t)(fi[u].v[i] + fb[u].v[i]);
+            lh = pin(lh);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float l = (float)lh[i];
+                float a = act == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
+                oh[i] = ((bits >> i) & 1u) ? (half_t)a : (half_t)0.0f;
+            }
+            st8h<FAST>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
+            st8h<FAST>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
+            st8h<FAST>(out, view_offset(out, c[u].ix), c[u].e0, c[u].nv, oh);
+        }
     }
 }
 
-__global__ __launch_bounds__(BLOCK) void k_add(RowSpace rs, View a, View b, View out, long nchunks,
-                                               int cpr) {
-    const long stride = (long)gridDim.x * BLOCK;
-    for (long idx = (long)blockIdx.x * BLOCK + threadIdx.x; idx < nchunks; idx += stride) {
-        long row = idx / cpr;
-        int e0 = (int)(idx - row * cpr) * 8;
-        int nv = rs.R - e0; nv = nv > 8 ? 8 : nv;
-        RowIdx ix = row_index(rs, row);
-        F8 fa = load8(a, view_offset(a, ix), e0, nv);
-        F8 fb = load8(b, view_offset(b, ix), e0, nv);
-        F8 o;
+template <bool FAST>
+__global__ __launch_bounds__(BLOCK) void k_add(RowSpace rs, View a, View b, View out, unsigned nchunks,
+                                               unsigned cpr) {
+    const unsigned stride = gridDim.x * BLOCK;
+    for (unsigned base = blockIdx.x * BLOCK + threadIdx.x; base < nchunks; base += stride * UNROLL) {
+        Chunk c[UNROLL];
+        F8 fa[UNROLL], fb[UNROLL];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o.v[i] = fa.v[i] + fb.v[i];
-        store8(out, view_offset(out, ix), e0, nv, o);
+        for (int u = 0; u < UNROLL; ++u) {
+            c[u] = chunk_of(rs, base + u * stride, nchunks, cpr);
+            fa[u] = ld8<FAST>(a, view_offset(a, c[u].ix), c[u].e0, c[u].nv);
+            // b may be a broadcast along the row (stride 0): generic load
+            fb[u] = b.vec ? ld8<FAST>(b, view_offset(b, c[u].ix), c[u].e0, c[u].nv)
+                          : load8(b, view_offset(b, c[u].ix), c[u].e0, c[u].nv);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            if (c[u].nv == 0) continue;
+            h8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = (half_t)(fa[u].v[i] + fb[u].v[i]);
+            st8h<FAST>(out, view_offset(out, c[u].ix), c[u].e0, c[u].nv, o);
+        }
     }
 }
 
 inline int elem_grid(long nchunks) {
-    long blocks = (nchunks + BLOCK - 1) / BLOCK;
+    long blocks = (nchunks + (long)BLOCK * UNROLL - 1) / ((long)BLOCK * UNROLL);
     const long cap = 256L * 32;
     return (int)(blocks < cap ? (blocks > 0 ? blocks : 1) : cap);
+}
+
+inline unsigned check_chunks(long nchunks, const char* what) {
+    if (nchunks >= (1L << 31)) fail(std::string(what) + ": tensor too large");
+    return (unsigned)nchunks;
 }
 
 }  // namespace
 
 void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, View out, int act,
                 PhiloxKey key, hipStream_t st) {
-    int cpr = (rs.R + 7) / 8;
-    long nchunks = rs.rows() * cpr;
+    unsigned cpr = (unsigned)((rs.R + 7) / 8);
+    unsigned nchunks = check_chunks(rs.rows() * cpr, "bias-activation-dropout");
     if (nchunks == 0) return;
-    hipLaunchKernelGGL(k_bad, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin, mask,
-                       out, act, key, nchunks, cpr);
+    const bool fast = in.vec && bias.vec && lin.vec && mask.vec && out.vec;
+    if (fast)
+        hipLaunchKernelGGL(k_bad<true>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
+                           mask, out, act, key, nchunks, cpr);
+    else
+        hipLaunchKernelGGL(k_bad<false>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
+                           mask, out, act, key, nchunks, cpr);
     check_launch("bias-activation-dropout");
 }
 
 void launch_add(const RowSpace& rs, View a, View b, View out, hipStream_t st) {
-    int cpr = (rs.R + 7) / 8;
-    long nchunks = rs.rows() * cpr;
+    unsigned cpr = (unsigned)((rs.R + 7) / 8);
+    unsigned nchunks = check_chunks(rs.rows() * cpr, "add");
     if (nchunks == 0) return;
-    hipLaunchKernelGGL(k_add, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, a, b, out, nchunks, cpr);
+    const bool fast = a.vec && out.vec;
+    if (fast)
+        hipLaunchKernelGGL(k_add<true>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, a, b, out, nchunks, cpr);
+    else
+        hipLaunchKernelGGL(k_add<false>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, a, b, out, nchunks, cpr);
     check_launch("add");
 }
 

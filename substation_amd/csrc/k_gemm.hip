@@ -405,9 +405,10 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     return ok ? 1 : 0;
 }
 
-// Block tile for a problem: 22 = 128x128, 42 = 256x128, 44 = 256x256.
+// Block tile for a problem: 22 = 128x128, 42 = 256x128, 21 = 128x64.
 int pick_tile(const GemmArgs& a, long batch) {
-    (void)a; (void)batch;
+    (void)batch;
+    if (a.N <= 64) return 21;      // head-size wide outputs of the attention products
     return 22;
 }
 
@@ -448,8 +449,8 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
     if (kind == 1) {
         static const int force = [] { const char* e = getenv("SUB_GEMM_TILE"); return e ? atoi(e) : 0; }();
         int tile = force ? force : pick_tile(c.a, batch);
-        if (tile == 44) launch_mfma<4, 4>(c.a, akc, bkc, batch, st);
-        else if (tile == 42) launch_mfma<4, 2>(c.a, akc, bkc, batch, st);
+        if (tile == 42) launch_mfma<4, 2>(c.a, akc, bkc, batch, st);
+        else if (tile == 21) launch_mfma<2, 1>(c.a, akc, bkc, batch, st);
         else launch_mfma<2, 2>(c.a, akc, bkc, batch, st);
     } else {
         long total = batch * (long)c.a.M * c.a.N;

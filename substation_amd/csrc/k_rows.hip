@@ -1,7 +1,8 @@
 // Row operators: softmax(+scale+dropout), softmax backward, bias+dropout+
 // residual+LayerNorm, LayerNorm backward(+dropout backward).
 // One wave64 per row, the whole row in registers (single global read), fp32 math,
-// 128-bit accesses where the row dimension is contiguous.
+// 128-bit accesses where the row dimension is contiguous.  Short rows are
+// processed several per wave at once so that enough loads are in flight.
 // Counterparts: pytorch_module/block_softmax.cuh:12-188, block_bs.cuh:13-156,
 // block_bdrln.cuh:17-352, block_blnrd.cuh:14-259.
 #include "sub_ops.hpp"
@@ -19,213 +20,272 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
     return n < 0 ? 0 : (n > 8 ? 8 : n);
 }
 
-template <int VPL>
+// VPL: 8-packs per lane (row length <= 512*VPL).  RPW: rows per wave per step.
+// FAST: all views vectorisable (see ld8).
+template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
-                                                   View drop, float scale, PhiloxKey key, long nrows) {
+                                                   View drop, float scale, PhiloxKey key, unsigned nrows) {
     const int lane = threadIdx.x & 63;
-    const long nwaves = (long)gridDim.x * WPB;
-    for (long row = (long)blockIdx.x * WPB + (threadIdx.x >> 6); row < nrows; row += nwaves) {
-        RowIdx ix = row_index(rs, row);
-        const long ob = view_offset(beta, ix);
-        float x[VPL][8];
-        float m = -INFINITY;
+    const unsigned step = gridDim.x * WPB * RPW;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+        float x[RPW][VPL][8];
+        RowIdx ix[RPW];
+        float m[RPW], s[RPW];
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            F8 f = load8(beta, ob, e0, nv, -INFINITY);
+        for (int r = 0; r < RPW; ++r) {
+            const bool live = row0 + r < nrows;
+            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const long ob = view_offset(beta, ix[r]);
+            m[r] = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                x[c][i] = f.v[i] * scale;
-                m = fmaxf(m, x[c][i]);
-            }
-        }
-        m = wave_max(m);
-        float s = 0.f;
-#pragma unroll
-        for (int c = 0; c < VPL; ++c)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                x[c][i] = __builtin_amdgcn_exp2f((x[c][i] - m) * LOG2E);
-                s += x[c][i];
-            }
-        s = wave_sum(s);
-        const float inv = 1.0f / s;
-        const long oa = view_offset(alpha, ix), om = view_offset(mask, ix), od = view_offset(drop, ix);
-#pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            if (nv > 0) {
-                h8 a, d;
-                uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0);
-                h8 mk = mask_h8(bits);
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = live ? nvalid_at(rs.R, e0) : 0;
+                F8 f = ld8<FAST>(beta, ob, e0, nv, -INFINITY);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    a[i] = (half_t)(x[c][i] * inv);
-                    d[i] = ((bits >> i) & 1u) ? a[i] : (half_t)0.0f;
+                    x[r][c][i] = f.v[i] * scale;
+                    m[r] = fmaxf(m[r], x[r][c][i]);
                 }
-                store8h(alpha, oa, e0, nv, a);
-                store8h(mask, om, e0, nv, mk);
-                store8h(drop, od, e0, nv, d);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) m[r] = wave_max(m[r]);
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            s[r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VPL; ++c)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    x[r][c][i] = __builtin_amdgcn_exp2f((x[r][c][i] - m[r]) * LOG2E);
+                    s[r] += x[r][c][i];
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) s[r] = wave_sum(s[r]);
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (row0 + r >= nrows) continue;
+            const float inv = 1.0f / s[r];
+            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = nvalid_at(rs.R, e0);
+                if (nv > 0) {
+                    h8 a, d;
+                    uint32_t bits = keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a[i] = (half_t)(x[r][c][i] * inv);
+                    a = pin(a);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) d[i] = ((bits >> i) & 1u) ? a[i] : (half_t)0.0f;
+                    st8h<FAST>(alpha, oa, e0, nv, a);
+                    st8h<FAST>(mask, om, e0, nv, mask_h8(bits));
+                    st8h<FAST>(drop, od, e0, nv, d);
+                }
             }
         }
     }
 }
 
-template <int VPL>
+template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask, View ddrop,
-                                              View dbeta, float scale, long nrows) {
+                                              View dbeta, float scale, unsigned nrows) {
     const int lane = threadIdx.x & 63;
-    const long nwaves = (long)gridDim.x * WPB;
-    for (long row = (long)blockIdx.x * WPB + (threadIdx.x >> 6); row < nrows; row += nwaves) {
-        RowIdx ix = row_index(rs, row);
-        const long oa = view_offset(alpha, ix), om = view_offset(mask, ix), od = view_offset(ddrop, ix);
-        float a[VPL][8], g[VPL][8];
-        float s = 0.f;
+    const unsigned step = gridDim.x * WPB * RPW;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+        float a[RPW][VPL][8], g[RPW][VPL][8];
+        RowIdx ix[RPW];
+        float s[RPW];
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            F8 fa = load8(alpha, oa, e0, nv), fm = load8(mask, om, e0, nv), fd = load8(ddrop, od, e0, nv);
+        for (int r = 0; r < RPW; ++r) {
+            const bool live = row0 + r < nrows;
+            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(ddrop, ix[r]);
+            s[r] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                a[c][i] = fa.v[i];
-                g[c][i] = fm.v[i] * fd.v[i];
-                s += a[c][i] * g[c][i];
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = live ? nvalid_at(rs.R, e0) : 0;
+                F8 fa = ld8<FAST>(alpha, oa, e0, nv), fm = ld8<FAST>(mask, om, e0, nv), fd = ld8<FAST>(ddrop, od, e0, nv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    a[r][c][i] = fa.v[i];
+                    g[r][c][i] = fm.v[i] * fd.v[i];
+                    s[r] += a[r][c][i] * g[r][c][i];
+                }
             }
         }
-        s = wave_sum(s);
-        const long oo = view_offset(dbeta, ix);
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            if (nv > 0) {
-                F8 o;
+        for (int r = 0; r < RPW; ++r) s[r] = wave_sum(s[r]);
 #pragma unroll
-                for (int i = 0; i < 8; ++i) o.v[i] = scale * a[c][i] * (g[c][i] - s);
-                store8(dbeta, oo, e0, nv, o);
+        for (int r = 0; r < RPW; ++r) {
+            if (row0 + r >= nrows) continue;
+            const long oo = view_offset(dbeta, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = nvalid_at(rs.R, e0);
+                if (nv > 0) {
+                    h8 o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) o[i] = (half_t)(scale * a[r][c][i] * (g[r][c][i] - s[r]));
+                    st8h<FAST>(dbeta, oo, e0, nv, o);
+                }
             }
         }
     }
 }
 
-template <int VPL>
+template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resid, View lin_bias,
                                                  View scale, View bias, View lin, View mask,
                                                  View diff, View normed, View out, View istd,
-                                                 PhiloxKey key, float eps, long nrows) {
+                                                 PhiloxKey key, float eps, unsigned nrows) {
     const int lane = threadIdx.x & 63;
-    const long nwaves = (long)gridDim.x * WPB;
+    const unsigned step = gridDim.x * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;
-    for (long row = (long)blockIdx.x * WPB + (threadIdx.x >> 6); row < nrows; row += nwaves) {
-        RowIdx ix = row_index(rs, row);
-        const long oi = view_offset(in, ix), orr = view_offset(resid, ix);
-        const long ol = view_offset(lin, ix), om = view_offset(mask, ix);
-        float r[VPL][8];
-        float s = 0.f;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+        float x[RPW][VPL][8];
+        uint32_t bits[RPW][VPL];
+        RowIdx ix[RPW];
+        float s[RPW], q[RPW];
+        // pass 1: loads of every row first, then bias/dropout/residual
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            F8 fi = load8(in, oi, e0, nv), fr = load8(resid, orr, e0, nv);
-            F8 fb = load8(lin_bias, 0, e0, nv);
-            uint32_t bits = nv > 0 ? keep_bits8(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0) : 0u;
-            h8 lh;
+        for (int r = 0; r < RPW; ++r) {
+            const bool live = row0 + r < nrows;
+            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const long oi = view_offset(in, ix[r]), orr = view_offset(resid, ix[r]);
+            const long ol = view_offset(lin, ix[r]), om = view_offset(mask, ix[r]);
+            s[r] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                lh[i] = (half_t)(fi.v[i] + fb.v[i]);           // LIN is stored; use its rounded value
-                float kept = ((bits >> i) & 1u) ? (float)lh[i] : 0.f;
-                r[c][i] = i < nv ? kept + fr.v[i] : 0.f;
-                s += r[c][i];
-            }
-            if (nv > 0) {
-                store8h(lin, ol, e0, nv, lh);
-                store8h(mask, om, e0, nv, mask_h8(bits));
-            }
-        }
-        const float mean = wave_sum(s) * invn;
-        float q = 0.f;
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = live ? nvalid_at(rs.R, e0) : 0;
+                F8 fi = ld8<FAST>(in, oi, e0, nv), fr = ld8<FAST>(resid, orr, e0, nv);
+                F8 fb = ld8<FAST>(lin_bias, 0, e0, nv);
+                bits[r][c] = nv > 0 ? keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0) : 0u;
+                h8 lh;
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                r[c][i] = i < nv ? r[c][i] - mean : 0.f;
-                q += r[c][i] * r[c][i];
-            }
-        }
-        const float var = wave_sum(q) * invn;
-        const float is = rsqrtf(var + eps);
-        if (lane == 0) istd.p[view_offset(istd, ix)] = (half_t)is;
-        const long od = view_offset(diff, ix), on = view_offset(normed, ix), oo = view_offset(out, ix);
-#pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            if (nv > 0) {
-                F8 fs = load8(scale, 0, e0, nv), fb = load8(bias, 0, e0, nv);
-                F8 d, n, o;
+                for (int i = 0; i < 8; ++i) lh[i] = (half_t)(fi.v[i] + fb.v[i]);
+                lh = pin(lh);                                      // LIN is stored; use its rounded value
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    d.v[i] = r[c][i];
-                    n.v[i] = r[c][i] * is;
-                    o.v[i] = n.v[i] * fs.v[i] + fb.v[i];
+                    float kept = ((bits[r][c] >> i) & 1u) ? (float)lh[i] : 0.f;
+                    x[r][c][i] = i < nv ? kept + fr.v[i] : 0.f;
+                    s[r] += x[r][c][i];
                 }
-                store8(diff, od, e0, nv, d);
-                store8(normed, on, e0, nv, n);
-                store8(out, oo, e0, nv, o);
+                if (nv > 0) {
+                    st8h<FAST>(lin, ol, e0, nv, lh);
+                    st8h<FAST>(mask, om, e0, nv, mask_h8(bits[r][c]));
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) s[r] = wave_sum(s[r]) * invn;      // mean
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            q[r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = nvalid_at(rs.R, e0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    x[r][c][i] = i < nv ? x[r][c][i] - s[r] : 0.f;
+                    q[r] += x[r][c][i] * x[r][c][i];
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) q[r] = rsqrtf(wave_sum(q[r]) * invn + eps);   // 1/std
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (row0 + r >= nrows) continue;
+            const float is = q[r];
+            if (lane == 0) istd.p[view_offset(istd, ix[r])] = (half_t)is;
+            const long od = view_offset(diff, ix[r]), on = view_offset(normed, ix[r]), oo = view_offset(out, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = nvalid_at(rs.R, e0);
+                if (nv > 0) {
+                    F8 fs = ld8<FAST>(scale, 0, e0, nv), fb = ld8<FAST>(bias, 0, e0, nv);
+                    h8 d, n, o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        float nn = x[r][c][i] * is;
+                        d[i] = (half_t)x[r][c][i];
+                        n[i] = (half_t)nn;
+                        o[i] = (half_t)(nn * fs.v[i] + fb.v[i]);
+                    }
+                    st8h<FAST>(diff, od, e0, nv, d);
+                    st8h<FAST>(normed, on, e0, nv, n);
+                    st8h<FAST>(out, oo, e0, nv, o);
+                }
             }
         }
     }
 }
 
-template <int VPL>
+template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View istd, View diff,
-                                                 View mask, View d_ln_in, View d_drop_in, long nrows) {
+                                                 View mask, View d_ln_in, View d_drop_in, unsigned nrows) {
     const int lane = threadIdx.x & 63;
-    const long nwaves = (long)gridDim.x * WPB;
+    const unsigned step = gridDim.x * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;
-    for (long row = (long)blockIdx.x * WPB + (threadIdx.x >> 6); row < nrows; row += nwaves) {
-        RowIdx ix = row_index(rs, row);
-        const long oo = view_offset(dout, ix), od = view_offset(diff, ix);
-        float g[VPL][8], df[VPL][8];
-        float s1 = 0.f, s2 = 0.f;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+        float g[RPW][VPL][8], df[RPW][VPL][8];
+        h8 mk[RPW][VPL];
+        RowIdx ix[RPW];
+        float s1[RPW], s2[RPW], is[RPW];
 #pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            F8 fg = load8(dout, oo, e0, nv), fd = load8(diff, od, e0, nv);
+        for (int r = 0; r < RPW; ++r) {
+            const bool live = row0 + r < nrows;
+            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const long oo = view_offset(dout, ix[r]), od = view_offset(diff, ix[r]), om = view_offset(mask, ix[r]);
+            is[r] = (float)istd.p[view_offset(istd, ix[r])];
+            s1[r] = 0.f; s2[r] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                g[c][i] = fg.v[i];
-                df[c][i] = fd.v[i];
-                s1 += g[c][i];
-                s2 += g[c][i] * df[c][i];
-            }
-        }
-        s1 = wave_sum(s1);
-        s2 = wave_sum(s2);
-        const float is = (float)istd.p[view_offset(istd, ix)];
-        const float c1 = s1 * is * invn;
-        const float c2 = s2 * is * is * is * invn;
-        const long om = view_offset(mask, ix), o1 = view_offset(d_ln_in, ix), o2 = view_offset(d_drop_in, ix);
-#pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            int e0 = (c * WAVE + lane) * 8;
-            int nv = nvalid_at(rs.R, e0);
-            if (nv > 0) {
-                F8 fm = load8(mask, om, e0, nv);
-                h8 a, b;
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = live ? nvalid_at(rs.R, e0) : 0;
+                F8 fg = ld8<FAST>(dout, oo, e0, nv), fd = ld8<FAST>(diff, od, e0, nv);
+                F8 fm = ld8<FAST>(mask, om, e0, nv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    a[i] = (half_t)(g[c][i] * is - c1 - df[c][i] * c2);
-                    b[i] = fm.v[i] != 0.f ? a[i] : (half_t)0.0f;
+                    g[r][c][i] = fg.v[i];
+                    df[r][c][i] = fd.v[i];
+                    mk[r][c][i] = (half_t)fm.v[i];
+                    s1[r] += g[r][c][i];
+                    s2[r] += g[r][c][i] * df[r][c][i];
                 }
-                store8h(d_ln_in, o1, e0, nv, a);
-                store8h(d_drop_in, o2, e0, nv, b);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) { s1[r] = wave_sum(s1[r]); s2[r] = wave_sum(s2[r]); }
+#pragma unroll
+        for (int r = 0; r < RPW; ++r) {
+            if (row0 + r >= nrows) continue;
+            const float c1 = s1[r] * is[r] * invn;
+            const float c2 = s2[r] * is[r] * is[r] * is[r] * invn;
+            const long o1 = view_offset(d_ln_in, ix[r]), o2 = view_offset(d_drop_in, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = nvalid_at(rs.R, e0);
+                if (nv > 0) {
+                    h8 a, b;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) a[i] = (half_t)(g[r][c][i] * is[r] - c1 - df[r][c][i] * c2);
+                    a = pin(a);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) b[i] = mk[r][c][i] != (half_t)0.0f ? a[i] : (half_t)0.0f;
+                    st8h<FAST>(d_ln_in, o1, e0, nv, a);
+                    st8h<FAST>(d_drop_in, o2, e0, nv, b);
+                }
             }
         }
     }
@@ -240,61 +300,83 @@ inline int pick_vpl(int R, const char* what) {
     fail(std::string(what) + ": rows longer than 4096 elements are not supported");
 }
 
-inline int row_grid(long nrows) {
-    long blocks = (nrows + WPB - 1) / WPB;
-    const long cap = 256L * 64;          // 256 CUs, waves beyond this loop
+inline int row_grid(long nrows, int rpw) {
+    long blocks = (nrows + (long)WPB * rpw - 1) / ((long)WPB * rpw);
+    const long cap = 256L * 64;          // 256 CUs; waves beyond this loop
     return (int)(blocks < cap ? (blocks > 0 ? blocks : 1) : cap);
+}
+
+inline unsigned check_rows(const RowSpace& rs, const char* what) {
+    long n = rs.rows();
+    if (n >= (1L << 31)) fail(std::string(what) + ": too many rows");
+    return (unsigned)n;
 }
 
 }  // namespace
 
-#define SUB_DISPATCH_VPL(vpl, KERNEL, ...)                                                   \
-    switch (vpl) {                                                                           \
-        case 1: hipLaunchKernelGGL(KERNEL<1>, dim3(grid), dim3(BLOCK), 0, st, __VA_ARGS__); break; \
-        case 2: hipLaunchKernelGGL(KERNEL<2>, dim3(grid), dim3(BLOCK), 0, st, __VA_ARGS__); break; \
-        case 4: hipLaunchKernelGGL(KERNEL<4>, dim3(grid), dim3(BLOCK), 0, st, __VA_ARGS__); break; \
-        default: hipLaunchKernelGGL(KERNEL<8>, dim3(grid), dim3(BLOCK), 0, st, __VA_ARGS__); break; \
-    }
+// Dispatch on (VPL, rows per wave, FAST).  Rows per wave: 4 for rows of up to 512
+// elements, 2 up to 1024, else 1; the generic (strided) path always takes 1.
+#define SUB_ROW_LAUNCH(KERNEL, V, RP, F, ...) \
+    hipLaunchKernelGGL((KERNEL<V, RP, F>), dim3(row_grid(nrows, RP)), dim3(BLOCK), 0, st, __VA_ARGS__)
+#define SUB_ROW_DISPATCH(KERNEL, vpl, fast, ...)                                   \
+    do {                                                                           \
+        if (fast) {                                                                \
+            switch (vpl) {                                                         \
+                case 1: SUB_ROW_LAUNCH(KERNEL, 1, 4, true, __VA_ARGS__); break;    \
+                case 2: SUB_ROW_LAUNCH(KERNEL, 2, 2, true, __VA_ARGS__); break;    \
+                case 4: SUB_ROW_LAUNCH(KERNEL, 4, 1, true, __VA_ARGS__); break;    \
+                default: SUB_ROW_LAUNCH(KERNEL, 8, 1, true, __VA_ARGS__); break;   \
+            }                                                                      \
+        } else {                                                                   \
+            switch (vpl) {                                                         \
+                case 1: SUB_ROW_LAUNCH(KERNEL, 1, 1, false, __VA_ARGS__); break;   \
+                case 2: SUB_ROW_LAUNCH(KERNEL, 2, 1, false, __VA_ARGS__); break;   \
+                case 4: SUB_ROW_LAUNCH(KERNEL, 4, 1, false, __VA_ARGS__); break;   \
+                default: SUB_ROW_LAUNCH(KERNEL, 8, 1, false, __VA_ARGS__); break;  \
+            }                                                                      \
+        }                                                                          \
+    } while (0)
 
 void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, float scale,
                     PhiloxKey key, hipStream_t st) {
-    long nrows = rs.rows();
+    unsigned nrows = check_rows(rs, "softmax");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax");
-    int grid = row_grid(nrows);
-    SUB_DISPATCH_VPL(vpl, k_softmax, rs, beta, alpha, mask, drop, scale, key, nrows);
+    bool fast = beta.vec && alpha.vec && mask.vec && drop.vec;
+    SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, scale, key, nrows);
     check_launch("softmax");
 }
 
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st) {
-    long nrows = rs.rows();
+    unsigned nrows = check_rows(rs, "softmax backward");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax backward");
-    int grid = row_grid(nrows);
-    SUB_DISPATCH_VPL(vpl, k_bs, rs, alpha, mask, ddrop, dbeta, scale, nrows);
+    bool fast = alpha.vec && mask.vec && ddrop.vec && dbeta.vec;
+    SUB_ROW_DISPATCH(k_bs, vpl, fast, rs, alpha, mask, ddrop, dbeta, scale, nrows);
     check_launch("softmax backward");
 }
 
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
                   float eps, hipStream_t st) {
-    long nrows = rs.rows();
+    unsigned nrows = check_rows(rs, "bias-dropout-residual-layernorm");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "bias-dropout-residual-layernorm");
-    int grid = row_grid(nrows);
-    SUB_DISPATCH_VPL(vpl, k_bdrln, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
+    bool fast = in.vec && resid.vec && lin_bias.vec && scale.vec && bias.vec && lin.vec && mask.vec &&
+                diff.vec && normed.vec && out.vec;
+    SUB_ROW_DISPATCH(k_bdrln, vpl, fast, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
                      out, istd, key, eps, nrows);
     check_launch("bias-dropout-residual-layernorm");
 }
 
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
                   View d_drop_in, hipStream_t st) {
-    long nrows = rs.rows();
+    unsigned nrows = check_rows(rs, "layernorm backward");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "layernorm backward");
-    int grid = row_grid(nrows);
-    SUB_DISPATCH_VPL(vpl, k_blnrd, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows);
+    bool fast = dout.vec && diff.vec && mask.vec && d_ln_in.vec && d_drop_in.vec;
+    SUB_ROW_DISPATCH(k_blnrd, vpl, fast, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows);
     check_launch("layernorm backward");
 }
 

@@ -19,9 +19,12 @@ constexpr int WAVE = 64;
 
 // Row space: up to four outer dimensions (canonical order) times a row of R
 // elements.  The canonical element index of (row r, column e) is r*R + e.
+// flat != 0: the three leading outer dims have extent 1 (after the host merged
+// dims that every view strides through uniformly), so row == i3.
 struct RowSpace {
     int n0, n1, n2, n3;
     int R;
+    int flat;
     long rows() const { return (long)n0 * n1 * n2 * n3; }
 };
 
@@ -39,26 +42,23 @@ struct F8 {
     float v[8];
 };
 
-__device__ __forceinline__ long row_offset(const RowSpace& rs, const View& t, long row) {
-    long i3 = row % rs.n3; long r = row / rs.n3;
-    long i2 = r % rs.n2; r /= rs.n2;
-    long i1 = r % rs.n1; long i0 = r / rs.n1;
-    return i0 * t.s0 + i1 * t.s1 + i2 * t.s2 + i3 * t.s3;
-}
-
 // Outer indices of a row, computed once and reused for every view.
 struct RowIdx {
-    long i0, i1, i2, i3;
+    unsigned i0, i1, i2, i3;
 };
-__device__ __forceinline__ RowIdx row_index(const RowSpace& rs, long row) {
+__device__ __forceinline__ RowIdx row_index(const RowSpace& rs, unsigned row) {
     RowIdx x;
-    x.i3 = row % rs.n3; long r = row / rs.n3;
-    x.i2 = r % rs.n2; r /= rs.n2;
-    x.i1 = r % rs.n1; x.i0 = r / rs.n1;
+    if (rs.flat) {
+        x.i0 = x.i1 = x.i2 = 0; x.i3 = row;
+    } else {
+        unsigned r = row / (unsigned)rs.n3; x.i3 = row - r * (unsigned)rs.n3;
+        unsigned q = r / (unsigned)rs.n2; x.i2 = r - q * (unsigned)rs.n2;
+        x.i0 = q / (unsigned)rs.n1; x.i1 = q - x.i0 * (unsigned)rs.n1;
+    }
     return x;
 }
 __device__ __forceinline__ long view_offset(const View& t, const RowIdx& x) {
-    return x.i0 * t.s0 + x.i1 * t.s1 + x.i2 * t.s2 + x.i3 * t.s3;
+    return (long)x.i0 * t.s0 + (long)x.i1 * t.s1 + (long)x.i2 * t.s2 + (long)x.i3 * t.s3;
 }
 
 // Load 8 row elements e0 .. e0+7 (nvalid of them inside the row) as fp32.
@@ -102,6 +102,34 @@ __device__ __forceinline__ void store8(const View& t, long base, int e0, int nva
     store8h(t, base, e0, nvalid, to_h8(x));
 }
 
+// FAST variants: every view is vectorisable and rows are whole 8-packs, so a
+// chunk is either entirely inside the row (nvalid == 8) or entirely outside.
+template <bool FAST>
+__device__ __forceinline__ F8 ld8(const View& t, long base, int e0, int nvalid, float fill = 0.f) {
+    if (FAST) {
+        F8 r;
+        if (nvalid) {
+            h8 v = *reinterpret_cast<const h8*>(t.p + base + e0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r.v[i] = (float)v[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) r.v[i] = fill;
+        }
+        return r;
+    }
+    return load8(t, base, e0, nvalid, fill);
+}
+
+template <bool FAST>
+__device__ __forceinline__ void st8h(const View& t, long base, int e0, int nvalid, h8 v) {
+    if (FAST) {
+        if (nvalid) *reinterpret_cast<h8*>(t.p + base + e0) = v;
+    } else {
+        store8h(t, base, e0, nvalid, v);
+    }
+}
+
 // ---- wave64 reductions ------------------------------------------------------
 // Two quad permutes, two row mirrors (DPP), then the four row totals are read
 // with v_readlane and combined; the result is uniform across the wave.
@@ -135,6 +163,16 @@ __device__ __forceinline__ float wave_max(float x) {
     float c = __int_as_float(__builtin_amdgcn_readlane(xi, 32));
     float d = __int_as_float(__builtin_amdgcn_readlane(xi, 48));
     return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+
+// Makes a rounded fp16 pack opaque to the optimiser, so that a second output
+// derived from it (value * {0,1} mask) is bit-identical to it rather than
+// recomputed through a differently rounded (fused) conversion.
+__device__ __forceinline__ h8 pin(h8 v) {
+    typedef int i4 __attribute__((ext_vector_type(4)));
+    i4 t = __builtin_bit_cast(i4, v);
+    asm volatile("" : "+v"(t));
+    return __builtin_bit_cast(h8, t);
 }
 
 // {0,1} mask pack from keep bits

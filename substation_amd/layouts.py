@@ -69,12 +69,12 @@ def mi355x_layouts():
     return _make(
         'BJI', 'BJI',
         'WKQV:QHPI BKQV:QHP WO:IHP BO:I S1:I B1:I LINB1:U LINW1:UI S2:I B2:I LINB2:I LINW2:IU',
-        'KKQQVV:QBJHP WKKWQQWVV:QBJHP BETA:BHJK ALPHA:BHJK ATTN_DROP_MASK:BHJK ATTN_DROP:BHJK '
+        'KKQQVV:QBJHP WKKWQQWVV:QBJHP BETA:HBJK ALPHA:HBJK ATTN_DROP_MASK:HBJK ATTN_DROP:HBJK '
         'GAMMA:BJHP ATT:BJI DROP1MASK:BJI SB1:BJI SB1_LINW1:BJU DROP2:BJU LIN1:BJU DROP2_LINW2:BJI '
         'LIN2:BJI LN2:BJI LN2STD:BJ LN2DIFF:BJI DROP2MASK:BJU DROP3MASK:BJI LN1:BJI LN1STD:BJ '
         'LN1DIFF:BJI',
         'DLN2:BJI DRESID2:BJI DLIN2:BJI DDROP2:BJU DLIN1:BJU DLIN1_LINW1:BJI DLN1:BJI DRESID1:BJI '
-        'DATT:BJI DXATT:BJI DGAMMA:BJHP DATTN_DROP:BHJK DBETA:BHJK DKKQQVV:QBJHP')
+        'DATT:BJI DXATT:BJI DGAMMA:BJHP DATTN_DROP:HBJK DBETA:HBJK DKKQQVV:QBJHP')
 
 
 def reference_layouts(name):
