@@ -109,6 +109,15 @@ int sub_set_stream(void* handle, void* hip_stream);  /* hipStream_t */
 int sub_set_rng(void* handle, uint64_t seed, uint32_t step);
 const char* sub_last_error(void);
 
+/* Options.  SUB_OPT_FUSE_EPILOGUES (default 1): add BKQV in the epilogue of the
+ * QKV projection and DRESID1 in the epilogue of the input-gradient projection,
+ * where the layouts allow it.  The separate operators aib (block_aib.cuh) and
+ * bei (block_bei.cuh) are then not launched and the intermediates WKKWQQWVV and
+ * DXATT, which only they consume, are left unwritten.  Set to 0 to materialise
+ * every intermediate exactly as pytorch_module/encoder.cu:87-299 does. */
+#define SUB_OPT_FUSE_EPILOGUES 1
+int sub_set_option(void* handle, int option, int value);
+
 /* Array forms of the two calls above: ptrs holds the same pointers in the same
  * order, without the handle (n must be 37 resp. 64). */
 int sub_encoder_forward(void* handle, void* const* ptrs, int n);

@@ -13,6 +13,7 @@ LIB_PATH = os.path.join(HERE, 'lib', 'libsubstation_amd.so')
 N_PARAMS, N_FWD, N_BWD = 12, 23, 14
 ABI_VERSION = 1
 ACTIVATIONS = {'relu': 0, 'gelu': 1}
+OPT_FUSE_EPILOGUES = 1
 
 
 class SubConfig(ctypes.Structure):
@@ -48,6 +49,7 @@ SIGNATURES = {
     'sub_set_stream': (_I, [_VP, _VP]),
     'sub_set_rng': (_I, [_VP, _U64, _U32]),
     'sub_last_error': (_CP, []),
+    'sub_set_option': (_I, [_VP, _I, _I]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_profile_enable': (_I, [_VP, _I]),
@@ -157,6 +159,9 @@ class Handle:
 
     def set_rng(self, seed, step=0):
         check(self.lib.sub_set_rng(self.ptr, seed, step), 'sub_set_rng')
+
+    def set_option(self, option, value):
+        check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')
 
     def profile_enable(self, on=True):
         check(self.lib.sub_profile_enable(self.ptr, 1 if on else 0), 'sub_profile_enable')

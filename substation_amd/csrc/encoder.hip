@@ -143,9 +143,14 @@ View vector_view(const void* p, int R) {
 struct GemmPlan {
     GemmShape shape;
     float alpha = 1.f;
+    bool ok = false;                  // fused variants only: the plan is usable
+    int64_t sM = 0, sN = 0, sb[3] = {0, 0, 0};   // addend strides
 };
 
-enum G { G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
+// G_QKV_BIAS: QKV projection writing KKQQVV directly with BKQV added in the
+// epilogue (replaces QKV-fused + aib).  G_DXQKV_RESID: input-gradient projection
+// writing DX directly with DRESID1 added (replaces dXQKV-fused + bei).
+enum G { G_QKV_BIAS, G_DXQKV_RESID, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
          G_DWOUT, G_DXOUT, G_DX1GAMMA, G_DX2GAMMA, G_DX1QKT, G_DX2QKT, G_DXQKV, G_DWQKV, G_COUNT };
 
 struct ProfEntry { const char* name; hipEvent_t a, b; };
@@ -166,6 +171,7 @@ struct Handle {
     float* ws = nullptr;
     size_t ws_floats = 0;
     bool profiling = false;
+    bool fuse_epilogues = true;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -300,6 +306,25 @@ void configure(Handle& h, const sub_config* c) {
     plan_gemm(h, G_DXQKV, h.lp[WKQV], h.lb[DKKQQVV], h.lb[DXATT], 1.f, "dXQKV-fused");
     plan_gemm(h, G_DWQKV, h.lX, h.lb[DKKQQVV], h.lp[WKQV], 1.f, "dWQKV-fused");
 
+    // Optional epilogue fusions; they need the addend to be N-contiguous like the
+    // output after the kernel's operand swap, which gemm_kernel_kind checks.
+    auto plan_fused = [&](int id, const Layout& la, const Layout& lb2, const Layout& lc, const Layout& lt) {
+        GemmPlan& p = h.gemm[id];
+        p.ok = false;
+        try {
+            p.shape = classify_einsum(la, lb2, lc);
+        } catch (const Error&) {
+            return;
+        }
+        p.alpha = 1.f;
+        if (!addend_strides(p.shape, lt, lc, p.sM, p.sN, p.sb)) return;
+        GemmEpilogue ep; ep.bias = (const half_t*)16; ep.sbM = p.sM; ep.sbN = p.sN;
+        for (int i = 0; i < 3; ++i) ep.sbb[i] = p.sb[i];
+        p.ok = gemm_kernel_kind(p.shape, (const void*)16, (const void*)16, (const void*)16, ep) == 1;
+    };
+    plan_fused(G_QKV_BIAS, h.lX, h.lp[WKQV], h.lf[KKQQVV], h.lp[BKQV]);
+    plan_fused(G_DXQKV_RESID, h.lp[WKQV], h.lb[DKKQQVV], h.lX, h.lb[DRESID1]);
+
     // The fp32 scratch of the column reductions is allocated by the first
     // operator that needs it, so that configuring needs no GPU.
     h.configured = true;
@@ -308,11 +333,19 @@ void configure(Handle& h, const sub_config* c) {
 // ---------------------------------------------------------------------------
 // Operators on a handle
 // ---------------------------------------------------------------------------
-void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const char* name) {
+void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const char* name,
+              const void* addend = nullptr) {
     ProfScope ps(h, name);
+    const GemmPlan& p = h.gemm[id];
     GemmEpilogue ep;
-    launch_gemm(h.gemm[id].shape, (const half_t*)A, (const half_t*)B, (half_t*)C, h.gemm[id].alpha, ep, h.stream);
+    if (addend) {
+        ep.bias = (const half_t*)addend; ep.sbM = p.sM; ep.sbN = p.sN;
+        for (int i = 0; i < 3; ++i) ep.sbb[i] = p.sb[i];
+    }
+    launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream);
 }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 void op_softmax(Handle& h, const void* beta, const Layout& lb, void* alpha, const Layout& la,
                 void* mask, const Layout& lm, void* drop, const Layout& ld, float scale, float p,
@@ -475,8 +508,11 @@ void forward(Handle& h, const FwdPtrs& t) {
     if (!h.configured) fail("encoder_forward: handle is not configured");
     h.prof_used = 0;
     void* const* W = t.W; void* const* F = t.F;
-    run_gemm(h, G_QKV, t.X, W[WKQV], F[WKKWQQWVV], "QKV-fused");
-    {
+    if (h.fuse_epilogues && h.gemm[G_QKV_BIAS].ok && aligned16(W[BKQV]) && aligned16(F[KKQQVV])) {
+        // projection + bias in one pass; WKKWQQWVV (the pre-bias copy) is not written
+        run_gemm(h, G_QKV_BIAS, t.X, W[WKQV], F[KKQQVV], "QKV-fused", W[BKQV]);
+    } else {
+        run_gemm(h, G_QKV, t.X, W[WKQV], F[WKKWQQWVV], "QKV-fused");
         ProfScope ps(h, "aib");
         op_aib(h, F[WKKWQQWVV], h.lf[WKKWQQWVV], W[BKQV], h.lp[BKQV], F[KKQQVV], h.lf[KKQQVV]);
     }
@@ -560,13 +596,20 @@ void backward(Handle& h, const BwdPtrs& t) {
     }
     run_gemm(h, G_DX1QKT, KK, D[DBETA], DQQ, "dX1QKT");
     run_gemm(h, G_DX2QKT, QQ, D[DBETA], DKK, "dX2QKT");
-    run_gemm(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused");
+    const bool fuse_dx = h.fuse_epilogues && h.gemm[G_DXQKV_RESID].ok && aligned16(D[DRESID1]) &&
+                         aligned16(t.DX);
+    if (fuse_dx) {
+        // DX = WKQV.DKKQQVV + DRESID1 in one pass; DXATT is not written
+        run_gemm(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1]);
+    } else {
+        run_gemm(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused");
+    }
     run_gemm(h, G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused");
     {
         ProfScope ps(h, "baib");
         op_baib(h, D[DKKQQVV], h.lb[DKKQQVV], DW[BKQV], h.lp[BKQV]);
     }
-    {
+    if (!fuse_dx) {
         ProfScope ps(h, "bei");
         op_bei(h, D[DXATT], h.lb[DXATT], D[DRESID1], h.lb[DRESID1], t.DX, h.lX);
     }
@@ -714,6 +757,14 @@ int encoder_backward(void* handle, void* DY,
                  f0, f1, f2, f3, f4, f5, f6, f7, f8, f9, f10, f11, f12, f13, f14, f15, f16, f17,
                  f18, f19, f20, f21, f22, X, DX};
     return sub_encoder_backward(handle, p, (int)(sizeof(p) / sizeof(p[0])));
+}
+
+int sub_set_option(void* handle, int option, int value) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
+        else fail("sub_set_option: unknown option");
+    });
 }
 
 int sub_profile_enable(void* handle, int on) {

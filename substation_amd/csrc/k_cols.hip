@@ -38,65 +38,67 @@ __device__ __forceinline__ float gelu_grad(float x) {
     return 0.5f * t + (1.5f * 0.044715f * c * x3 + 0.5f * c * x) * sech2 + 0.5f;
 }
 
+template <int KIND> struct ColIn;      // which views are read: count and indices into ColArgs::v
+template <> struct ColIn<COL_BSB> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; };
+template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; };
+template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; };
+template <> struct ColIn<COL_BAOB> { static constexpr int N = 1; static constexpr int idx[4] = {0, 0, 0, 0}; };
+
+// One 8-pack of one row: elementwise output (stored to v[3]) and the running sums.
 template <int KIND>
-__device__ __forceinline__ void col_process(const RowSpace& rs, const ColArgs& a, const RowIdx& ix,
-                                            int e0, int nv, const F8& fscale,
+__device__ __forceinline__ void col_compute(const ColArgs& a, const RowIdx& ix, int e0, int nv,
+                                            const F8 (&in)[4], const F8& fscale,
                                             float (&acc)[ColTraits<KIND>::NS][8]) {
     if (KIND == COL_BSB) {
-        // v0 IN (normed), v1 DOUT, v3 DIN
-        F8 fi = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
-        F8 fd = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
-        F8 o;
+        // in0 IN (normed), in1 DOUT -> DIN
+        h8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            o.v[i] = fd.v[i] * fscale.v[i];
-            acc[0][i] += fd.v[i] * fi.v[i];
-            acc[1][i] += fd.v[i];
+            o[i] = (half_t)(in[1].v[i] * fscale.v[i]);
+            acc[0][i] += in[1].v[i] * in[0].v[i];
+            acc[1][i] += in[1].v[i];
         }
-        store8(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
+        store8h(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
     } else if (KIND == COL_EBSB) {
-        // v0 IN, v1 DOUT1, v2 DOUT2, v4 DLINEAR, v3 DIN
-        F8 fi = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
-        F8 f1 = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
-        F8 f2 = load8(a.v[2], view_offset(a.v[2], ix), e0, nv);
-        F8 fl = load8(a.v[4], view_offset(a.v[4], ix), e0, nv);
-        F8 o;
+        // in0 IN, in1 DOUT1, in2 DOUT2, in3 DLINEAR -> DIN
+        h8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float d = f1.v[i] + f2.v[i];
-            o.v[i] = d * fscale.v[i];
-            acc[0][i] += d * fi.v[i];
+            float d = in[1].v[i] + in[2].v[i];
+            o[i] = (half_t)(d * fscale.v[i]);
+            acc[0][i] += d * in[0].v[i];
             acc[1][i] += d;
-            acc[2][i] += fl.v[i];
+            acc[2][i] += in[3].v[i];
         }
-        store8(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
+        store8h(a.v[3], view_offset(a.v[3], ix), e0, nv, o);
     } else if (KIND == COL_BDRLB) {
-        // v0 DDROP, v1 MASK, v2 LIN, v3 DLINEAR
-        F8 fd = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
-        F8 fm = load8(a.v[1], view_offset(a.v[1], ix), e0, nv);
-        F8 fl = load8(a.v[2], view_offset(a.v[2], ix), e0, nv);
+        // in0 DDROP, in1 MASK, in2 LIN -> DLINEAR
         h8 oh;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float d = fd.v[i] * fm.v[i];
-            float g = a.act == ACT_GELU ? gelu_grad(fl.v[i]) * d : (fl.v[i] > 0.f ? d : 0.f);
+            float d = in[0].v[i] * in[1].v[i];
+            float g = a.act == ACT_GELU ? gelu_grad(in[2].v[i]) * d : (in[2].v[i] > 0.f ? d : 0.f);
             oh[i] = (half_t)g;
-            acc[0][i] += i < nv ? (float)oh[i] : 0.f;
         }
+        oh = pin(oh);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[0][i] += i < nv ? (float)oh[i] : 0.f;
         store8h(a.v[3], view_offset(a.v[3], ix), e0, nv, oh);
     } else {
-        F8 fd = load8(a.v[0], view_offset(a.v[0], ix), e0, nv);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[0][i] += fd.v[i];
+        for (int i = 0; i < 8; ++i) acc[0][i] += in[0].v[i];
     }
 }
 
 // grid.x = feature strips of lpr*8 features, grid.y = token chunks, grid.z = kept
 // outer index (i0,i1).  The sums run over the two inner outer dims (i2,i3).
-template <int KIND>
+// FAST: every big tensor is vectorisable (128-bit packs kept raw until used).
+template <int KIND, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, float* ws, int lpr_log2,
                                                      long rows_per_block, long nrows) {
     constexpr int NS = ColTraits<KIND>::NS;
+    constexpr int NIN = ColIn<KIND>::N;
+    constexpr int U = FAST ? (NIN >= 3 ? 2 : 4) : 1;   // rows in flight per lane
     __shared__ float red[BLOCK][9];          // +1 pad: conflict-free column reads
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lpr = 1 << lpr_log2, rpw = WAVE >> lpr_log2;
@@ -113,11 +115,42 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
     F8 fscale;
     if (KIND == COL_BSB || KIND == COL_EBSB) fscale = load8(a.v[5], 0, e0, nv);
     if (nv > 0) {
-        RowIdx ix;
-        ix.i1 = blockIdx.z % (unsigned)rs.n1; ix.i0 = blockIdx.z / (unsigned)rs.n1;
-        for (unsigned row = (unsigned)row_begin + wave * rpw + sub; row < (unsigned)row_end; row += WPB * rpw) {
-            ix.i2 = row / (unsigned)rs.n3; ix.i3 = row - ix.i2 * (unsigned)rs.n3;
-            col_process<KIND>(rs, a, ix, e0, nv, fscale, acc);
+        const unsigned n3 = (unsigned)rs.n3, stride = WPB * rpw;
+        const unsigned i1 = blockIdx.z % (unsigned)rs.n1, i0 = blockIdx.z / (unsigned)rs.n1;
+        for (unsigned row = (unsigned)row_begin + wave * rpw + sub; row < (unsigned)row_end; row += stride * U) {
+            RowIdx ix[U];
+            h8 raw[U][NIN];
+            F8 gen[4];
+            int nvu[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                unsigned r = row + u * stride;
+                nvu[u] = r < (unsigned)row_end ? nv : 0;
+                r = nvu[u] ? r : row;
+                ix[u].i0 = i0; ix[u].i1 = i1;
+                ix[u].i2 = r / n3; ix[u].i3 = r - ix[u].i2 * n3;
+#pragma unroll
+                for (int t = 0; t < NIN; ++t) {
+                    const View& v = a.v[ColIn<KIND>::idx[t]];
+                    if (FAST) {
+                        raw[u][t] = (h8)(half_t)0.0f;
+                        if (nvu[u]) raw[u][t] = *reinterpret_cast<const h8*>(v.p + view_offset(v, ix[u]) + e0);
+                    } else {
+                        gen[t] = load8(v, view_offset(v, ix[u]), e0, nvu[u]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (!nvu[u]) continue;
+                if (FAST) {
+#pragma unroll
+                    for (int t = 0; t < NIN; ++t)
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) gen[t].v[i] = (float)raw[u][t][i];
+                }
+                col_compute<KIND>(a, ix[u], e0, nvu[u], gen, fscale, acc);
+            }
         }
     }
     const int ntc = gridDim.y;
@@ -189,10 +222,10 @@ inline ColPlan col_plan(const RowSpace& rs) {
     p.nstrips = (chunks + lpr - 1) / lpr;
     long nrows = (long)rs.n2 * rs.n3;
     int rows_per_iter = WPB * (WAVE / lpr);
-    // aim for ~1024 blocks in total, at least two row-iterations per block
-    long want_tc = 1024 / (p.nstrips * nbatch); if (want_tc < 1) want_tc = 1;
+    // aim for ~768 blocks in total, at least one 4-row-deep iteration per wave
+    long want_tc = 768 / (p.nstrips * nbatch); if (want_tc < 1) want_tc = 1;
     long rpb = (nrows + want_tc - 1) / want_tc;
-    if (rpb < 2L * rows_per_iter) rpb = 2L * rows_per_iter;
+    if (rpb < 4L * rows_per_iter) rpb = 4L * rows_per_iter;
     rpb = (rpb + rows_per_iter - 1) / rows_per_iter * rows_per_iter;
     p.rows_per_block = rpb;
     p.ntc = (int)((nrows + rpb - 1) / rpb);
@@ -212,8 +245,15 @@ void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hip
     if (nrows == 0 || nbatch == 0) return;
     if (nbatch > 65535) fail(std::string(what) + ": too many kept rows");
     fo.n1 = rs.n1;
-    hipLaunchKernelGGL(k_colreduce<KIND>, dim3(p.nstrips, p.ntc, nbatch), dim3(BLOCK), 0, st, rs, a, ws,
-                       p.lpr_log2, p.rows_per_block, nrows);
+    bool fast = true;       // inputs and the elementwise output are all 128-bit addressable
+    for (int t = 0; t < ColIn<KIND>::N; ++t) fast = fast && a.v[ColIn<KIND>::idx[t]].vec;
+    if (KIND != COL_BAOB) fast = fast && a.v[3].vec;
+    if (fast)
+        hipLaunchKernelGGL((k_colreduce<KIND, true>), dim3(p.nstrips, p.ntc, nbatch), dim3(BLOCK), 0, st, rs,
+                           a, ws, p.lpr_log2, p.rows_per_block, nrows);
+    else
+        hipLaunchKernelGGL((k_colreduce<KIND, false>), dim3(p.nstrips, p.ntc, nbatch), dim3(BLOCK), 0, st, rs,
+                           a, ws, p.lpr_log2, p.rows_per_block, nrows);
     check_launch(what);
     long n = (long)NS * nbatch * rs.R;
     hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((n + 31) / 32)), dim3(BLOCK), 0, st,

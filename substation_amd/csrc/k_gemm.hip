@@ -51,10 +51,11 @@ __global__ __launch_bounds__(256) void k_gemm_scalar(GemmArgs g, long total) {
         const half_t* b0p = bp + (long)k0 * g.sBK0;
         for (int k = 0; k < g.K1; ++k) acc += (float)a0[(long)k * g.sAK1] * (float)b0p[(long)k * g.sBK1];
     }
-    acc *= g.alpha;
-    if (g.bias)
-        acc += (float)g.bias[b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] + (long)m * g.sbM + (long)n * g.sbN];
-    g.C[b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2] + (long)m * g.sCM + (long)n * g.sCN] = (half_t)acc;
+    half_t out = (half_t)(acc * g.alpha);
+    if (g.bias)     // same two roundings as the product followed by a separate add
+        out = (half_t)((float)out + (float)g.bias[b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] +
+                                                  (long)m * g.sbM + (long)n * g.sbN]);
+    g.C[b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2] + (long)m * g.sCM + (long)n * g.sCN] = out;
 }
 
 // ---------------------------------------------------------------------------
@@ -327,14 +328,7 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
                 h4 w;
                 int ncol = j * 32 + q * 8 + hi * 4;        // within the wave's columns
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float x = acc[i][j][q * 4 + e] * g.alpha;
-                    if (biasb) {
-                        int mm = mrow + l32, nn = n0 + wn * 32 * TN + ncol + e;
-                        if (mm < g.M && nn < g.N) x += (float)biasb[(long)mm * g.sbM + (long)nn * g.sbN];
-                    }
-                    w[e] = (half_t)x;
-                }
+                for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[i][j][q * 4 + e] * g.alpha);
                 *reinterpret_cast<h4*>(stage + l32 * STAGE_PITCH + ncol) = w;
             }
         // LDS operations of one wave execute in order: the reads below see the writes above.
@@ -343,8 +337,15 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
             int r = it * RPI + lane / LPR, c8 = (lane % LPR) * 8;
             h8 val = *reinterpret_cast<const h8*>(stage + r * STAGE_PITCH + c8);
             int mm = mrow + r, nn = n0 + wn * 32 * TN + c8;
-            if (mm < g.M && nn + 8 <= g.N)
+            if (mm < g.M && nn + 8 <= g.N) {
+                if (biasb) {
+                    // the addend (a bias row or a whole tensor) is N-contiguous like C
+                    h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
+                }
                 *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
+            }
         }
     }
 }
@@ -396,6 +397,9 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     if (!bkc && a.sBN != 1) return 0;
     if (!al16(a.A) || !al16(a.B) || !al16(a.C)) return 0;
     if (a.K0 > 1 && a.K1 % BK != 0) return 0;
+    if (a.bias && !(a.sbN == 1 && mult8(a.sbM) && mult8(a.sbb[0]) && mult8(a.sbb[1]) && mult8(a.sbb[2]) &&
+                    al16(a.bias)))
+        return 0;
     // every 16-byte access must be aligned and whole
     bool ok = mult8(a.N) && mult8(a.sCM) && mult8(a.sCb[0]) && mult8(a.sCb[1]) && mult8(a.sCb[2]);
     ok = ok && mult8(a.sAK0) && mult8(a.sAb[0]) && mult8(a.sAb[1]) && mult8(a.sAb[2]);
@@ -432,8 +436,8 @@ void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, hipStream_t 
 
 }  // namespace
 
-int gemm_kernel_kind(const GemmShape& s, const void* A, const void* B, const void* C) {
-    GemmEpilogue ep;
+int gemm_kernel_kind(const GemmShape& s, const void* A, const void* B, const void* C,
+                     const GemmEpilogue& ep) {
     Canon c = canonicalise(s, (const half_t*)A, (const half_t*)B, (half_t*)C, 1.f, ep);
     bool akc, bkc;
     return pick_kind(c, akc, bkc);

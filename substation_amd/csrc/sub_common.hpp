@@ -120,6 +120,9 @@ struct GemmShape {
     int nbatch = 0;
     int64_t nb[3] = {1, 1, 1};
     int64_t sAb[3] = {0, 0, 0}, sBb[3] = {0, 0, 0}, sCb[3] = {0, 0, 0};
+    // logical dims of the M group, the N group (outer to inner) and the batch dims
+    int nmd = 0, nnd = 0;
+    int mdims[NDIM] = {0}, ndims[NDIM] = {0}, bdims[3] = {0, 0, 0};
     int64_t batch() const { return nb[0] * nb[1] * nb[2]; }
     int64_t K() const { return K0 * K1; }
 };
@@ -192,6 +195,11 @@ inline GemmShape classify_einsum(const Layout& A, const Layout& B, const Layout&
         g.sBb[i] = B.has[d] ? B.stride[d] : 0;
         g.sCb[i] = C.stride[d];
     }
+    for (int i = 0; i < g.nbatch; ++i) g.bdims[i] = batch[i];
+    mg = ordered_by(mg, C); ng = ordered_by(ng, C);
+    g.nmd = (int)mg.size(); g.nnd = (int)ng.size();
+    for (int i = 0; i < g.nmd; ++i) g.mdims[i] = mg[i];
+    for (int i = 0; i < g.nnd; ++i) g.ndims[i] = ng[i];
     g.M = prod(mg, A); g.sAM = group_stride(mg, A); g.sCM = group_stride(mg, C);
     g.N = prod(ng, B); g.sBN = group_stride(ng, B); g.sCN = group_stride(ng, C);
     // contraction: one merged group, or an outer + inner split
@@ -212,6 +220,35 @@ inline GemmShape classify_einsum(const Layout& A, const Layout& B, const Layout&
         if (!ok) fail("einsum: contraction dimensions are not contiguous in " + A.str() + " / " + B.str());
     }
     return g;
+}
+
+// Strides of a tensor T (its dims a subset of C's) along the M, N and batch
+// indices of a classified contraction, so that T can be added to C in the GEMM
+// epilogue.  False when a merged group does not map to a single stride of T.
+inline bool addend_strides(const GemmShape& g, const Layout& T, const Layout& C, int64_t& sM, int64_t& sN,
+                           int64_t (&sb)[3]) {
+    auto group = [&](const int* dims, int n, int64_t& out) {
+        // dims outer -> inner; present dims must chain like a dense sub-block,
+        // absent ones must all be absent (broadcast)
+        int present = 0;
+        for (int i = 0; i < n; ++i) present += T.has[dims[i]] ? 1 : 0;
+        if (present == 0) { out = 0; return true; }
+        if (present != n) return false;
+        for (int i = 0; i + 1 < n; ++i)
+            if (T.stride[dims[i]] != C.size[dims[i + 1]] * T.stride[dims[i + 1]]) return false;
+        out = n ? T.stride[dims[n - 1]] : 0;
+        return true;
+    };
+    if (!group(g.mdims, g.nmd, sM) || !group(g.ndims, g.nnd, sN)) return false;
+    int covered = 0;
+    for (int i = 0; i < 3; ++i) sb[i] = 0;
+    for (int i = 0; i < g.nbatch; ++i) {
+        sb[i] = T.has[g.bdims[i]] ? T.stride[g.bdims[i]] : 0;
+        covered += T.has[g.bdims[i]] ? 1 : 0;
+    }
+    for (int i = 0; i < g.nmd; ++i) covered += T.has[g.mdims[i]] ? 1 : 0;
+    for (int i = 0; i < g.nnd; ++i) covered += T.has[g.ndims[i]] ? 1 : 0;
+    return covered == T.rank;     // every dim of T is one of C's free or batch dims
 }
 
 }  // namespace sub

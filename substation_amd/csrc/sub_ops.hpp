@@ -55,14 +55,17 @@ void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, 
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
 
 // --- tensor contraction ------------------------------------------------------
+// Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
+// that broadcasts along M or N, or a whole tensor (a residual).
 struct GemmEpilogue {
-    const half_t* bias = nullptr;   // optional bias added after alpha scaling
-    int64_t sbM = 0, sbN = 0;       // bias strides along M and N
+    const half_t* bias = nullptr;
+    int64_t sbM = 0, sbN = 0;       // addend strides along M and N
     int64_t sbb[3] = {0, 0, 0};     // and along the batch dims
 };
 void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C, float alpha,
                  const GemmEpilogue& ep, hipStream_t st);
 // Which kernel launch_gemm would pick: 0 = scalar fallback, 1 = MFMA.
-int gemm_kernel_kind(const GemmShape& g, const void* A, const void* B, const void* C);
+int gemm_kernel_kind(const GemmShape& g, const void* A, const void* B, const void* C,
+                     const GemmEpilogue& ep = GemmEpilogue());
 
 }  // namespace sub

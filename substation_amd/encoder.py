@@ -70,6 +70,10 @@ class Encoder(torch.nn.Module):
         self._handle = _lib.Handle(config)
         if profiling:
             self._handle.profile_enable(True)
+        if enable_debug:
+            # debug capture promises every named intermediate: keep the separate
+            # aib / bei operators instead of fusing them into GEMM epilogues
+            self._handle.set_option(_lib.OPT_FUSE_EPILOGUES, 0)
         handle = self._handle
         lib = handle.lib
         module = self
