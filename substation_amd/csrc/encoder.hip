@@ -168,8 +168,10 @@ struct Handle {
     int pos_p[SUB_N_PARAMS], pos_f[SUB_N_FWD], pos_b[SUB_N_BWD];   // internal id -> caller position
     Layout lKK, lQQ, lDKK, lDQQ, lWsub, lBsub;
     GemmPlan gemm[G_COUNT];
-    float* ws = nullptr;
+    float* ws = nullptr;          // column-reduction partials
     size_t ws_floats = 0;
+    float* gws = nullptr;         // split-k partials of the small-output contractions
+    size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
     bool fuse_epilogues = true;
     std::vector<ProfEntry> prof;
@@ -177,6 +179,7 @@ struct Handle {
 
     ~Handle() {
         if (ws) (void)hipFree(ws);
+        if (gws) (void)hipFree(gws);
         for (auto& e : prof) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
     }
 };
@@ -325,6 +328,11 @@ void configure(Handle& h, const sub_config* c) {
     plan_fused(G_QKV_BIAS, h.lX, h.lp[WKQV], h.lf[KKQQVV], h.lp[BKQV]);
     plan_fused(G_DXQKV_RESID, h.lp[WKQV], h.lb[DKKQQVV], h.lX, h.lb[DRESID1]);
 
+    h.gws_need = 0;
+    for (int i = 0; i < G_COUNT; ++i) {
+        size_t n = gemm_splitk_ws_floats(h.gemm[i].shape);
+        if (n > h.gws_need) h.gws_need = n;
+    }
     // The fp32 scratch of the column reductions is allocated by the first
     // operator that needs it, so that configuring needs no GPU.
     h.configured = true;
@@ -342,7 +350,14 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
         ep.bias = (const half_t*)addend; ep.sbM = p.sM; ep.sbN = p.sN;
         for (int i = 0; i < 3; ++i) ep.sbb[i] = p.sb[i];
     }
-    launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream);
+    if (h.gws_need > h.gws_floats) {
+        if (h.gws) hip_check(hipFree(h.gws), "hipFree");
+        h.gws = nullptr; h.gws_floats = 0;
+        hip_check(hipMalloc((void**)&h.gws, h.gws_need * sizeof(float)), "hipMalloc(split-k workspace)");
+        h.gws_floats = h.gws_need;
+    }
+    launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream, h.gws,
+                h.gws_floats);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

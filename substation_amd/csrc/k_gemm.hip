@@ -31,6 +31,8 @@ struct GemmArgs {
     long sAb[3], sBb[3], sCb[3];
     float alpha;
     const half_t* bias; long sbM, sbN, sbb[3];
+    int splits;                   // > 1: the k range is split, fp32 partial tiles go to `partial`
+    float* partial;               // [split][batch][M][N]
 };
 
 // ---------------------------------------------------------------------------
@@ -199,6 +201,8 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
         if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
     }
     const int per_batch = tiles_m * tiles_n;
+    const int split = (int)(lid % g.splits);        // k-splits of one tile sit next to each other
+    lid /= g.splits;
     long bz = lid / per_batch;
     int r = (int)(lid - bz * per_batch);
     constexpr int GM = 8;
@@ -214,7 +218,10 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
     const int mleft = g.M - m0, nleft = g.N - n0;
 
     const int tiles_per_k1 = (g.K1 + BK - 1) / BK;
-    const int nkt = g.K0 * tiles_per_k1;
+    const int nkt_all = g.K0 * tiles_per_k1;
+    // this workgroup's share of the k-tiles
+    const int kt_begin = (int)((long)nkt_all * split / g.splits);
+    const int nkt = (int)((long)nkt_all * (split + 1) / g.splits) - kt_begin;
 
     f16v acc[TM][TN];
 #pragma unroll
@@ -235,9 +242,9 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
     // Running (wave-uniform) pointers to the next k-tile to fetch.  Past the last
     // tile they stay on it: the surplus prefetches re-read valid memory and are
     // never consumed, which keeps the loop body free of branches.
-    const half_t* pa = Ab;
-    const half_t* pb = Bb;
-    int kin = 0, fetched = 0;
+    int kin = kt_begin % tiles_per_k1, fetched = 0;
+    const half_t* pa = Ab + (long)(kt_begin / tiles_per_k1) * g.sAK0 + (long)kin * BK * g.sAK1;
+    const half_t* pb = Bb + (long)(kt_begin / tiles_per_k1) * g.sBK0 + (long)kin * BK * g.sBK1;
     const long stepA = (long)BK * g.sAK1, stepB = (long)BK * g.sBK1;
     const long wrapA = g.sAK0 - (long)(tiles_per_k1 - 1) * stepA;
     const long wrapB = g.sBK0 - (long)(tiles_per_k1 - 1) * stepB;
@@ -311,6 +318,26 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 #undef SUB_GEMM_STORE
 #undef SUB_GEMM_ISSUE
 
+    if (g.splits > 1) {
+        // split k: raw fp32 partial tile, [split][batch][M][N]; a second kernel adds them up
+        const long nb_total = (long)gridDim.x / g.splits / per_batch;
+        float* P = g.partial + ((long)split * nb_total + bz) * (long)g.M * g.N;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    int mm = m0 + wm * 32 * TM + i * 32 + l32;
+                    int nn = n0 + wn * 32 * TN + j * 32 + q * 8 + hi * 4;
+                    if (mm < g.M && nn + 4 <= g.N) {
+                        float4 v4 = make_float4(acc[i][j][q * 4 + 0], acc[i][j][q * 4 + 1],
+                                                acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+                        *reinterpret_cast<float4*>(P + (long)mm * g.N + nn) = v4;
+                    }
+                }
+        return;
+    }
     // Epilogue: per 32-row slab, accumulators -> LDS (8-byte packs of 4
     // consecutive n) -> 16-byte row segments -> global.
     half_t* stage = lds + wave * STAGE_WAVE;
@@ -350,6 +377,269 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// Asynchronous variant for full tiles: global memory -> LDS directly
+// (global_load_lds_dwordx4), a ring of S stages, no staging registers and no
+// ds_write.  Each wave instruction deposits 64 x 16 bytes at consecutive LDS
+// addresses, so the lane -> global-chunk map is chosen such that the bytes land
+// in the (bank-swizzled) tile layout the fragment reads expect.  The stages are
+// separate __shared__ arrays and the k loop is unrolled over them, which lets
+// the compiler see that the fragment reads of one stage do not depend on the
+// loads in flight to another; completion is tracked by hand with s_waitcnt
+// vmcnt(n) followed by a plain s_barrier.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef __attribute__((address_space(1))) const void* global_void_ptr;
+
+constexpr int waitcnt_vm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | 0x0F70; }
+
+template <int ROWS, bool KC>
+struct DTile {
+    static constexpr int HALVES = ROWS * BK;
+    static constexpr int NV = ROWS / 32;            // loads per thread (16 per tile per wave group)
+    static constexpr int VPR = ROWS / 8;            // 16-byte units per k-row (!KC)
+
+    static __device__ __forceinline__ int kc_off(int row, int slot) {
+        return row * BK + ((slot ^ (row ^ (row >> 3))) & 7) * 8;
+    }
+    // !KC: [k][free] with the 16-byte unit index xor-ed so that the four k-rows a
+    // 16-lane group of the transpose read touches fall into different banks.
+    static __device__ __forceinline__ int mc_swz(int k) {
+        return VPR >= 16 ? ((k & 3) << 2) : (((k >> 1) & 1) << 2);
+    }
+
+    // Element offset (from the tile's first element in global memory) of the
+    // chunk lane `lane` of wave `wave` fetches with its i-th load.
+    static __device__ __forceinline__ void offsets(unsigned (&off)[NV], long sF, long sK, int wave, int lane) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int inst = wave * NV + i;          // which 1024-byte slab of the tile
+            if (KC) {
+                int row = inst * 8 + (lane >> 3), pslot = lane & 7;
+                int lslot = (pslot ^ (row ^ (row >> 3))) & 7;
+                off[i] = (unsigned)((long)row * sF + lslot * 8);
+            } else {
+                constexpr int KPI = 64 / VPR;        // k-rows per instruction
+                int k = inst * KPI + lane / VPR, punit = lane % VPR;
+                int lunit = punit ^ mc_swz(k);
+                off[i] = (unsigned)((long)k * sK + lunit * 8);
+            }
+        }
+    }
+
+    static __device__ __forceinline__ void issue(half_t* stage, const half_t* tile, const unsigned (&off)[NV],
+                                                 int wave) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+            __builtin_amdgcn_global_load_lds((global_void_ptr)(tile + off[i]),
+                                             (lds_void_ptr)(stage + (wave * NV + i) * 512), 16, 0, 0);
+    }
+
+    static __device__ __forceinline__ h8 frag(const half_t* lds, int row0, int ks, int lane) {
+        if (KC) {
+            return *reinterpret_cast<const h8*>(lds + kc_off(row0 + (lane & 31), ks * 2 + (lane >> 5)));
+        } else {
+            const int g = lane >> 4, l = lane & 15;
+            const int k = ks * 16 + 8 * (g >> 1) + (l >> 2);       // and k + 4 for the second half
+            const int m = row0 + 16 * (g & 1) + 4 * (l & 3);
+            // k & 3 == (k + 4) & 3 and ((k+4) >> 1) & 1 differs: recompute the swizzle per row
+            const half_t* p0 = lds + k * ROWS + (((m >> 3) ^ mc_swz(k)) << 3) + (m & 7);
+            const half_t* p1 = lds + (k + 4) * ROWS + (((m >> 3) ^ mc_swz(k + 4)) << 3) + (m & 7);
+            typedef s4v __attribute__((address_space(3))) * lds_s4;
+            s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p0));
+            s4v hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p1));
+            typedef short s8 __attribute__((ext_vector_type(8)));
+            s8 r = __builtin_shufflevector(lo, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(h8, r);
+        }
+    }
+};
+
+template <int TM, int TN, bool AKC, bool BKC>
+__global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
+    constexpr int BM = 64 * TM, BN = 64 * TN;
+    using TA = DTile<BM, AKC>;
+    using TB = DTile<BN, BKC>;
+    constexpr int STAGE = TA::HALVES + TB::HALVES;
+    constexpr int STAGE_PITCH = 32 * TN + 8;
+    constexpr int STAGE_WAVE = 32 * STAGE_PITCH;
+    static_assert(4 * STAGE_WAVE <= STAGE, "epilogue staging must fit one stage");
+    __shared__ __attribute__((aligned(16))) half_t st0[STAGE];
+    __shared__ __attribute__((aligned(16))) half_t st1[STAGE];
+    __shared__ __attribute__((aligned(16))) half_t st2[STAGE];
+    constexpr int L = TA::NV + TB::NV;               // loads per thread per tile
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int l32 = lane & 31, hi = lane >> 5;
+
+    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+    long lid = blockIdx.x;
+    {
+        const long nblocks = gridDim.x;
+        if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
+    }
+    const int per_batch = tiles_m * tiles_n;
+    long bz = lid / per_batch;
+    int r = (int)(lid - bz * per_batch);
+    constexpr int GM = 8;
+    const int grp = r / (GM * tiles_n), first_m = grp * GM;
+    const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
+    const int rr = r - grp * GM * tiles_n;
+    const int tile_m = first_m + rr % gsz, tile_n = rr / gsz;
+    long b2 = bz % g.nb2; long t = bz / g.nb2;
+    long b1 = t % g.nb1; long b0 = t / g.nb1;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const half_t* pa = g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM;
+    const half_t* pb = g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN;
+
+    const int tiles_per_k1 = g.K1 / BK;
+    const int nkt = g.K0 * tiles_per_k1;
+
+    f16v acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+    unsigned offa[TA::NV], offb[TB::NV];
+    TA::offsets(offa, g.sAM, g.sAK1, wave, lane);
+    TB::offsets(offb, g.sBN, g.sBK1, wave, lane);
+
+    int kin = 0, fetched = 0;
+    const long stepA = (long)BK * g.sAK1, stepB = (long)BK * g.sBK1;
+    const long wrapA = g.sAK0 - (long)(tiles_per_k1 - 1) * stepA;
+    const long wrapB = g.sBK0 - (long)(tiles_per_k1 - 1) * stepB;
+
+    // Fetch the next k-tile into `stage`; past the last tile the pointers stay put
+    // (surplus fetches re-read valid memory and keep the vmcnt bookkeeping uniform).
+#define SUB_DMA_ISSUE(stage_)                                                                     \
+    do {                                                                                          \
+        TA::issue(stage_, pa, offa, wave);                                                        \
+        TB::issue(stage_ + TA::HALVES, pb, offb, wave);                                           \
+        const bool more_ = fetched + 1 < nkt;                                                     \
+        const bool wrap_ = kin + 1 == tiles_per_k1;                                               \
+        pa += more_ ? (wrap_ ? wrapA : stepA) : 0;                                                \
+        pb += more_ ? (wrap_ ? wrapB : stepB) : 0;                                                \
+        kin = more_ ? (wrap_ ? 0 : kin + 1) : kin;                                                \
+        fetched += more_ ? 1 : 0;                                                                 \
+    } while (0)
+
+#define SUB_DMA_COMPUTE(stage_)                                                                   \
+    do {                                                                                          \
+        const half_t* sA = stage_;                                                                \
+        const half_t* sB = stage_ + TA::HALVES;                                                   \
+        h8 fa[2][TM], fb[2][TN];                                                                  \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                            \
+            fa[0][i] = TA::frag(sA, (wm * TM + i) * 32, 0, lane);                                 \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
+            fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
+        _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
+            if (ks + 1 < BK / 16) {                                                               \
+                _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
+                    fa[(ks + 1) & 1][i] = TA::frag(sA, (wm * TM + i) * 32, ks + 1, lane);         \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
+                    fb[(ks + 1) & 1][j] = TB::frag(sB, (wn * TN + j) * 32, ks + 1, lane);         \
+            }                                                                                     \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i)                                        \
+                _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][j], fa[ks & 1][i], \
+                                                                       acc[i][j], 0, 0, 0);       \
+        }                                                                                         \
+    } while (0)
+
+    // One step: tile kt is complete once at most the L loads of tile kt+1 are
+    // outstanding; the barrier also says every wave is done reading the stage
+    // that the fetch below overwrites (it was computed on one step earlier).
+#define SUB_DMA_STEP(cur_, nxt2_)                                                                 \
+    do {                                                                                          \
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));                                                \
+        __builtin_amdgcn_s_barrier();                                                             \
+        SUB_DMA_ISSUE(nxt2_);                                                                     \
+        SUB_DMA_COMPUTE(cur_);                                                                    \
+    } while (0)
+
+    SUB_DMA_ISSUE(st0);                // tile 0
+    SUB_DMA_ISSUE(st1);                // tile 1 (or a surplus copy of the last tile)
+    const int ntriples = nkt / 3;
+    for (int p = 0; p < ntriples; ++p) {
+        SUB_DMA_STEP(st0, st2);
+        SUB_DMA_STEP(st1, st0);
+        SUB_DMA_STEP(st2, st1);
+    }
+    const int rem = nkt - 3 * ntriples;
+    if (rem >= 1) SUB_DMA_STEP(st0, st2);
+    if (rem >= 2) SUB_DMA_STEP(st1, st0);
+#undef SUB_DMA_STEP
+#undef SUB_DMA_COMPUTE
+#undef SUB_DMA_ISSUE
+    // surplus fetches may still be landing: drain them before LDS is reused
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+
+    half_t* stage = st0 + wave * STAGE_WAVE;
+    half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
+    const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
+    constexpr int LPR = 4 * TN;
+    constexpr int RPI = 64 / LPR;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int mrow = m0 + wm * 32 * TM + i * 32;
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                h4 w;
+                int ncol = j * 32 + q * 8 + hi * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[i][j][q * 4 + e] * g.alpha);
+                *reinterpret_cast<h4*>(stage + l32 * STAGE_PITCH + ncol) = w;
+            }
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            int rr2 = it * RPI + lane / LPR, c8 = (lane % LPR) * 8;
+            h8 val = *reinterpret_cast<const h8*>(stage + rr2 * STAGE_PITCH + c8);
+            int mm = mrow + rr2, nn = n0 + wn * 32 * TN + c8;
+            if (biasb) {
+                h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
+            }
+            *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
+        }
+    }
+}
+
+// Adds the k-split partials: C[b,m,n] = fp16(alpha * sum_s P[s][b][m][n]) (+ addend).
+__global__ __launch_bounds__(256) void k_gemm_splitk_reduce(GemmArgs g, long nb_total) {
+    const long quads = (long)g.N / 4;
+    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= nb_total * g.M * quads) return;
+    int nq = (int)(idx % quads); long rr = idx / quads;
+    int m = (int)(rr % g.M); long bz = rr / g.M;
+    const long slab = nb_total * (long)g.M * g.N;
+    const float* p = g.partial + (bz * g.M + m) * (long)g.N + nq * 4;
+    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int s = 0; s < g.splits; ++s) {
+        float4 v = *reinterpret_cast<const float4*>(p + (long)s * slab);
+        t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
+    }
+    long b2 = bz % g.nb2; long tt = bz / g.nb2;
+    long b1 = tt % g.nb1; long b0 = tt / g.nb1;
+    half_t* c = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2] + (long)m * g.sCM + nq * 4;
+    h4 o;
+    o[0] = (half_t)(t.x * g.alpha); o[1] = (half_t)(t.y * g.alpha);
+    o[2] = (half_t)(t.z * g.alpha); o[3] = (half_t)(t.w * g.alpha);
+    if (g.bias) {
+        const half_t* ad = g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] + (long)m * g.sbM + nq * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (half_t)((float)o[e] + (float)ad[e]);
+    }
+    *reinterpret_cast<h4*>(c) = o;
+}
+
 inline bool mult8(long x) { return (x & 7) == 0; }
 inline bool al16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -383,6 +673,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     a.nb1 = (int)s.nb[1]; a.nb2 = (int)s.nb[2];
     for (int i = 0; i < 3; ++i) { a.sCb[i] = s.sCb[i]; a.sbb[i] = ep.sbb[i]; }
     a.alpha = alpha; a.bias = ep.bias;
+    a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;
 }
@@ -425,13 +716,45 @@ void launch_mfma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t 
 }
 
 template <int TM, int TN>
-void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, hipStream_t st) {
-    long nblocks = (long)((a.N + 64 * TN - 1) / (64 * TN)) * ((a.M + 64 * TM - 1) / (64 * TM)) * batch;
+void launch_dma(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
+    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true>), grid, dim3(256), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false>), grid, dim3(256), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false>), grid, dim3(256), 0, st, a);
+}
+
+template <int TM, int TN, bool DMA_OK>
+void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, bool dma, hipStream_t st) {
+    long nblocks = (long)((a.N + 64 * TN - 1) / (64 * TN)) * ((a.M + 64 * TM - 1) / (64 * TM)) * batch *
+                   a.splits;
     if (nblocks > 0x7fffffffL) fail("gemm: too many tiles");
     dim3 grid((unsigned)nblocks);
     const bool full = a.M % (64 * TM) == 0 && a.N % (64 * TN) == 0 && a.K1 % BK == 0;
+    if (DMA_OK && full && dma && a.splits == 1) { launch_dma<TM, TN>(a, akc, bkc, grid, st); return; }
     if (full) launch_mfma2<TM, TN, true>(a, akc, bkc, grid, st);
     else launch_mfma2<TM, TN, false>(a, akc, bkc, grid, st);
+    if (a.splits > 1) {
+        long n = batch * (long)a.M * (a.N / 4);
+        hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, batch);
+    }
+}
+
+constexpr size_t kSplitMaxOut = 2u << 20;     // largest output (elements) whose contraction is split
+
+// How many ways to split k so that a small output still fills the chip: the
+// weight-gradient products have few output tiles and a long contraction.
+int pick_splits(const GemmArgs& a, long batch, size_t ws_floats) {
+    static const int force = [] { const char* e = getenv("SUB_GEMM_SPLITK"); return e ? atoi(e) : 0; }();
+    const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
+    const int nkt = a.K0 * ((a.K1 + BK - 1) / BK);
+    int splits = force > 0 ? force : (int)((384 + tiles - 1) / tiles);
+    if (force < 0) splits = 1;
+    if (splits > 8) splits = 8;
+    while (splits > 1 && nkt / splits < 8) --splits;
+    const size_t need = (size_t)batch * a.M * a.N;          // floats per split
+    while (splits > 1 && need * splits > ws_floats) --splits;
+    if (a.N % 4 != 0) splits = 1;
+    return splits < 1 ? 1 : splits;
 }
 
 }  // namespace
@@ -443,8 +766,19 @@ int gemm_kernel_kind(const GemmShape& s, const void* A, const void* B, const voi
     return pick_kind(c, akc, bkc);
 }
 
+size_t gemm_splitk_ws_floats(const GemmShape& s) {
+    // only small outputs are split (measured: beyond ~2M elements the fp32 partial
+    // traffic costs more than the extra workgroups gain)
+    size_t per = (size_t)s.batch() * s.M * s.N;
+    long tiles = ((s.M + 127) / 128) * ((s.N + 127) / 128) * s.batch();
+    if (tiles >= 384 || per > kSplitMaxOut) return 0;
+    size_t splits = (384 + tiles - 1) / tiles;
+    if (splits > 8) splits = 8;
+    return per * splits;
+}
+
 void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C, float alpha,
-                 const GemmEpilogue& ep, hipStream_t st) {
+                 const GemmEpilogue& ep, hipStream_t st, float* ws, size_t ws_floats) {
     long batch = s.batch();
     if (batch == 0 || s.M == 0 || s.N == 0) return;
     Canon c = canonicalise(s, A, B, C, alpha, ep);
@@ -453,9 +787,19 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
     if (kind == 1) {
         static const int force = [] { const char* e = getenv("SUB_GEMM_TILE"); return e ? atoi(e) : 0; }();
         int tile = force ? force : pick_tile(c.a, batch);
-        if (tile == 42) launch_mfma<4, 2>(c.a, akc, bkc, batch, st);
-        else if (tile == 21) launch_mfma<2, 1>(c.a, akc, bkc, batch, st);
-        else launch_mfma<2, 2>(c.a, akc, bkc, batch, st);
+        // SUB_GEMM_DMA: -1 never / 1 always use the asynchronous kernel; default: when both
+        // operands are k-contiguous and there is at most about one tile per CU, where
+        // the register-staged kernel has no second workgroup to hide its waits behind.
+        static const int dma_env = [] { const char* e = getenv("SUB_GEMM_DMA"); return e ? atoi(e) : 0; }();
+        const long tiles128 = (long)((c.a.M + 127) / 128) * ((c.a.N + 127) / 128) * batch;
+        if (ws && (size_t)batch * c.a.M * c.a.N <= kSplitMaxOut) {
+            c.a.splits = pick_splits(c.a, batch, ws_floats);
+            c.a.partial = ws;
+        }
+        const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
+        if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
+        else if (tile == 21) launch_mfma<2, 1, false>(c.a, akc, bkc, batch, false, st);
+        else launch_mfma<2, 2, true>(c.a, akc, bkc, batch, dma, st);
     } else {
         long total = batch * (long)c.a.M * c.a.N;
         long blocks = (total + 255) / 256;

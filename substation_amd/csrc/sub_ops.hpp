@@ -62,8 +62,12 @@ struct GemmEpilogue {
     int64_t sbM = 0, sbN = 0;       // addend strides along M and N
     int64_t sbb[3] = {0, 0, 0};     // and along the batch dims
 };
+// `ws` (optional): fp32 scratch of ws_floats elements for splitting the
+// contraction of small-output products across workgroups.
 void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C, float alpha,
-                 const GemmEpilogue& ep, hipStream_t st);
+                 const GemmEpilogue& ep, hipStream_t st, float* ws = nullptr, size_t ws_floats = 0);
+// Scratch (in floats) that launch_gemm can make use of for this shape; 0 if none.
+size_t gemm_splitk_ws_floats(const GemmShape& g);
 // Which kernel launch_gemm would pick: 0 = scalar fallback, 1 = MFMA.
 int gemm_kernel_kind(const GemmShape& g, const void* A, const void* B, const void* C,
                      const GemmEpilogue& ep = GemmEpilogue());
