@@ -165,6 +165,9 @@ def main():
     ap.add_argument('--profile-steps', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--per-op', action='store_true', help='print the per-operator table to stderr')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
+                         'FETCH_SIZE / WRITE_SIZE readings')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py: this build runs the encoder layer on ONE GPU only (no collectives exist on '
@@ -196,6 +199,14 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.copy_calibration:
+        a = torch.empty(128 << 20, dtype=torch.float16, device='cuda').normal_()
+        b = torch.empty_like(a)
+        for _ in range(5):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
 
     # Per-operator durations: HIP events recorded by the library around every
     # launch, on the stream the kernels run on.

@@ -191,9 +191,12 @@ int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, c
  * (0 for absent dims) under the handle's sizes. */
 int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]);
 /* einsumparser.h:9-55.  out = {batch, M, N, K, sAM, sAK, sAB0, sBN, sBK, sBB0,
- * sCM, sCN, sCB0, nbatchdims, K0, sAK0, sBK0, kernel_kind} */
+ * sCM, sCN, sCB0, nbatchdims, K0, sAK0, sBK0, kernel_kind (0 scalar, 1 MFMA),
+ * nb[3], sAb[3], sBb[3], sCb[3], K1, 0}: up to three batch dims with their own
+ * strides (0 where an operand lacks the dim) and K = K0 * K1 (outer x inner
+ * contraction group). */
 int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const char* l_C,
-                        int64_t out[18]);
+                        int64_t out[32]);
 /* The 16-bit random fields of canonical elements start .. start+n-1, computed
  * on the host by the same code the kernels run. */
 int sub_philox_fields_host(uint64_t seed, uint32_t site, uint32_t step, uint64_t start,

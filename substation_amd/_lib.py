@@ -178,12 +178,15 @@ class Handle:
         return dict(zip('BJKHPIUQ', out))
 
     def classify(self, la, lb, lc):
-        out = (ctypes.c_int64 * 18)()
+        out = (ctypes.c_int64 * 32)()
         check(self.lib.sub_einsum_classify(self.ptr, la.encode(), lb.encode(), lc.encode(), out),
               'sub_einsum_classify')
         keys = ('batch', 'M', 'N', 'K', 'sAM', 'sAK', 'sAB', 'sBN', 'sBK', 'sBB', 'sCM', 'sCN', 'sCB',
                 'nbatch', 'K0', 'sAK0', 'sBK0', 'kernel')
-        return dict(zip(keys, out))
+        d = dict(zip(keys, out))
+        d['nb'] = list(out[18:21]); d['sAb'] = list(out[21:24]); d['sBb'] = list(out[24:27])
+        d['sCb'] = list(out[27:30]); d['K1'] = out[30]
+        return d
 
 
 def philox_fields_host(seed, site, step, start, n):

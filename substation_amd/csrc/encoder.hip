@@ -931,7 +931,7 @@ int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]) {
 }
 
 int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const char* l_C,
-                        int64_t out[18]) {
+                        int64_t out[32]) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
         GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), L(h, l_C));
@@ -942,6 +942,10 @@ int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const ch
         out[13] = g.nbatch; out[14] = g.K0; out[15] = g.sAK0; out[16] = g.sBK0;
         // alignment of real buffers is unknown here: assume 16-byte aligned bases
         out[17] = gemm_kernel_kind(g, (const void*)16, (const void*)16, (const void*)16);
+        for (int i = 0; i < 3; ++i) {
+            out[18 + i] = g.nb[i]; out[21 + i] = g.sAb[i]; out[24 + i] = g.sBb[i]; out[27 + i] = g.sCb[i];
+        }
+        out[30] = g.K1; out[31] = 0;
     });
 }
 

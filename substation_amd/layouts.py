@@ -13,7 +13,6 @@ pytorch_module/encoder.py:56,81,111,117,229-376)::
 ``algorithms`` (cuBLAS algorithm ids) are accepted and ignored: the HIP kernels
 vectorise along whichever dim is contiguous and there is one GEMM kernel family.
 """
-import io
 import pickle
 
 PARAM_NAMES = ['WKQV', 'BKQV', 'WO', 'BO', 'S1', 'B1', 'LINB1', 'LINW1', 'S2', 'B2', 'LINB2', 'LINW2']
@@ -136,12 +135,77 @@ def validate(layouts):
     return layouts
 
 
-class _DataOnlyUnpickler(pickle.Unpickler):
-    """Loads dict/list/tuple/str pickles and refuses every global lookup, so that
-    nothing from the file can execute."""
+def _read_data_pickle(data):
+    """Decodes a pickle that holds only dict / list / tuple / str / int / bool /
+    None.  The byte stream is walked with ``pickletools.genops`` (a disassembler)
+    and rebuilt by the small stack machine below; opcodes that name, import or
+    call anything (GLOBAL, REDUCE, BUILD, NEWOBJ, ...) are rejected, so nothing
+    from the file can execute."""
+    import pickletools
+    stack, marks, memo = [], [], {}
+    mark = object()
 
-    def find_class(self, module, name):
-        raise pickle.UnpicklingError(f'layouts file refers to {module}.{name}; only plain data is allowed')
+    def pop_mark():
+        i = len(stack) - 1 - stack[::-1].index(mark)
+        items = stack[i + 1:]
+        del stack[i:]
+        return items
+
+    for op, arg, _ in pickletools.genops(data):
+        n = op.name
+        if n in ('PROTO', 'FRAME'):
+            continue
+        elif n == 'STOP':
+            break
+        elif n == 'MARK':
+            stack.append(mark)
+        elif n == 'EMPTY_DICT':
+            stack.append({})
+        elif n == 'EMPTY_LIST':
+            stack.append([])
+        elif n == 'EMPTY_TUPLE':
+            stack.append(())
+        elif n in ('BINUNICODE', 'SHORT_BINUNICODE', 'BINUNICODE8', 'UNICODE', 'BININT', 'BININT1',
+                   'BININT2', 'INT', 'LONG1', 'BINFLOAT'):
+            stack.append(arg)
+        elif n == 'NONE':
+            stack.append(None)
+        elif n in ('NEWTRUE', 'NEWFALSE'):
+            stack.append(n == 'NEWTRUE')
+        elif n in ('MEMOIZE',):
+            memo[len(memo)] = stack[-1]
+        elif n in ('BINPUT', 'LONG_BINPUT', 'PUT'):
+            memo[arg] = stack[-1]
+        elif n in ('BINGET', 'LONG_BINGET', 'GET'):
+            stack.append(memo[arg])
+        elif n == 'TUPLE':
+            stack.append(tuple(pop_mark()))
+        elif n in ('TUPLE1', 'TUPLE2', 'TUPLE3'):
+            k = int(n[-1])
+            items = stack[-k:]
+            del stack[-k:]
+            stack.append(tuple(items))
+        elif n == 'APPEND':
+            v = stack.pop(); stack[-1].append(v)
+        elif n == 'APPENDS':
+            items = pop_mark(); stack[-1].extend(items)
+        elif n == 'SETITEM':
+            v = stack.pop(); k = stack.pop(); stack[-1][k] = v
+        elif n == 'SETITEMS':
+            items = pop_mark()
+            for i in range(0, len(items), 2):
+                stack[-1][items[i]] = items[i + 1]
+        elif n == 'DICT':
+            items = pop_mark()
+            stack.append({items[i]: items[i + 1] for i in range(0, len(items), 2)})
+        elif n == 'LIST':
+            stack.append(list(pop_mark()))
+        else:
+            raise pickle.UnpicklingError(
+                f'layouts file uses pickle opcode {n}; only plain dict/list/tuple/str data is allowed')
+    if len(stack) != 1:
+        raise pickle.UnpicklingError('malformed layouts pickle')
+    return stack[0]
 
 
 def load_layouts(path):
@@ -149,7 +213,7 @@ def load_layouts(path):
     config_selection/optimize.py:443-493 (or by save_layouts)."""
     with open(path, 'rb') as f:
         data = f.read()
-    return validate(_DataOnlyUnpickler(io.BytesIO(data)).load())
+    return validate(_read_data_pickle(data))
 
 
 def save_layouts(layouts, path):
