@@ -34,6 +34,22 @@ CONFIGS = {
             name='configs[4]: wide encoder layer fwd+bwd B=4 L=2048 H=32 E=4096 P=128 FF=16384 GELU fp16'),
 }
 
+# HBM-side bytes per launch at the default workload and layouts: rocprofv3 FETCH_SIZE (x2.000) +
+# WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
+# profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
+MEASURED_TRAFFIC_CFG3 = {
+    'QKV-fused': 91621893, 'QKT': 84086417, 'softmax': 268701348,
+    'gamma': 84090513, 'out': 33751434, 'bdrln1': 59106304,
+    'lin1': 99703334, 'bad': 134437888, 'lin2': 109241083,
+    'bdrln2': 59105728, 'bsb': 26412177, 'blnrd1': 42148836,
+    'dXlin2': 100605894, 'dWlin2': 109277047, 'bdrlb': 135210466,
+    'dXlin1': 109264486, 'dWlin1': 109276901, 'ebsb': 43702960,
+    'blnrd2': 42148434, 'baob': 9025049, 'dWout': 129458241,
+    'dXout': 33775166, 'dX1gamma': 84086545, 'dX2gamma': 84086362,
+    'bs': 268534218, 'dX1QKT': 84087478, 'dX2QKT': 84084698,
+    'dXQKV-fused': 92489041, 'dWQKV-fused': 115567343, 'baib': 26066282,
+}
+
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
             'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
 
@@ -260,7 +276,9 @@ def main():
                    'baseline': 'reference README.md:23: 6.71 ms on V100-SXM2 (other hardware)'},
         'roofline': {
             'kernel': dom['op'], 'bound': dom['bound'], 'achieved': dom['achieved'], 'peak': dom['peak'],
-            'unit': dom['unit'], 'frac': dom['frac'], 'traffic': None,
+            'unit': dom['unit'], 'frac': dom['frac'],
+            'traffic': (MEASURED_TRAFFIC_CFG3.get(dom['op']) if args.config == 3 and args.layouts == 'mi355x'
+                        else None),
             'launch_us': dom['us'], 'launches_per_step': 1,
         },
         'op_time_us': round(total_us, 1),

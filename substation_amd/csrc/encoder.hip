@@ -170,6 +170,10 @@ struct Handle {
     GemmPlan gemm[G_COUNT];
     float* ws = nullptr;          // column-reduction partials
     size_t ws_floats = 0;
+    size_t ws_need_bwd = 0;       // sum over the backward pass's column reductions
+    bool deferring = false;       // backward pass: finish all column reductions in one launch
+    size_t ws_cursor = 0;
+    FinishJobs deferred;
     float* gws = nullptr;         // split-k partials of the small-output contractions
     size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
@@ -219,6 +223,20 @@ void ensure_ws(Handle& h, size_t floats) {
     hip_check(hipMalloc((void**)&h.ws, floats * sizeof(float)), "hipMalloc(workspace)");
     h.ws_floats = floats;
 }
+
+// Scratch for one column reduction.  While a backward pass defers the finishing
+// stage, every reduction gets its own region of the (pre-sized) buffer.
+float* take_ws(Handle& h, size_t floats) {
+    if (!h.deferring) {
+        ensure_ws(h, floats);
+        return h.ws;
+    }
+    if (h.ws_cursor + floats > h.ws_floats) fail("column-reduction workspace exhausted");
+    float* p = h.ws + h.ws_cursor;
+    h.ws_cursor += (floats + 63) & ~(size_t)63;
+    return p;
+}
+FinishJobs* defer_of(Handle& h) { return h.deferring ? &h.deferred : nullptr; }
 
 // ---------------------------------------------------------------------------
 // Configuration
@@ -328,6 +346,15 @@ void configure(Handle& h, const sub_config* c) {
     plan_fused(G_QKV_BIAS, h.lX, h.lp[WKQV], h.lf[KKQQVV], h.lp[BKQV]);
     plan_fused(G_DXQKV_RESID, h.lp[WKQV], h.lb[DKKQQVV], h.lX, h.lb[DRESID1]);
 
+    {   // scratch of the five column reductions of one backward pass, side by side
+        Space si = make_space(sz, {dB, dJ}, dI), su = make_space(sz, {dB, dJ}, dU);
+        Space sq = make_space(sz, {dQ, dH, dB, dJ}, dP);
+        RowSpace merged{1, (int)sz.n[dQ], (int)sz.n[dB], (int)sz.n[dJ], (int)(sz.n[dH] * sz.n[dP]), 0};
+        size_t baib = colreduce_ws_floats(sq.rs, 1), baib2 = colreduce_ws_floats(merged, 1);
+        h.ws_need_bwd = colreduce_ws_floats(si.rs, 2) + colreduce_ws_floats(si.rs, 3) +
+                        colreduce_ws_floats(su.rs, 1) + colreduce_ws_floats(si.rs, 1) +
+                        (baib > baib2 ? baib : baib2) + 6 * 64;
+    }
     h.gws_need = 0;
     for (int i = 0; i < G_COUNT; ++i) {
         size_t n = gemm_splitk_ws_floats(h.gemm[i].shape);
@@ -419,9 +446,10 @@ void op_bad(Handle& h, const void* in, const Layout& lin_, const void* bias, voi
 void op_bsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* dout,
             const Layout& ldout, void* din, const Layout& ldin, void* dscale, void* dbias) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
-    ensure_ws(h, colreduce_ws_floats(sp.rs, 2));
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 2));
     launch_bsb(sp.rs, make_view(in, lin_, sp), make_view(dout, ldout, sp), vector_view(scale, sp.rs.R),
-               make_view(din, ldin, sp), ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, h.ws, h.stream);
+               make_view(din, ldin, sp), ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, ws, h.stream,
+               defer_of(h));
 }
 
 void op_ebsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* d1,
@@ -429,25 +457,25 @@ void op_ebsb(Handle& h, const void* in, const Layout& lin_, const void* scale, c
              const Layout& ldl, void* din, const Layout& ldin, void* dscale, void* dbias,
              void* dlinear_bias) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
-    ensure_ws(h, colreduce_ws_floats(sp.rs, 3));
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 3));
     launch_ebsb(sp.rs, make_view(in, lin_, sp), make_view(d1, l1, sp), make_view(d2, l2, sp),
                 make_view(dlinear, ldl, sp), vector_view(scale, sp.rs.R), make_view(din, ldin, sp),
-                ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, ColOut{(half_t*)dlinear_bias}, h.ws,
-                h.stream);
+                ColOut{(half_t*)dscale}, ColOut{(half_t*)dbias}, ColOut{(half_t*)dlinear_bias}, ws,
+                h.stream, defer_of(h));
 }
 
 void op_bdrlb(Handle& h, const void* ddrop, const Layout& ld, const void* mask, const Layout& lm,
               const void* lin, const Layout& ll, void* dlinear, const Layout& lo, void* dbias) {
     Space sp = make_space(h.sz, {dB, dJ}, dU);
-    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 1));
     launch_bdrlb(sp.rs, make_view(ddrop, ld, sp), make_view(mask, lm, sp), make_view(lin, ll, sp),
-                 make_view(dlinear, lo, sp), ColOut{(half_t*)dbias}, h.act, h.ws, h.stream);
+                 make_view(dlinear, lo, sp), ColOut{(half_t*)dbias}, h.act, ws, h.stream, defer_of(h));
 }
 
 void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
-    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
-    launch_baob(sp.rs, make_view(datt, l, sp), ColOut{(half_t*)dbo}, h.ws, h.stream);
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 1));
+    launch_baob(sp.rs, make_view(datt, l, sp), ColOut{(half_t*)dbo}, ws, h.stream, defer_of(h));
 }
 
 // out[q,p,h,b,j] = in[q,p,h,b,j] + bias[q,p,h].  The row dim is the innermost
@@ -484,15 +512,15 @@ void op_baib(Handle& h, const void* d, const Layout& ld, void* dbias, const Layo
         v.sr = 1;
         v.vec = ((H * P) % 8 == 0 && v.s1 % 8 == 0 && v.s2 % 8 == 0 && v.s3 % 8 == 0 &&
                  (reinterpret_cast<uintptr_t>(d) & 15) == 0) ? 1 : 0;
-        ensure_ws(h, colreduce_ws_floats(rs, 1));
-        launch_colsum(rs, v, (half_t*)dbias, 0, lbias.stride[dQ], 1, h.ws, h.stream);
+        float* ws = take_ws(h, colreduce_ws_floats(rs, 1));
+        launch_colsum(rs, v, (half_t*)dbias, 0, lbias.stride[dQ], 1, ws, h.stream, defer_of(h));
         return;
     }
     // general: rows of P features, kept (q,h), summed over (b,j)
     Space sp = make_space(h.sz, {dQ, dH, dB, dJ}, dP);
-    ensure_ws(h, colreduce_ws_floats(sp.rs, 1));
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 1));
     launch_colsum(sp.rs, make_view(d, ld, sp), (half_t*)dbias, lbias.stride[dQ], lbias.stride[dH],
-                  lbias.stride[dP], h.ws, h.stream);
+                  lbias.stride[dP], ws, h.stream, defer_of(h));
 }
 
 void op_bei(Handle& h, const void* a, const Layout& la, const void* b, const Layout& lb_, void* o,
@@ -565,6 +593,15 @@ void forward(Handle& h, const FwdPtrs& t) {
 void backward(Handle& h, const BwdPtrs& t) {
     if (!h.configured) fail("encoder_backward: handle is not configured");
     h.prof_used = 0;
+    // The five bias / scale gradients are only consumed by the caller: their
+    // reductions leave fp32 partials in separate scratch regions and one launch
+    // at the end of the pass finishes them all.  (With per-operator timing on,
+    // each finishes on its own so that its time is attributed to it.)
+    ensure_ws(h, h.ws_need_bwd);
+    h.deferring = !h.profiling;
+    h.ws_cursor = 0;
+    h.deferred.n = 0;
+    struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
     void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
     {
         ProfScope ps(h, "bsb");
@@ -628,6 +665,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         ProfScope ps(h, "bei");
         op_bei(h, D[DXATT], h.lb[DXATT], D[DRESID1], h.lb[DRESID1], t.DX, h.lX);
     }
+    if (h.deferring) launch_colfinish(h.deferred, h.stream);
 }
 
 void unpack_forward(const Handle& h, void* const* p, FwdPtrs& t) {

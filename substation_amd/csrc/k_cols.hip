@@ -98,7 +98,7 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
                                                      long rows_per_block, long nrows) {
     constexpr int NS = ColTraits<KIND>::NS;
     constexpr int NIN = ColIn<KIND>::N;
-    constexpr int U = FAST ? (NIN >= 3 ? 2 : 4) : 1;   // rows in flight per lane
+    constexpr int U = FAST ? 2 : 1;                    // rows in flight per lane
     __shared__ float red[BLOCK][9];          // +1 pad: conflict-free column reads
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lpr = 1 << lpr_log2, rpw = WAVE >> lpr_log2;
@@ -173,27 +173,22 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
     }
 }
 
-struct FinishArgs {
-    half_t* out[3];
-    long ob0, ob1, of;      // output strides of the kept dims (i0, i1) and of the feature
-    int n1;
-};
-
-// Adds the ntc partials of every (sum, kept index, feature): 32 features x 8
-// slices per block, the slices combined through LDS.
-__global__ __launch_bounds__(BLOCK) void k_colfinish(const float* ws, FinishArgs o, int ns, int nbatch,
-                                                     int ntc, int R) {
+// Adds the ntc partials of every (sum, kept index, feature) of up to
+// kMaxFinishJobs operators in one launch: blockIdx.y selects the operator, 32
+// features x 8 slices per block, the slices combined through LDS.
+__global__ __launch_bounds__(BLOCK) void k_colfinish(FinishJobs jobs) {
     __shared__ float red[8][33];
+    const FinishJob& j = jobs.j[blockIdx.y];
     const int fl = threadIdx.x & 31, sl = threadIdx.x >> 5;
     long idx = (long)blockIdx.x * 32 + fl;
-    const bool ok = idx < (long)ns * nbatch * R;
+    const bool ok = idx < (long)j.ns * j.nbatch * j.R;
     int s = 0, f = 0, z = 0;
     float t = 0.f;
     if (ok) {
-        long sz = idx / R; f = (int)(idx - sz * R);
-        s = (int)(sz / nbatch); z = (int)(sz - (long)s * nbatch);
-        const float* p = ws + sz * ntc * R + f;
-        for (int c = sl; c < ntc; c += 8) t += p[(long)c * R];
+        long sz = idx / j.R; f = (int)(idx - sz * j.R);
+        s = (int)(sz / j.nbatch); z = (int)(sz - (long)s * j.nbatch);
+        const float* p = j.ws + sz * j.ntc * j.R + f;
+        for (int c = sl; c < j.ntc; c += 8) t += p[(long)c * j.R];
     }
     red[sl][fl] = t;
     __syncthreads();
@@ -201,7 +196,7 @@ __global__ __launch_bounds__(BLOCK) void k_colfinish(const float* ws, FinishArgs
         float tot = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) tot += red[i][fl];
-        o.out[s][(long)(z / o.n1) * o.ob0 + (long)(z % o.n1) * o.ob1 + (long)f * o.of] = (half_t)tot;
+        j.fo.out[s][(long)(z / j.fo.n1) * j.fo.ob0 + (long)(z % j.fo.n1) * j.fo.ob1 + (long)f * j.fo.of] = (half_t)tot;
     }
 }
 
@@ -222,10 +217,10 @@ inline ColPlan col_plan(const RowSpace& rs) {
     p.nstrips = (chunks + lpr - 1) / lpr;
     long nrows = (long)rs.n2 * rs.n3;
     int rows_per_iter = WPB * (WAVE / lpr);
-    // aim for ~768 blocks in total, at least one 4-row-deep iteration per wave
-    long want_tc = 768 / (p.nstrips * nbatch); if (want_tc < 1) want_tc = 1;
+    // aim for ~2048 blocks in total (8 per CU), at least one 2-row-deep iteration per wave
+    long want_tc = 2048 / (p.nstrips * nbatch); if (want_tc < 1) want_tc = 1;
     long rpb = (nrows + want_tc - 1) / want_tc;
-    if (rpb < 4L * rows_per_iter) rpb = 4L * rows_per_iter;
+    if (rpb < 2L * rows_per_iter) rpb = 2L * rows_per_iter;
     rpb = (rpb + rows_per_iter - 1) / rows_per_iter * rows_per_iter;
     p.rows_per_block = rpb;
     p.ntc = (int)((nrows + rpb - 1) / rpb);
@@ -235,7 +230,7 @@ inline ColPlan col_plan(const RowSpace& rs) {
 
 template <int KIND>
 void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hipStream_t st,
-             const char* what) {
+             const char* what, FinishJobs* defer) {
     constexpr int NS = ColTraits<KIND>::NS;
     if (rs.R <= 0) return;
     if (!ws) fail(std::string(what) + ": no reduction workspace");
@@ -255,10 +250,14 @@ void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hip
         hipLaunchKernelGGL((k_colreduce<KIND, false>), dim3(p.nstrips, p.ntc, nbatch), dim3(BLOCK), 0, st, rs,
                            a, ws, p.lpr_log2, p.rows_per_block, nrows);
     check_launch(what);
-    long n = (long)NS * nbatch * rs.R;
-    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((n + 31) / 32)), dim3(BLOCK), 0, st,
-                       (const float*)ws, fo, NS, nbatch, p.ntc, rs.R);
-    check_launch(what);
+    FinishJob job{ws, fo, NS, nbatch, p.ntc, rs.R};
+    if (defer) {
+        if (defer->n >= kMaxFinishJobs) fail(std::string(what) + ": too many deferred reductions");
+        defer->j[defer->n++] = job;
+    } else {
+        FinishJobs one; one.n = 1; one.j[0] = job;
+        launch_colfinish(one, st);
+    }
 }
 
 // One wave per (i0,i1,i2): sum over i3 and the row.
@@ -287,45 +286,56 @@ __global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, Vie
 
 }  // namespace
 
+void launch_colfinish(const FinishJobs& jobs, hipStream_t st) {
+    if (jobs.n == 0) return;
+    long maxn = 0;
+    for (int i = 0; i < jobs.n; ++i) {
+        long n = (long)jobs.j[i].ns * jobs.j[i].nbatch * jobs.j[i].R;
+        if (n > maxn) maxn = n;
+    }
+    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((maxn + 31) / 32), jobs.n), dim3(BLOCK), 0, st, jobs);
+    check_launch("column-sum finish");
+}
+
 size_t colreduce_ws_floats(const RowSpace& rs, int nsums) {
     ColPlan p = col_plan(rs);
     return (size_t)nsums * rs.n0 * rs.n1 * p.ntc * rs.R;
 }
 
 void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
-                ColOut dbias, float* ws, hipStream_t st) {
+                ColOut dbias, float* ws, hipStream_t st, FinishJobs* defer) {
     ColArgs a{}; a.v[0] = in; a.v[1] = dout; a.v[3] = din; a.v[5] = scale; a.act = 0;
     FinishArgs fo{{dscale.p, dbias.p, nullptr}, 0, 0, 1, 1};
-    run_col<COL_BSB>(rs, a, fo, ws, st, "backward scale-bias");
+    run_col<COL_BSB>(rs, a, fo, ws, st, "backward scale-bias", defer);
 }
 
 void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dlinear, View scale,
                  View din, ColOut dscale, ColOut dbias, ColOut dlinear_bias, float* ws,
-                 hipStream_t st) {
+                 hipStream_t st, FinishJobs* defer) {
     ColArgs a{}; a.v[0] = in; a.v[1] = dout1; a.v[2] = dout2; a.v[3] = din; a.v[4] = dlinear;
     a.v[5] = scale; a.act = 0;
     FinishArgs fo{{dscale.p, dbias.p, dlinear_bias.p}, 0, 0, 1, 1};
-    run_col<COL_EBSB>(rs, a, fo, ws, st, "extended backward scale-bias");
+    run_col<COL_EBSB>(rs, a, fo, ws, st, "extended backward scale-bias", defer);
 }
 
 void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
-                  int act, float* ws, hipStream_t st) {
+                  int act, float* ws, hipStream_t st, FinishJobs* defer) {
     ColArgs a{}; a.v[0] = ddrop; a.v[1] = mask; a.v[2] = lin; a.v[3] = dlinear; a.act = act;
     FinishArgs fo{{dbias.p, nullptr, nullptr}, 0, 0, 1, 1};
-    run_col<COL_BDRLB>(rs, a, fo, ws, st, "backward dropout-activation-bias");
+    run_col<COL_BDRLB>(rs, a, fo, ws, st, "backward dropout-activation-bias", defer);
 }
 
-void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st) {
+void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st, FinishJobs* defer) {
     ColArgs a{}; a.v[0] = datt; a.act = 0;
     FinishArgs fo{{dbo.p, nullptr, nullptr}, 0, 0, 1, 1};
-    run_col<COL_BAOB>(rs, a, fo, ws, st, "backward attention-output bias");
+    run_col<COL_BAOB>(rs, a, fo, ws, st, "backward attention-output bias", defer);
 }
 
 void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, long of, float* ws,
-                   hipStream_t st) {
+                   hipStream_t st, FinishJobs* defer) {
     ColArgs a{}; a.v[0] = d; a.act = 0;
     FinishArgs fo{{out, nullptr, nullptr}, ob0, ob1, of, 1};
-    run_col<COL_BAOB>(rs, a, fo, ws, st, "column sum");
+    run_col<COL_BAOB>(rs, a, fo, ws, st, "column sum", defer);
 }
 
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st) {

@@ -321,9 +321,13 @@ inline unsigned check_rows(const RowSpace& rs, const char* what) {
 #define SUB_ROW_DISPATCH(KERNEL, vpl, fast, ...)                                   \
     do {                                                                           \
         if (fast) {                                                                \
+            /* several rows per wave only while that still leaves >= 16 waves per CU */ \
+            const bool many = nrows >= 256u * 16u * 4u;                            \
             switch (vpl) {                                                         \
-                case 1: SUB_ROW_LAUNCH(KERNEL, 1, 4, true, __VA_ARGS__); break;    \
-                case 2: SUB_ROW_LAUNCH(KERNEL, 2, 2, true, __VA_ARGS__); break;    \
+                case 1: if (many) SUB_ROW_LAUNCH(KERNEL, 1, 4, true, __VA_ARGS__);  \
+                        else SUB_ROW_LAUNCH(KERNEL, 1, 1, true, __VA_ARGS__); break; \
+                case 2: if (many) SUB_ROW_LAUNCH(KERNEL, 2, 2, true, __VA_ARGS__);  \
+                        else SUB_ROW_LAUNCH(KERNEL, 2, 1, true, __VA_ARGS__); break; \
                 case 4: SUB_ROW_LAUNCH(KERNEL, 4, 1, true, __VA_ARGS__); break;    \
                 default: SUB_ROW_LAUNCH(KERNEL, 8, 1, true, __VA_ARGS__); break;   \
             }                                                                      \

@@ -39,18 +39,38 @@ void launch_add(const RowSpace& rs, View a, View b, View out, hipStream_t st);
 struct ColOut {
     half_t* p;   // dense [R]
 };
+// The second stage of a column reduction (adding the per-chunk partials).  It
+// can be deferred: several operators then share one finishing launch, each with
+// its own scratch region.
+struct FinishArgs {
+    half_t* out[3];
+    long ob0, ob1, of;      // output strides of the kept dims (i0, i1) and of the feature
+    int n1;
+};
+struct FinishJob {
+    const float* ws;
+    FinishArgs fo;
+    int ns, nbatch, ntc, R;
+};
+constexpr int kMaxFinishJobs = 6;
+struct FinishJobs {
+    FinishJob j[kMaxFinishJobs];
+    int n = 0;
+};
+void launch_colfinish(const FinishJobs& jobs, hipStream_t st);
 size_t colreduce_ws_floats(const RowSpace& rs, int nsums);
 void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
-                ColOut dbias, float* ws, hipStream_t st);
+                ColOut dbias, float* ws, hipStream_t st, FinishJobs* defer = nullptr);
 void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dlinear, View scale,
                  View din, ColOut dscale, ColOut dbias, ColOut dlinear_bias, float* ws,
-                 hipStream_t st);
+                 hipStream_t st, FinishJobs* defer = nullptr);
 void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
-                  int act, float* ws, hipStream_t st);
-void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st);
+                  int act, float* ws, hipStream_t st, FinishJobs* defer = nullptr);
+void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st,
+                 FinishJobs* defer = nullptr);
 // out[i0,i1,e] = sum over (i2,i3) of d; out strides ob0, ob1 (kept dims) and of.
 void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, long of, float* ws,
-                   hipStream_t st);
+                   hipStream_t st, FinishJobs* defer = nullptr);
 // Row sums: out[row-group] = sum over (n3, R) for each (n0,n1,n2): baib.
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
 
