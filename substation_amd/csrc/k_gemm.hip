@@ -455,8 +455,9 @@ struct DTile {
     }
 };
 
-template <int TM, int TN, bool AKC, bool BKC>
+template <int TM, int TN, bool AKC, bool BKC, int S>
 __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
+    static_assert(S == 2 || S == 3, "two or three LDS stages");
     constexpr int BM = 64 * TM, BN = 64 * TN;
     using TA = DTile<BM, AKC>;
     using TB = DTile<BN, BKC>;
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
     static_assert(4 * STAGE_WAVE <= STAGE, "epilogue staging must fit one stage");
     __shared__ __attribute__((aligned(16))) half_t st0[STAGE];
     __shared__ __attribute__((aligned(16))) half_t st1[STAGE];
-    __shared__ __attribute__((aligned(16))) half_t st2[STAGE];
+    __shared__ __attribute__((aligned(16))) half_t st2[S == 3 ? STAGE : 8];
     constexpr int L = TA::NV + TB::NV;               // loads per thread per tile
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -555,23 +556,36 @@ __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
     // that the fetch below overwrites (it was computed on one step earlier).
 #define SUB_DMA_STEP(cur_, nxt2_)                                                                 \
     do {                                                                                          \
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));                                                \
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(S == 3 ? L : 0));                                   \
         __builtin_amdgcn_s_barrier();                                                             \
         SUB_DMA_ISSUE(nxt2_);                                                                     \
+        /* keep the fetches ahead of the multiply phase: the scheduler must not sink them */      \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
         SUB_DMA_COMPUTE(cur_);                                                                    \
     } while (0)
 
-    SUB_DMA_ISSUE(st0);                // tile 0
-    SUB_DMA_ISSUE(st1);                // tile 1 (or a surplus copy of the last tile)
-    const int ntriples = nkt / 3;
-    for (int p = 0; p < ntriples; ++p) {
-        SUB_DMA_STEP(st0, st2);
-        SUB_DMA_STEP(st1, st0);
-        SUB_DMA_STEP(st2, st1);
+    if (S == 3) {
+        SUB_DMA_ISSUE(st0);                // tile 0
+        SUB_DMA_ISSUE(st1);                // tile 1 (or a surplus copy of the last tile)
+        const int ntriples = nkt / 3;
+        for (int p = 0; p < ntriples; ++p) {
+            SUB_DMA_STEP(st0, st2);
+            SUB_DMA_STEP(st1, st0);
+            SUB_DMA_STEP(st2, st1);
+        }
+        const int rem = nkt - 3 * ntriples;
+        if (rem >= 1) SUB_DMA_STEP(st0, st2);
+        if (rem >= 2) SUB_DMA_STEP(st1, st0);
+    } else {
+        // two stages: the next tile is in flight while the current one is multiplied
+        SUB_DMA_ISSUE(st0);
+        const int npairs = nkt / 2;
+        for (int p = 0; p < npairs; ++p) {
+            SUB_DMA_STEP(st0, st1);
+            SUB_DMA_STEP(st1, st0);
+        }
+        if (nkt & 1) SUB_DMA_STEP(st0, st1);
     }
-    const int rem = nkt - 3 * ntriples;
-    if (rem >= 1) SUB_DMA_STEP(st0, st2);
-    if (rem >= 2) SUB_DMA_STEP(st1, st0);
 #undef SUB_DMA_STEP
 #undef SUB_DMA_COMPUTE
 #undef SUB_DMA_ISSUE
@@ -700,10 +714,16 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     return ok ? 1 : 0;
 }
 
-// Block tile for a problem: 22 = 128x128, 42 = 256x128, 21 = 128x64.
+// Block tile for a problem: 22 = 128x128, 42 = 256x128, 44 = 256x256, 21 = 128x64.
 int pick_tile(const GemmArgs& a, long batch) {
-    (void)batch;
     if (a.N <= 64) return 21;      // head-size wide outputs of the attention products
+    // 256x256 tiles halve the L2->LDS traffic per flop; they pay once the output
+    // alone has enough of them for most of the 256 CUs (asynchronous kernel only:
+    // whole tiles, no split contraction).
+    static const int min44 = [] { const char* e = getenv("SUB_GEMM_MIN44"); return e ? atoi(e) : 192; }();
+    if (a.M % 256 == 0 && a.N % 256 == 0 && a.K1 % BK == 0 && a.splits == 1 &&
+        (long)(a.M / 256) * (a.N / 256) * batch >= min44)
+        return 44;
     return 22;
 }
 
@@ -717,10 +737,11 @@ void launch_mfma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t 
 
 template <int TM, int TN>
 void launch_dma(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
-    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true>), grid, dim3(256), 0, st, a);
-    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false>), grid, dim3(256), 0, st, a);
-    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false>), grid, dim3(256), 0, st, a);
+    constexpr int S = (TM * TN >= 16) ? 2 : 3;      // 256x256 tiles: two 64 KiB stages
+    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true, S>), grid, dim3(256), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false, S>), grid, dim3(256), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true, S>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false, S>), grid, dim3(256), 0, st, a);
 }
 
 template <int TM, int TN, bool DMA_OK>
@@ -786,7 +807,6 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
     int kind = pick_kind(c, akc, bkc);
     if (kind == 1) {
         static const int force = [] { const char* e = getenv("SUB_GEMM_TILE"); return e ? atoi(e) : 0; }();
-        int tile = force ? force : pick_tile(c.a, batch);
         // SUB_GEMM_DMA: -1 never / 1 always use the asynchronous kernel; default: when both
         // operands are k-contiguous and there is at most about one tile per CU, where
         // the register-staged kernel has no second workgroup to hide its waits behind.
@@ -796,8 +816,10 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             c.a.splits = pick_splits(c.a, batch, ws_floats);
             c.a.partial = ws;
         }
+        const int tile = force ? force : pick_tile(c.a, batch);
         const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
-        if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
+        if (tile == 44) launch_mfma<4, 4, true>(c.a, akc, bkc, batch, true, st);
+        else if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
         else if (tile == 21) launch_mfma<2, 1, false>(c.a, akc, bkc, batch, false, st);
         else launch_mfma<2, 2, true>(c.a, akc, bkc, batch, dma, st);
     } else {
