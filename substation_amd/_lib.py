@@ -8,7 +8,8 @@ import os
 from . import layouts as _lay
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, 'lib', 'libsubstation_amd.so')
+#: the in-tree build; SUBSTATION_AMD_LIB names another build of the same sources
+LIB_PATH = os.environ.get('SUBSTATION_AMD_LIB') or os.path.join(HERE, 'lib', 'libsubstation_amd.so')
 
 N_PARAMS, N_FWD, N_BWD = 12, 23, 14
 ABI_VERSION = 1

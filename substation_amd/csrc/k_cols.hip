@@ -39,10 +39,23 @@ __device__ __forceinline__ float gelu_grad(float x) {
 }
 
 template <int KIND> struct ColIn;      // which views are read: count and indices into ColArgs::v
-template <> struct ColIn<COL_BSB> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; };
-template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; };
-template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; };
-template <> struct ColIn<COL_BAOB> { static constexpr int N = 1; static constexpr int idx[4] = {0, 0, 0, 0}; };
+// `nt`: inputs saved by the forward pass, read here for the last time (streamed)
+template <> struct ColIn<COL_BSB> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; static constexpr bool nt[4] = {true, false, false, false}; };
+template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; static constexpr bool nt[4] = {true, false, false, false}; };
+template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; static constexpr bool nt[4] = {false, true, true, false}; };
+template <> struct ColIn<COL_BAOB> { static constexpr int N = 1; static constexpr int idx[4] = {0, 0, 0, 0}; static constexpr bool nt[4] = {false, false, false, false}; };
+
+// Raw 128-bit loads of the inputs of one row chunk (inputs T, T+1, ...).
+template <int KIND, int T>
+__device__ __forceinline__ void col_load_raw(const ColArgs& a, const RowIdx& ix, int e0, int nv,
+                                             h8 (&raw)[ColIn<KIND>::N]) {
+    if constexpr (T < ColIn<KIND>::N) {
+        const View& v = a.v[ColIn<KIND>::idx[T]];
+        raw[T] = (h8)(half_t)0.0f;
+        if (nv) raw[T] = ldg8<ColIn<KIND>::nt[T]>(v.p + view_offset(v, ix) + e0);
+        col_load_raw<KIND, T + 1>(a, ix, e0, nv, raw);
+    }
+}
 
 // One 8-pack of one row: elementwise output (stored to v[3]) and the running sums.
 template <int KIND>
@@ -129,13 +142,12 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
                 r = nvu[u] ? r : row;
                 ix[u].i0 = i0; ix[u].i1 = i1;
                 ix[u].i2 = r / n3; ix[u].i3 = r - ix[u].i2 * n3;
+                if (FAST) {
+                    col_load_raw<KIND, 0>(a, ix[u], e0, nvu[u], raw[u]);
+                } else {
 #pragma unroll
-                for (int t = 0; t < NIN; ++t) {
-                    const View& v = a.v[ColIn<KIND>::idx[t]];
-                    if (FAST) {
-                        raw[u][t] = (h8)(half_t)0.0f;
-                        if (nvu[u]) raw[u][t] = *reinterpret_cast<const h8*>(v.p + view_offset(v, ix[u]) + e0);
-                    } else {
+                    for (int t = 0; t < NIN; ++t) {
+                        const View& v = a.v[ColIn<KIND>::idx[t]];
                         gen[t] = load8(v, view_offset(v, ix[u]), e0, nvu[u]);
                     }
                 }

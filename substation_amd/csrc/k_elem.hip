@@ -64,8 +64,8 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
                 float a = act == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
                 oh[i] = ((bits >> i) & 1u) ? (half_t)a : (half_t)0.0f;
             }
-            st8h<FAST>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
-            st8h<FAST>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
+            st8h<FAST, true>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
+            st8h<FAST, true>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
             st8h<FAST>(out, view_offset(out, c[u].ix), c[u].e0, c[u].nv, oh);
         }
     }

@@ -81,8 +81,8 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
                     a = pin(a);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) d[i] = ((bits >> i) & 1u) ? a[i] : (half_t)0.0f;
-                    st8h<FAST>(alpha, oa, e0, nv, a);
-                    st8h<FAST>(mask, om, e0, nv, mask_h8(bits));
+                    st8h<FAST, true>(alpha, oa, e0, nv, a);
+                    st8h<FAST, true>(mask, om, e0, nv, mask_h8(bits));
                     st8h<FAST>(drop, od, e0, nv, d);
                 }
             }
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fa = ld8<FAST>(alpha, oa, e0, nv), fm = ld8<FAST>(mask, om, e0, nv), fd = ld8<FAST>(ddrop, od, e0, nv);
+                F8 fa = ld8<FAST, true>(alpha, oa, e0, nv), fm = ld8<FAST, true>(mask, om, e0, nv), fd = ld8<FAST>(ddrop, od, e0, nv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     a[r][c][i] = fa.v[i];
@@ -178,8 +178,8 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                     s[r] += x[r][c][i];
                 }
                 if (nv > 0) {
-                    st8h<FAST>(lin, ol, e0, nv, lh);
-                    st8h<FAST>(mask, om, e0, nv, mask_h8(bits[r][c]));
+                    st8h<FAST, true>(lin, ol, e0, nv, lh);
+                    st8h<FAST, true>(mask, om, e0, nv, mask_h8(bits[r][c]));
                 }
             }
         }
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                         n[i] = (half_t)nn;
                         o[i] = (half_t)(nn * fs.v[i] + fb.v[i]);
                     }
-                    st8h<FAST>(diff, od, e0, nv, d);
-                    st8h<FAST>(normed, on, e0, nv, n);
+                    st8h<FAST, true>(diff, od, e0, nv, d);
+                    st8h<FAST, true>(normed, on, e0, nv, n);
                     st8h<FAST>(out, oo, e0, nv, o);
                 }
             }
@@ -252,8 +252,8 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fg = ld8<FAST>(dout, oo, e0, nv), fd = ld8<FAST>(diff, od, e0, nv);
-                F8 fm = ld8<FAST>(mask, om, e0, nv);
+                F8 fg = ld8<FAST>(dout, oo, e0, nv), fd = ld8<FAST, true>(diff, od, e0, nv);
+                F8 fm = ld8<FAST, true>(mask, om, e0, nv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     g[r][c][i] = fg.v[i];

@@ -104,12 +104,29 @@ __device__ __forceinline__ void store8(const View& t, long base, int e0, int nva
 
 // FAST variants: every view is vectorisable and rows are whole 8-packs, so a
 // chunk is either entirely inside the row (nvalid == 8) or entirely outside.
-template <bool FAST>
+// NT marks a streamed tensor: one saved for the backward pass (written now,
+// read again only much later) or read for the last time.  The nontemporal hint
+// keeps it from displacing lines that the next launch is about to read; tensors
+// handed to the next launch and the per-feature vectors every wave re-reads are
+// accessed normally.  (A compile-time choice: a run-time select between the two
+// access forms is folded into one plain access by the optimiser.)
+template <bool NT>
+__device__ __forceinline__ h8 ldg8(const half_t* p) {
+    return NT ? __builtin_nontemporal_load(reinterpret_cast<const h8*>(p))
+              : *reinterpret_cast<const h8*>(p);
+}
+template <bool NT>
+__device__ __forceinline__ void stg8(half_t* p, h8 v) {
+    if (NT) __builtin_nontemporal_store(v, reinterpret_cast<h8*>(p));
+    else *reinterpret_cast<h8*>(p) = v;
+}
+
+template <bool FAST, bool NT = false>
 __device__ __forceinline__ F8 ld8(const View& t, long base, int e0, int nvalid, float fill = 0.f) {
     if (FAST) {
         F8 r;
         if (nvalid) {
-            h8 v = *reinterpret_cast<const h8*>(t.p + base + e0);
+            h8 v = ldg8<NT>(t.p + base + e0);
 #pragma unroll
             for (int i = 0; i < 8; ++i) r.v[i] = (float)v[i];
         } else {
@@ -121,10 +138,10 @@ __device__ __forceinline__ F8 ld8(const View& t, long base, int e0, int nvalid, 
     return load8(t, base, e0, nvalid, fill);
 }
 
-template <bool FAST>
+template <bool FAST, bool NT = false>
 __device__ __forceinline__ void st8h(const View& t, long base, int e0, int nvalid, h8 v) {
     if (FAST) {
-        if (nvalid) *reinterpret_cast<h8*>(t.p + base + e0) = v;
+        if (nvalid) stg8<NT>(t.p + base + e0, v);
     } else {
         store8h(t, base, e0, nvalid, v);
     }

@@ -83,6 +83,9 @@ class Encoder(torch.nn.Module):
         fwd_array = ctypes.c_void_p * n_fwd
         bwd_array = ctypes.c_void_p * n_bwd
 
+        in_shape = tuple(sizes[s] for s in layouts['input'][1])
+        out_shape = tuple(sizes[s] for s in layouts['output'][1])
+
         def _alloc(key, device):
             return [torch.empty(*tuple(sizes[s] for s in layout), device=device,
                                 dtype=module.torch_dtype, requires_grad=False)
@@ -93,9 +96,13 @@ class Encoder(torch.nn.Module):
             def forward(ctx, X, *weights):
                 if not X.is_cuda:
                     raise RuntimeError('Encoder.forward needs a tensor on the GPU')
+                if tuple(X.shape) != in_shape:
+                    raise ValueError(f"X has shape {tuple(X.shape)}, the configured input layout "
+                                     f"{layouts['input'][1]} needs {in_shape}")
                 dev = X.device
                 X = X.contiguous()
-                Y = torch.empty_like(X)
+                # same element count as X, shaped in the output's own dimension order
+                Y = torch.empty(out_shape, device=dev, dtype=X.dtype)
                 forward_intermediate = _alloc('forward_interm', dev)
                 weights_c = [t.contiguous() for t in weights]
                 handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)
@@ -116,7 +123,7 @@ class Encoder(torch.nn.Module):
             def backward(ctx, DY):
                 dev = DY.device
                 DY = DY.contiguous()
-                DX = torch.empty_like(DY)
+                DX = torch.empty(in_shape, device=dev, dtype=DY.dtype)
                 backward_intermediate = _alloc('backward_interm', dev)
                 param_gradients = _alloc('params', dev)
                 handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)

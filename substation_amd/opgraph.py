@@ -1,0 +1,125 @@
+"""Operator graph of the encoder layer: which tensors each launch touches.
+
+Counterpart of the ``OperatorDef`` tables of config_selection/ops.py:61-257 and
+the linear order of config_selection/optimize.py:13-53, reduced to what a
+search over layouts needs: per operator, the named tensors whose layouts decide
+its running time.  Names are those of the layouts pickle
+(pytorch_module/encoder.cu:87-299); ``SB2`` stands for both the layer output and
+the incoming gradient DY, ``X`` for the input and the outgoing gradient DX
+(config_selection/ops.py:265-289 ties them), and every weight gradient has the
+layout of its weight.
+"""
+import itertools
+
+from . import layouts as _lay
+
+#: (operator, pass, tensors) in launch order
+OPERATORS = [
+    ('QKV-fused', 'fwd', ('X', 'WKQV', 'BKQV', 'WKKWQQWVV', 'KKQQVV')),
+    ('aib', 'fwd', ('WKKWQQWVV', 'BKQV', 'KKQQVV')),
+    ('QKT', 'fwd', ('KKQQVV', 'BETA')),
+    ('softmax', 'fwd', ('BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP')),
+    ('gamma', 'fwd', ('KKQQVV', 'ATTN_DROP', 'GAMMA')),
+    ('out', 'fwd', ('WO', 'GAMMA', 'ATT')),
+    ('bdrln1', 'fwd', ('ATT', 'X', 'DROP1MASK', 'LN1DIFF', 'LN1', 'SB1', 'LN1STD')),
+    ('lin1', 'fwd', ('SB1', 'LINW1', 'SB1_LINW1')),
+    ('bad', 'fwd', ('SB1_LINW1', 'LIN1', 'DROP2MASK', 'DROP2')),
+    ('lin2', 'fwd', ('DROP2', 'LINW2', 'DROP2_LINW2')),
+    ('bdrln2', 'fwd', ('DROP2_LINW2', 'SB1', 'LIN2', 'DROP3MASK', 'LN2DIFF', 'LN2', 'SB2', 'LN2STD')),
+    ('bsb', 'bwd', ('LN2', 'SB2', 'DLN2')),
+    ('blnrd1', 'bwd', ('DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
+    ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
+    ('dWlin2', 'bwd', ('DLIN2', 'DROP2', 'LINW2')),
+    ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DLIN1')),
+    ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
+    ('dWlin1', 'bwd', ('DLIN1', 'SB1', 'LINW1')),
+    ('ebsb', 'bwd', ('LN1', 'DRESID2', 'DLIN1_LINW1', 'DLIN2', 'DLN1')),
+    ('blnrd2', 'bwd', ('DLN1', 'LN1STD', 'LN1DIFF', 'DROP1MASK', 'DRESID1', 'DATT')),
+    ('baob', 'bwd', ('DATT',)),
+    ('dWout', 'bwd', ('GAMMA', 'DATT', 'WO')),
+    ('dXout', 'bwd', ('WO', 'DATT', 'DGAMMA')),
+    ('dX1gamma', 'bwd', ('KKQQVV', 'DGAMMA', 'DATTN_DROP')),
+    ('dX2gamma', 'bwd', ('DGAMMA', 'ATTN_DROP', 'DKKQQVV')),
+    ('bs', 'bwd', ('ALPHA', 'ATTN_DROP_MASK', 'DATTN_DROP', 'DBETA')),
+    ('dX1QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
+    ('dX2QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
+    ('dXQKV-fused', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X')),
+    ('dWQKV-fused', 'bwd', ('X', 'DKKQQVV', 'WKQV')),
+    ('baib', 'bwd', ('DKKQQVV', 'BKQV')),
+    ('bei', 'bwd', ('DXATT', 'DRESID1', 'X')),
+]
+OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
+
+#: the 18 contractions (pytorch_module/encoder.cu:90-276; canonical list
+#: tc_profiling/einsum_perms.py:367-394): name -> (A, B, C) operand names, where
+#: KK/QQ/VV and DKK/DQQ/DVV are the Q-slices of the stacked tensors
+EINSUMS = {
+    'QKV-fused': ('X', 'WKQV', 'WKKWQQWVV'),
+    'QKT': ('KK', 'QQ', 'BETA'),
+    'gamma': ('VV', 'ATTN_DROP', 'GAMMA'),
+    'out': ('WO', 'GAMMA', 'ATT'),
+    'lin1': ('SB1', 'LINW1', 'SB1_LINW1'),
+    'lin2': ('DROP2', 'LINW2', 'DROP2_LINW2'),
+    'dXlin2': ('DLIN2', 'LINW2', 'DDROP2'),
+    'dWlin2': ('DLIN2', 'DROP2', 'DLINW2'),
+    'dXlin1': ('DLIN1', 'LINW1', 'DLIN1_LINW1'),
+    'dWlin1': ('DLIN1', 'SB1', 'DLINW1'),
+    'dWout': ('GAMMA', 'DATT', 'DWO'),
+    'dXout': ('WO', 'DATT', 'DGAMMA'),
+    'dX1gamma': ('VV', 'DGAMMA', 'DATTN_DROP'),
+    'dX2gamma': ('DGAMMA', 'ATTN_DROP', 'DVV'),
+    'dX1QKT': ('KK', 'DBETA', 'DQQ'),
+    'dX2QKT': ('QQ', 'DBETA', 'DKK'),
+    'dXQKV-fused': ('WKQV', 'DKKQQVV', 'DXATT'),
+    'dWQKV-fused': ('X', 'DKKQQVV', 'DWKQV'),
+}
+
+
+def tensor_layouts(layouts):
+    """name -> layout string for every tensor a layouts dict names."""
+    return dict(list(layouts['params']) + list(layouts['forward_interm'])
+                + list(layouts['backward_interm'])
+                + [tuple(layouts['input']), tuple(layouts['output'])])
+
+
+def operand_layouts(layouts):
+    """tensor_layouts() plus the derived GEMM operands: weight gradients (layout of
+    the weight) and the Q-slices, with the key/value sequence dim renamed J->K
+    (pytorch_module/encoder.py:339-347)."""
+    t = tensor_layouts(layouts)
+    for k, v in list(layouts['params']):
+        t['D' + k] = v
+    kk, dkk = t['KKQQVV'][1:], t['DKKQQVV'][1:]
+    t['QQ'] = kk
+    t['KK'] = t['VV'] = kk.replace('J', 'K')
+    t['DQQ'] = dkk
+    t['DKK'] = t['DVV'] = dkk.replace('J', 'K')
+    return t
+
+
+def with_layouts(layouts, changes):
+    """A copy of ``layouts`` with ``changes`` (name -> layout) applied."""
+    def sub(pairs):
+        return [(n, changes.get(n, l)) for n, l in pairs]
+    out = dict(layouts)
+    out['input'] = ('X', changes.get('X', layouts['input'][1]))
+    out['output'] = ('SB2', changes.get('SB2', layouts['output'][1]))
+    for key in ('params', 'forward_interm', 'backward_interm'):
+        out[key] = sub(layouts[key])
+    return out
+
+
+def candidate_layouts(name):
+    """Every layout a tensor may take: permutations of its dims, with the stacking
+    dim first where pytorch_module/encoder.py:318-327 requires it."""
+    dims = _lay.CANONICAL[name]
+    if name in _lay._Q_FIRST:
+        rest = dims.replace('Q', '')
+        return ['Q' + ''.join(p) for p in itertools.permutations(rest)]
+    return [''.join(p) for p in itertools.permutations(dims)]
+
+
+def searchable_tensors():
+    """Tensors with more than one possible layout, in pickle order."""
+    names = ['X', 'SB2'] + _lay.PARAM_NAMES + _lay.FWD_NAMES + _lay.BWD_NAMES
+    return [n for n in names if len(candidate_layouts(n)) > 1]

@@ -17,6 +17,8 @@ SEED = 0xC0FFEE
 
 def _layouts(which):
     from substation_amd import layouts as L
+    if isinstance(which, dict):
+        return which
     return L.mi355x_layouts() if which == 'mi355x' else L.reference_layouts(which)
 
 
@@ -106,6 +108,37 @@ def _compare(want, got, tol=1e-2, names=CHECK):
 @pytest.mark.parametrize('p,act', [(0.0, 'relu'), (0.1, 'relu'), (0.1, 'gelu')])
 def test_layer_small(which, p, act):
     want, got = run_layer(2, 32, 2, 64, which, p, act, seed_data=1)
+    _compare(want, got)
+
+
+def _random_layouts(seed, dims=(2, 32, 2, 64)):
+    """A random walk over valid configurations: tensor by tensor, in random order,
+    a random dimension order (stacking dim first where the module requires it),
+    kept when the contractions can still be expressed as GEMMs (the same
+    constraint einsumparser.h:9-55 puts on the reference's layouts)."""
+    from substation_amd import _lib, layouts as L, opgraph as og
+    rng = np.random.default_rng(seed)
+    lay = L.mi355x_layouts()
+    names = og.searchable_tensors()
+    for i in rng.permutation(len(names)):
+        cands = og.candidate_layouts(names[i])
+        for j in rng.permutation(len(cands))[:4]:
+            trial = og.with_layouts(lay, {names[i]: cands[j]})
+            try:
+                _lib.Handle(_lib.make_config(*dims, trial)).close()
+            except _lib.SubstationError:
+                continue
+            lay = trial
+            break
+    return L.validate(lay)
+
+
+@pytest.mark.parametrize('seed', range(6))
+def test_layer_random_layouts(seed):
+    """The kernels take strides at run time: any assignment of dimension orders
+    must give the same numbers (the layout search relies on it)."""
+    lay = _random_layouts(100 + seed)
+    want, got = run_layer(2, 32, 2, 64, lay, 0.1, 'relu' if seed % 2 else 'gelu', seed_data=10 + seed)
     _compare(want, got)
 
 
