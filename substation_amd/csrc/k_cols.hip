@@ -39,10 +39,11 @@ __device__ __forceinline__ float gelu_grad(float x) {
 }
 
 template <int KIND> struct ColIn;      // which views are read: count and indices into ColArgs::v
-// `nt`: inputs saved by the forward pass, read here for the last time (streamed)
+// `nt`: inputs read here for the last time (saved by the forward pass, or the
+// previous launch's output that nothing else consumes): streamed
 template <> struct ColIn<COL_BSB> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; static constexpr bool nt[4] = {true, false, false, false}; };
-template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; static constexpr bool nt[4] = {true, false, false, false}; };
-template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; static constexpr bool nt[4] = {false, true, true, false}; };
+template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; static constexpr bool nt[4] = {true, true, false, true}; };
+template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; static constexpr bool nt[4] = {true, true, true, false}; };
 template <> struct ColIn<COL_BAOB> { static constexpr int N = 1; static constexpr int idx[4] = {0, 0, 0, 0}; static constexpr bool nt[4] = {false, false, false, false}; };
 
 // Raw 128-bit loads of the inputs of one row chunk (inputs T, T+1, ...).
@@ -200,7 +201,14 @@ __global__ __launch_bounds__(BLOCK) void k_colfinish(FinishJobs jobs) {
         long sz = idx / j.R; f = (int)(idx - sz * j.R);
         s = (int)(sz / j.nbatch); z = (int)(sz - (long)s * j.nbatch);
         const float* p = j.ws + sz * j.ntc * j.R + f;
-        for (int c = sl; c < j.ntc; c += 8) t += p[(long)c * j.R];
+        // eight independent loads per round trip instead of one
+        for (int c = sl; c < j.ntc; c += 64) {
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = c + 8 * k < j.ntc ? p[(long)(c + 8 * k) * j.R] : 0.f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) t += v[k];
+        }
     }
     red[sl][fl] = t;
     __syncthreads();

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             c[u] = chunk_of(rs, base + u * stride, nchunks, cpr);
-            fi[u] = ld8<FAST>(in, view_offset(in, c[u].ix), c[u].e0, c[u].nv);
+            fi[u] = ld8<FAST, true>(in, view_offset(in, c[u].ix), c[u].e0, c[u].nv);
             fb[u] = ld8<FAST>(bias, 0, c[u].e0, c[u].nv);
         }
 #pragma unroll

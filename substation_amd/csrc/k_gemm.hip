@@ -636,10 +636,12 @@ __global__ __launch_bounds__(256) void k_gemm_splitk_reduce(GemmArgs g, long nb_
     const long slab = nb_total * (long)g.M * g.N;
     const float* p = g.partial + (bz * g.M + m) * (long)g.N + nq * 4;
     float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s = 0; s < g.splits; ++s) {
-        float4 v = *reinterpret_cast<const float4*>(p + (long)s * slab);
-        t.x += v.x; t.y += v.y; t.z += v.z; t.w += v.w;
-    }
+    float4 v[8];                  // at most 8 splits: all loads in flight at once
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        v[s] = s < g.splits ? *reinterpret_cast<const float4*>(p + (long)s * slab) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) { t.x += v[s].x; t.y += v[s].y; t.z += v[s].z; t.w += v[s].w; }
     long b2 = bz % g.nb2; long tt = bz / g.nb2;
     long b1 = tt % g.nb1; long b0 = tt / g.nb1;
     half_t* c = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2] + (long)m * g.sCM + nq * 4;

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 f = ld8<FAST>(beta, ob, e0, nv, -INFINITY);
+                F8 f = ld8<FAST, true>(beta, ob, e0, nv, -INFINITY);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     x[r][c][i] = f.v[i] * scale;
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fa = ld8<FAST, true>(alpha, oa, e0, nv), fm = ld8<FAST, true>(mask, om, e0, nv), fd = ld8<FAST>(ddrop, od, e0, nv);
+                F8 fa = ld8<FAST, true>(alpha, oa, e0, nv), fm = ld8<FAST, true>(mask, om, e0, nv), fd = ld8<FAST, true>(ddrop, od, e0, nv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     a[r][c][i] = fa.v[i];
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fi = ld8<FAST>(in, oi, e0, nv), fr = ld8<FAST>(resid, orr, e0, nv);
+                F8 fi = ld8<FAST, true>(in, oi, e0, nv), fr = ld8<FAST>(resid, orr, e0, nv);
                 F8 fb = ld8<FAST>(lin_bias, 0, e0, nv);
                 bits[r][c] = nv > 0 ? keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0) : 0u;
                 h8 lh;
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fg = ld8<FAST>(dout, oo, e0, nv), fd = ld8<FAST, true>(diff, od, e0, nv);
+                F8 fg = ld8<FAST, true>(dout, oo, e0, nv), fd = ld8<FAST, true>(diff, od, e0, nv);
                 F8 fm = ld8<FAST, true>(mask, om, e0, nv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
