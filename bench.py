@@ -66,6 +66,9 @@ def algorithmic_work(B, L, H, E):
         'bsb': ('hbm', 3 * bji * 2), 'ebsb': ('hbm', 5 * bji * 2), 'baob': ('hbm', bji * 2),
         'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', 4 * bju * 2), 'bdrlb': ('hbm', 4 * bju * 2),
         'baib': ('hbm', q * 2),
+        # single-launch forms: the scaled gradient is written but not read back
+        # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
+        'bsb+blnrd1': ('hbm', 7 * bji * 2), 'ebsb+blnrd2+baob': ('hbm', 9 * bji * 2),
     }
     tok = B * L
     proj = (2 * tok * 3 * E * E, 2 * (tok * E + 3 * E * E + 3 * tok * E))
@@ -181,6 +184,9 @@ def main():
     ap.add_argument('--profile-steps', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--per-op', action='store_true', help='print the per-operator table to stderr')
+    ap.add_argument('--option', action='append', default=[], metavar='ID=VALUE',
+                    help='library option to set (sub_set_option), e.g. 2=0 runs the LayerNorm backward '
+                         'as separate launches')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE readings')
@@ -197,6 +203,9 @@ def main():
     torch.cuda.set_device(0)
     cfg = CONFIGS[args.config]
     enc, X, DY = make_encoder(cfg, args.layouts)
+    for item in args.option:
+        k, v = item.split('=')
+        enc._handle.set_option(int(k), int(v))
 
     params = list(enc.parameters())
 

@@ -116,6 +116,15 @@ const char* sub_last_error(void);
  * DXATT, which only they consume, are left unwritten.  Set to 0 to materialise
  * every intermediate exactly as pytorch_module/encoder.cu:87-299 does. */
 #define SUB_OPT_FUSE_EPILOGUES 1
+/* SUB_OPT_FUSE_LN_BACKWARD (default 1): run BackwardScaleBias +
+ * BackwardLayerNormResidualDropout (encoder.cu:160-166) as one launch, and
+ * ExtendedBackwardScaleBias + BackwardLayerNormResidualDropout +
+ * BackwardAttnOutBias (encoder.cu:196-212) as another, where the embedding size
+ * (<= 1024) and the layouts (feature dim contiguous) allow it.  Every tensor the
+ * separate kernels write is still written, from the same fp16-rounded
+ * intermediates; the bias / scale gradients are summed in a different order
+ * (fp32), so results can differ from the separate launches in the last bit. */
+#define SUB_OPT_FUSE_LN_BACKWARD 2
 int sub_set_option(void* handle, int option, int value);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same

@@ -15,6 +15,7 @@ N_PARAMS, N_FWD, N_BWD = 12, 23, 14
 ABI_VERSION = 1
 ACTIVATIONS = {'relu': 0, 'gelu': 1}
 OPT_FUSE_EPILOGUES = 1
+OPT_FUSE_LN_BACKWARD = 2
 
 
 class SubConfig(ctypes.Structure):

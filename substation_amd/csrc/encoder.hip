@@ -178,6 +178,7 @@ struct Handle {
     size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
     bool fuse_epilogues = true;
+    bool fuse_ln_backward = true;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -214,6 +215,7 @@ struct ProfScope {
         hip_check(hipEventRecord(e->a, h.stream), "hipEventRecord");
     }
     ~ProfScope() { if (e) (void)hipEventRecord(e->b, h.stream); }
+    void cancel() { if (e) { --h.prof_used; e = nullptr; } }     // nothing was launched
 };
 
 void ensure_ws(Handle& h, size_t floats) {
@@ -354,6 +356,11 @@ void configure(Handle& h, const sub_config* c) {
         h.ws_need_bwd = colreduce_ws_floats(si.rs, 2) + colreduce_ws_floats(si.rs, 3) +
                         colreduce_ws_floats(su.rs, 1) + colreduce_ws_floats(si.rs, 1) +
                         (baib > baib2 ? baib : baib2) + 6 * 64;
+        // the fused LayerNorm-backward launches replace four of those reductions;
+        // size for whichever set is larger
+        size_t fused = lnbwd_ws_floats(si.rs, false) + lnbwd_ws_floats(si.rs, true) +
+                       colreduce_ws_floats(su.rs, 1) + (baib > baib2 ? baib : baib2) + 6 * 64;
+        if (fused > h.ws_need_bwd) h.ws_need_bwd = fused;
     }
     h.gws_need = 0;
     for (int i = 0; i < G_COUNT; ++i) {
@@ -476,6 +483,34 @@ void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 1));
     launch_baob(sp.rs, make_view(datt, l, sp), ColOut{(half_t*)dbo}, ws, h.stream, defer_of(h));
+}
+
+// bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
+// false, having done nothing, when the shape or the layouts rule the fused
+// kernel out; the caller then runs the separate operators.
+bool op_lnbwd(Handle& h, bool ext, const void* in, const Layout& lin_, const void* scale, const void* d1,
+              const Layout& l1, const void* d2, const Layout& l2, const void* dlinear, const Layout& ldl,
+              const void* istd, const Layout& listd, const void* diff, const Layout& ldiff,
+              const void* mask, const Layout& lmask, void* g, const Layout& lg, void* d_ln_in,
+              const Layout& lo1, void* d_drop_in, const Layout& lo2, void* dscale, void* dbias,
+              void* dlinear_bias, void* dout_bias) {
+    Space sp = make_space(h.sz, {dB, dJ}, dI);
+    LnBwdArgs a;
+    a.in = make_view(in, lin_, sp); a.d1 = make_view(d1, l1, sp);
+    a.d2 = ext ? make_view(d2, l2, sp) : a.d1;
+    a.dlinear = ext ? make_view(dlinear, ldl, sp) : a.d1;
+    a.diff = make_view(diff, ldiff, sp); a.mask = make_view(mask, lmask, sp);
+    a.istd = make_view(istd, listd, sp);
+    a.g = make_view(g, lg, sp); a.d_ln_in = make_view(d_ln_in, lo1, sp);
+    a.d_drop_in = make_view(d_drop_in, lo2, sp);
+    flatten(sp.rs, {&a.in, &a.d1, &a.d2, &a.dlinear, &a.diff, &a.mask, &a.istd, &a.g, &a.d_ln_in,
+                    &a.d_drop_in});
+    a.scale = vector_view(scale, sp.rs.R);
+    if (!lnbwd_supported(sp.rs, a, ext)) return false;
+    float* ws = take_ws(h, lnbwd_ws_floats(sp.rs, ext));
+    half_t* sums[4] = {(half_t*)dscale, (half_t*)dbias, (half_t*)dlinear_bias, (half_t*)dout_bias};
+    launch_lnbwd(sp.rs, a, ext, sums, ws, h.stream, defer_of(h));
+    return true;
 }
 
 // out[q,p,h,b,j] = in[q,p,h,b,j] + bias[q,p,h].  The row dim is the innermost
@@ -603,14 +638,25 @@ void backward(Handle& h, const BwdPtrs& t) {
     h.deferred.n = 0;
     struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
     void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
-    {
-        ProfScope ps(h, "bsb");
-        op_bsb(h, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, D[DLN2], h.lb[DLN2], DW[S2], DW[B2]);
+    bool fused = false;
+    if (h.fuse_ln_backward) {
+        ProfScope ps(h, "bsb+blnrd1");
+        fused = op_lnbwd(h, false, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, nullptr, h.lY, nullptr, h.lY,
+                         F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF], F[DROP3MASK], h.lf[DROP3MASK],
+                         D[DLN2], h.lb[DLN2], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2],
+                         DW[S2], DW[B2], nullptr, nullptr);
+        if (!fused) ps.cancel();
     }
-    {
-        ProfScope ps(h, "blnrd1");
-        op_blnrd(h, D[DLN2], h.lb[DLN2], F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF],
-                 F[DROP3MASK], h.lf[DROP3MASK], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2]);
+    if (!fused) {
+        {
+            ProfScope ps(h, "bsb");
+            op_bsb(h, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, D[DLN2], h.lb[DLN2], DW[S2], DW[B2]);
+        }
+        {
+            ProfScope ps(h, "blnrd1");
+            op_blnrd(h, D[DLN2], h.lb[DLN2], F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF],
+                     F[DROP3MASK], h.lf[DROP3MASK], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2]);
+        }
     }
     run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
     run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
@@ -621,19 +667,30 @@ void backward(Handle& h, const BwdPtrs& t) {
     }
     run_gemm(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1");
     run_gemm(h, G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1");
-    {
-        ProfScope ps(h, "ebsb");
-        op_ebsb(h, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
-                h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], D[DLN1], h.lb[DLN1], DW[S1], DW[B1], DW[LINB2]);
+    fused = false;
+    if (h.fuse_ln_backward) {
+        ProfScope ps(h, "ebsb+blnrd2+baob");
+        fused = op_lnbwd(h, true, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
+                         h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], F[LN1STD], h.lf[LN1STD], F[LN1DIFF],
+                         h.lf[LN1DIFF], F[DROP1MASK], h.lf[DROP1MASK], D[DLN1], h.lb[DLN1], D[DRESID1],
+                         h.lb[DRESID1], D[DATT], h.lb[DATT], DW[S1], DW[B1], DW[LINB2], DW[BO]);
+        if (!fused) ps.cancel();
     }
-    {
-        ProfScope ps(h, "blnrd2");
-        op_blnrd(h, D[DLN1], h.lb[DLN1], F[LN1STD], h.lf[LN1STD], F[LN1DIFF], h.lf[LN1DIFF],
-                 F[DROP1MASK], h.lf[DROP1MASK], D[DRESID1], h.lb[DRESID1], D[DATT], h.lb[DATT]);
-    }
-    {
-        ProfScope ps(h, "baob");
-        op_baob(h, D[DATT], h.lb[DATT], DW[BO]);
+    if (!fused) {
+        {
+            ProfScope ps(h, "ebsb");
+            op_ebsb(h, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
+                    h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], D[DLN1], h.lb[DLN1], DW[S1], DW[B1], DW[LINB2]);
+        }
+        {
+            ProfScope ps(h, "blnrd2");
+            op_blnrd(h, D[DLN1], h.lb[DLN1], F[LN1STD], h.lf[LN1STD], F[LN1DIFF], h.lf[LN1DIFF],
+                     F[DROP1MASK], h.lf[DROP1MASK], D[DRESID1], h.lb[DRESID1], D[DATT], h.lb[DATT]);
+        }
+        {
+            ProfScope ps(h, "baob");
+            op_baob(h, D[DATT], h.lb[DATT], DW[BO]);
+        }
     }
     run_gemm(h, G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout");
     run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
@@ -816,6 +873,7 @@ int sub_set_option(void* handle, int option, int value) {
     return guarded([&] {
         Handle& h = as_handle(handle);
         if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
+        else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
         else fail("sub_set_option: unknown option");
     });
 }

@@ -1,0 +1,188 @@
+// The backward pass around one LayerNorm in a single launch.
+//
+// The reference runs it as two or three kernels that hand a [B,J,I] tensor to
+// each other through memory (pytorch_module/encoder.cu:160-166 and 196-212):
+//   BackwardScaleBias            (block_bsb_ebsb.cuh:178-216)   G = DOUT * gamma, d gamma, d beta
+//     or ExtendedBackwardScaleBias (block_bsb_ebsb.cuh:376-420) G = (D1 + D2) * gamma, ..., d linear-bias
+//   BackwardLayerNormResidualDropout (block_blnrd.cuh:203-259)  from G: d(LN input), d(dropout input)
+//   BackwardAttnOutBias          (block_baob.cuh:79-97)         column sum of d(dropout input)
+// Every one of them works on whole rows of I features, so one wave can take a
+// row through all the steps while it is in registers: G is rounded to fp16 and
+// stored exactly as the separate kernels would, the later steps start from the
+// rounded value as they do there, and the column sums accumulate per lane over
+// the rows the wave visits.  Waves of a block combine their sums
+// through LDS into one fp32 partial row per block; the shared finishing launch
+// adds the partial rows.
+#include "sub_ops.hpp"
+
+namespace sub {
+
+namespace {
+
+constexpr int LN_BLOCK = 512;
+constexpr int LN_WPB = LN_BLOCK / WAVE;
+
+// VPL: 128-bit packs per lane and row (row length <= VPL * 512).  EXT: the
+// extended form (two incoming gradients, linear-bias and output-bias sums).
+template <int VPL, bool EXT>
+__global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, float* ws, unsigned nrows) {
+    constexpr int NS = EXT ? 4 : 2;
+    __shared__ float red[LN_WPB][VPL * WAVE * 8];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float invn = 1.0f / (float)rs.R;
+    float acc[NS][VPL][8];
+#pragma unroll
+    for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int c = 0; c < VPL; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[s][c][i] = 0.f;
+    int nv[VPL];
+    F8 fsc[VPL];
+#pragma unroll
+    for (int c = 0; c < VPL; ++c) {
+        const int e0 = (c * WAVE + lane) * 8;
+        nv[c] = e0 < rs.R ? 8 : 0;                 // rows are whole 8-packs here
+        fsc[c] = ld8<true>(a.scale, 0, e0, nv[c]);
+    }
+    for (unsigned row = blockIdx.x * LN_WPB + wave; row < nrows; row += gridDim.x * LN_WPB) {
+        const RowIdx ix = row_index(rs, row);
+        const long oin = view_offset(a.in, ix), o1 = view_offset(a.d1, ix), odf = view_offset(a.diff, ix),
+                   omk = view_offset(a.mask, ix);
+        const long o2 = EXT ? view_offset(a.d2, ix) : 0, odl = EXT ? view_offset(a.dlinear, ix) : 0;
+        const float is = (float)a.istd.p[view_offset(a.istd, ix)];
+        h8 rin[VPL], rd1[VPL], rd2[VPL], rdl[VPL], rdf[VPL], rmk[VPL];
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            const int e0 = (c * WAVE + lane) * 8;
+            rin[c] = rd1[c] = rd2[c] = rdl[c] = rdf[c] = rmk[c] = (h8)(half_t)0.0f;
+            if (nv[c]) {
+                rin[c] = ldg8<true>(a.in.p + oin + e0);          // saved by the forward pass
+                // the incoming gradient of the plain form is the caller's tensor;
+                // those of the extended form are intermediates on their last use
+                rd1[c] = ldg8<EXT>(a.d1.p + o1 + e0);
+                if (EXT) {
+                    rd2[c] = ldg8<true>(a.d2.p + o2 + e0);
+                    rdl[c] = ldg8<true>(a.dlinear.p + odl + e0);
+                }
+                rdf[c] = ldg8<true>(a.diff.p + odf + e0);
+                rmk[c] = ldg8<true>(a.mask.p + omk + e0);
+            }
+        }
+        float g[VPL][8], df[VPL][8];
+        float s1 = 0.f, s2 = 0.f;
+        const long og = view_offset(a.g, ix);
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            const int e0 = (c * WAVE + lane) * 8;
+            h8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float d = EXT ? (float)rd1[c][i] + (float)rd2[c][i] : (float)rd1[c][i];
+                o[i] = (half_t)(d * fsc[c].v[i]);
+                acc[0][c][i] += d * (float)rin[c][i];
+                acc[1][c][i] += d;
+                if (EXT) acc[2][c][i] += (float)rdl[c][i];
+            }
+            o = pin(o);
+            if (nv[c]) stg8<true>(a.g.p + og + e0, o);           // nothing reads G again
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                g[c][i] = (float)o[i];
+                df[c][i] = (float)rdf[c][i];
+                s1 += g[c][i];
+                s2 = __fmaf_rn(g[c][i], df[c][i], s2);
+            }
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        const float c1 = s1 * is * invn;
+        const float c2 = s2 * is * is * is * invn;
+        const long oa = view_offset(a.d_ln_in, ix), ob = view_offset(a.d_drop_in, ix);
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            const int e0 = (c * WAVE + lane) * 8;
+            if (!nv[c]) continue;
+            h8 x, y;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = (half_t)ln_bwd_value(g[c][i], df[c][i], is, c1, c2);
+            x = pin(x);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                y[i] = rmk[c][i] != (half_t)0.0f ? x[i] : (half_t)0.0f;
+                if (EXT) acc[3][c][i] += (float)y[i];
+            }
+            stg8<false>(a.d_ln_in.p + oa + e0, x);
+            stg8<false>(a.d_drop_in.p + ob + e0, y);
+        }
+    }
+    // One partial row per block and sum: ws[(s * gridDim.x + block) * R + feature].
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            float* dst = &red[wave][(c * WAVE + lane) * 8];
+            *reinterpret_cast<float4*>(dst) = make_float4(acc[s][c][0], acc[s][c][1], acc[s][c][2], acc[s][c][3]);
+            *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[s][c][4], acc[s][c][5], acc[s][c][6], acc[s][c][7]);
+        }
+        __syncthreads();
+        for (int f = threadIdx.x; f < rs.R; f += LN_BLOCK) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < LN_WPB; ++w) t += red[w][f];
+            ws[((long)s * gridDim.x + blockIdx.x) * rs.R + f] = t;
+        }
+    }
+}
+
+inline int lnbwd_blocks(long nrows) {
+    // two rows per wave where there are enough rows; at most 2048 waves
+    long blocks = (nrows + 2L * LN_WPB - 1) / (2L * LN_WPB);
+    if (blocks < 1) blocks = 1;
+    if (blocks > 256) blocks = 256;
+    return (int)blocks;
+}
+
+}  // namespace
+
+bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext) {
+    if (rs.R <= 0 || rs.R > 1024 || rs.R % 8 != 0) return false;
+    if (rs.rows() <= 0 || rs.rows() >= (1L << 31)) return false;
+    bool ok = a.in.vec && a.d1.vec && a.diff.vec && a.mask.vec && a.g.vec && a.d_ln_in.vec && a.d_drop_in.vec &&
+              a.scale.vec;
+    if (ext) ok = ok && a.d2.vec && a.dlinear.vec;
+    return ok;
+}
+
+size_t lnbwd_ws_floats(const RowSpace& rs, bool ext) {
+    return (size_t)(ext ? 4 : 2) * lnbwd_blocks(rs.rows()) * rs.R;
+}
+
+void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* const sums[4], float* ws,
+                  hipStream_t st, FinishJobs* defer) {
+    if (!lnbwd_supported(rs, a, ext)) fail("fused LayerNorm backward: unsupported shape or layout");
+    if (!ws) fail("fused LayerNorm backward: no reduction workspace");
+    const unsigned nrows = (unsigned)rs.rows();
+    const int blocks = lnbwd_blocks(nrows);
+    const int vpl = rs.R <= 512 ? 1 : 2;
+    if (ext) {
+        if (vpl == 1) hipLaunchKernelGGL((k_lnbwd<1, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+        else hipLaunchKernelGGL((k_lnbwd<2, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+    } else {
+        if (vpl == 1) hipLaunchKernelGGL((k_lnbwd<1, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+        else hipLaunchKernelGGL((k_lnbwd<2, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+    }
+    check_launch("fused LayerNorm backward");
+    FinishArgs fo{{sums[0], sums[1], sums[2], sums[3]}, 0, 0, 1, 1};
+    FinishJob job{ws, fo, ext ? 4 : 2, 1, blocks, rs.R};
+    if (defer) {
+        if (defer->n >= kMaxFinishJobs) fail("fused LayerNorm backward: too many deferred reductions");
+        defer->j[defer->n++] = job;
+    } else {
+        FinishJobs one; one.n = 1; one.j[0] = job;
+        launch_colfinish(one, st);
+    }
+}
+
+}  // namespace sub

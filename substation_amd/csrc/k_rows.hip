@@ -260,7 +260,7 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
                     df[r][c][i] = fd.v[i];
                     mk[r][c][i] = (half_t)fm.v[i];
                     s1[r] += g[r][c][i];
-                    s2[r] += g[r][c][i] * df[r][c][i];
+                    s2[r] = __fmaf_rn(g[r][c][i], df[r][c][i], s2[r]);
                 }
             }
         }
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
                 if (nv > 0) {
                     h8 a, b;
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) a[i] = (half_t)(g[r][c][i] * is[r] - c1 - df[r][c][i] * c2);
+                    for (int i = 0; i < 8; ++i) a[i] = (half_t)ln_bwd_value(g[r][c][i], df[r][c][i], is[r], c1, c2);
                     a = pin(a);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) b[i] = mk[r][c][i] != (half_t)0.0f ? a[i] : (half_t)0.0f;

@@ -147,6 +147,12 @@ __device__ __forceinline__ void st8h(const View& t, long base, int e0, int nvali
     }
 }
 
+// d(LN input) of one element: g * istd - c1 - diff * c2, with the contraction
+// into FMAs spelled out so that every kernel that evaluates it rounds alike.
+__device__ __forceinline__ float ln_bwd_value(float g, float diff, float istd, float c1, float c2) {
+    return __fmaf_rn(-diff, c2, __fmaf_rn(g, istd, -c1));
+}
+
 // ---- wave64 reductions ------------------------------------------------------
 // Two quad permutes, two row mirrors (DPP), then the four row totals are read
 // with v_readlane and combined; the result is uniform across the wave.

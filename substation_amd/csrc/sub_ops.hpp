@@ -43,7 +43,7 @@ struct ColOut {
 // can be deferred: several operators then share one finishing launch, each with
 // its own scratch region.
 struct FinishArgs {
-    half_t* out[3];
+    half_t* out[4];
     long ob0, ob1, of;      // output strides of the kept dims (i0, i1) and of the feature
     int n1;
 };
@@ -71,6 +71,18 @@ void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream
 // out[i0,i1,e] = sum over (i2,i3) of d; out strides ob0, ob1 (kept dims) and of.
 void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, long of, float* ws,
                    hipStream_t st, FinishJobs* defer = nullptr);
+// The backward pass around one LayerNorm in one launch: the scale/bias gradients
+// (and, extended, the linear-bias and output-bias gradients) with G = (d1 [+ d2])
+// * scale, then the LayerNorm and dropout backward from G.  sums = {dscale, dbias,
+// dlinear_bias, d_output_bias}; the last two only in the extended form.
+struct LnBwdArgs {
+    View in, d1, d2, dlinear, diff, mask, istd, scale;     // inputs (d2, dlinear: extended form)
+    View g, d_ln_in, d_drop_in;                            // outputs
+};
+bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext);
+size_t lnbwd_ws_floats(const RowSpace& rs, bool ext);
+void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* const sums[4], float* ws,
+                  hipStream_t st, FinishJobs* defer = nullptr);
 // Row sums: out[row-group] = sum over (n3, R) for each (n0,n1,n2): baib.
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
 

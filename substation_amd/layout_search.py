@@ -180,17 +180,19 @@ class LayoutSearch:
         self._last_say = time.monotonic()
 
     # -- table ------------------------------------------------------------- #
-    #: operators the library folds into a contraction's epilogue when the layouts
-    #: allow it: whether they run depends on that contraction's tensors too, and
-    #: a run without them enters 0 s
-    FOLDED = {'aib': 'QKV-fused', 'bei': 'dXQKV-fused'}
-
-    @classmethod
-    def key_tensors(cls, op):
-        tensors = _og.OP_TENSORS[op]
-        if op in cls.FOLDED:
-            tensors = tensors + tuple(n for n in _og.OP_TENSORS[cls.FOLDED[op]] if n not in tensors)
-        return tensors
+    @staticmethod
+    def key_tensors(op):
+        """Tensors whose layouts decide an operator's time: its own, and for
+        launches that can stand in for one another those of the whole group
+        (which of them run depends on all of them; the ones that do not run
+        enter 0 s)."""
+        for group in _og.ALTERNATIVES:
+            if op in group:
+                seen = []
+                for member in group:
+                    seen += [n for n in _og.OP_TENSORS[member] if n not in seen]
+                return tuple(seen)
+        return _og.OP_TENSORS[op]
 
     @classmethod
     def _keys(cls, layouts):
@@ -203,7 +205,7 @@ class LayoutSearch:
             raise KeyError(f'timed operators missing from the operator graph: {sorted(unknown)}')
         t = _og.tensor_layouts(layouts)
         for op, k in self._keys(layouts).items():
-            if op not in times and op not in self.FOLDED:
+            if op not in times and not any(op in g for g in _og.ALTERNATIVES):
                 raise KeyError(f'operator {op} was not timed')
             sec = times.get(op, 0.0)
             new = k not in self.table
@@ -221,7 +223,9 @@ class LayoutSearch:
             return sum(self.table[k] for k in keys.values())
         if not self.timer.usable(layouts):
             return float('inf')
-        self._enter(layouts, self.timer.measure(layouts))
+        times = self.timer.measure(layouts)
+        self._timed = set(times)
+        self._enter(layouts, times)
         self.evaluations += 1
         if time.monotonic() - self._last_say > 20:
             self._say(f'  ... {self.evaluations} runs, {len(self.table)} table entries')
@@ -348,7 +352,7 @@ class LayoutSearch:
         keys = self._keys(layouts)
         for op, which, tensors in _og.OPERATORS:
             sec = self.table.get(keys[op])
-            if sec is None or (op in self.FOLDED and sec == 0.0):
+            if sec is None or (sec == 0.0 and op not in self._timed):
                 continue
             best = min(v for (o, _), v in self.table.items() if o == op)
             tot[which] += sec

@@ -26,6 +26,7 @@ OPERATORS = [
     ('bad', 'fwd', ('SB1_LINW1', 'LIN1', 'DROP2MASK', 'DROP2')),
     ('lin2', 'fwd', ('DROP2', 'LINW2', 'DROP2_LINW2')),
     ('bdrln2', 'fwd', ('DROP2_LINW2', 'SB1', 'LIN2', 'DROP3MASK', 'LN2DIFF', 'LN2', 'SB2', 'LN2STD')),
+    ('bsb+blnrd1', 'bwd', ('LN2', 'SB2', 'DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
     ('bsb', 'bwd', ('LN2', 'SB2', 'DLN2')),
     ('blnrd1', 'bwd', ('DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
     ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
@@ -33,6 +34,8 @@ OPERATORS = [
     ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DLIN1')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
     ('dWlin1', 'bwd', ('DLIN1', 'SB1', 'LINW1')),
+    ('ebsb+blnrd2+baob', 'bwd', ('LN1', 'DRESID2', 'DLIN1_LINW1', 'DLIN2', 'DLN1', 'LN1STD', 'LN1DIFF',
+                                 'DROP1MASK', 'DRESID1', 'DATT')),
     ('ebsb', 'bwd', ('LN1', 'DRESID2', 'DLIN1_LINW1', 'DLIN2', 'DLN1')),
     ('blnrd2', 'bwd', ('DLN1', 'LN1STD', 'LN1DIFF', 'DROP1MASK', 'DRESID1', 'DATT')),
     ('baob', 'bwd', ('DATT',)),
@@ -49,6 +52,17 @@ OPERATORS = [
     ('bei', 'bwd', ('DXATT', 'DRESID1', 'X')),
 ]
 OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
+
+#: Launches that stand for one another: where the sizes and layouts allow it the
+#: library runs the first entry of a group in place of the others (an addend
+#: folded into a contraction's epilogue, several row kernels in one launch), so
+#: which of them run depends on the layouts of the whole group's tensors.
+ALTERNATIVES = [
+    ('QKV-fused', 'aib'),
+    ('dXQKV-fused', 'bei'),
+    ('bsb+blnrd1', 'bsb', 'blnrd1'),
+    ('ebsb+blnrd2+baob', 'ebsb', 'blnrd2', 'baob'),
+]
 
 #: the 18 contractions (pytorch_module/encoder.cu:90-276; canonical list
 #: tc_profiling/einsum_perms.py:367-394): name -> (A, B, C) operand names, where
