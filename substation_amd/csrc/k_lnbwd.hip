@@ -22,6 +22,41 @@ namespace {
 constexpr int LN_BLOCK = 512;
 constexpr int LN_WPB = LN_BLOCK / WAVE;
 
+// The inputs of one row, as loaded (one 128-bit pack per lane and chunk).
+template <int VPL>
+struct LnRow {
+    h8 in[VPL], d1[VPL], d2[VPL], dl[VPL], df[VPL], mk[VPL];
+    float is;
+    RowIdx ix;
+};
+
+template <int VPL, bool EXT>
+__device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs& a, unsigned row, int lane,
+                                            const int (&nv)[VPL], LnRow<VPL>& r) {
+    r.ix = row_index(rs, row);
+    const long oin = view_offset(a.in, r.ix), o1 = view_offset(a.d1, r.ix), odf = view_offset(a.diff, r.ix),
+               omk = view_offset(a.mask, r.ix);
+    const long o2 = EXT ? view_offset(a.d2, r.ix) : 0, odl = EXT ? view_offset(a.dlinear, r.ix) : 0;
+    r.is = (float)a.istd.p[view_offset(a.istd, r.ix)];
+#pragma unroll
+    for (int c = 0; c < VPL; ++c) {
+        const int e0 = (c * WAVE + lane) * 8;
+        r.in[c] = r.d1[c] = r.d2[c] = r.dl[c] = r.df[c] = r.mk[c] = (h8)(half_t)0.0f;
+        if (nv[c]) {
+            r.in[c] = ldg8<true>(a.in.p + oin + e0);          // saved by the forward pass
+            // the incoming gradient of the plain form is the caller's tensor;
+            // those of the extended form are intermediates on their last use
+            r.d1[c] = ldg8<EXT>(a.d1.p + o1 + e0);
+            if (EXT) {
+                r.d2[c] = ldg8<true>(a.d2.p + o2 + e0);
+                r.dl[c] = ldg8<true>(a.dlinear.p + odl + e0);
+            }
+            r.df[c] = ldg8<true>(a.diff.p + odf + e0);
+            r.mk[c] = ldg8<true>(a.mask.p + omk + e0);
+        }
+    }
+}
+
 // VPL: 128-bit packs per lane and row (row length <= VPL * 512).  EXT: the
 // extended form (two incoming gradients, linear-bias and output-bias sums).
 template <int VPL, bool EXT>
@@ -45,51 +80,36 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
         nv[c] = e0 < rs.R ? 8 : 0;                 // rows are whole 8-packs here
         fsc[c] = ld8<true>(a.scale, 0, e0, nv[c]);
     }
-    for (unsigned row = blockIdx.x * LN_WPB + wave; row < nrows; row += gridDim.x * LN_WPB) {
-        const RowIdx ix = row_index(rs, row);
-        const long oin = view_offset(a.in, ix), o1 = view_offset(a.d1, ix), odf = view_offset(a.diff, ix),
-                   omk = view_offset(a.mask, ix);
-        const long o2 = EXT ? view_offset(a.d2, ix) : 0, odl = EXT ? view_offset(a.dlinear, ix) : 0;
-        const float is = (float)a.istd.p[view_offset(a.istd, ix)];
-        h8 rin[VPL], rd1[VPL], rd2[VPL], rdl[VPL], rdf[VPL], rmk[VPL];
-#pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            const int e0 = (c * WAVE + lane) * 8;
-            rin[c] = rd1[c] = rd2[c] = rdl[c] = rdf[c] = rmk[c] = (h8)(half_t)0.0f;
-            if (nv[c]) {
-                rin[c] = ldg8<true>(a.in.p + oin + e0);          // saved by the forward pass
-                // the incoming gradient of the plain form is the caller's tensor;
-                // those of the extended form are intermediates on their last use
-                rd1[c] = ldg8<EXT>(a.d1.p + o1 + e0);
-                if (EXT) {
-                    rd2[c] = ldg8<true>(a.d2.p + o2 + e0);
-                    rdl[c] = ldg8<true>(a.dlinear.p + odl + e0);
-                }
-                rdf[c] = ldg8<true>(a.diff.p + odf + e0);
-                rmk[c] = ldg8<true>(a.mask.p + omk + e0);
-            }
-        }
+    const unsigned stride = gridDim.x * LN_WPB;
+    unsigned row = blockIdx.x * LN_WPB + wave;
+    LnRow<VPL> cur, nxt;
+    if (row < nrows) ln_load_row<VPL, EXT>(rs, a, row, lane, nv, cur);
+    for (; row < nrows; row += stride) {
+        // the next row's loads are in flight while this one is worked on
+        const bool more = row + stride < nrows;
+        if (more) ln_load_row<VPL, EXT>(rs, a, row + stride, lane, nv, nxt);
         float g[VPL][8], df[VPL][8];
         float s1 = 0.f, s2 = 0.f;
-        const long og = view_offset(a.g, ix);
+        const long og = view_offset(a.g, cur.ix);
+        const float is = cur.is;
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
             const int e0 = (c * WAVE + lane) * 8;
             h8 o;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const float d = EXT ? (float)rd1[c][i] + (float)rd2[c][i] : (float)rd1[c][i];
+                const float d = EXT ? (float)cur.d1[c][i] + (float)cur.d2[c][i] : (float)cur.d1[c][i];
                 o[i] = (half_t)(d * fsc[c].v[i]);
-                acc[0][c][i] += d * (float)rin[c][i];
+                acc[0][c][i] += d * (float)cur.in[c][i];
                 acc[1][c][i] += d;
-                if (EXT) acc[2][c][i] += (float)rdl[c][i];
+                if (EXT) acc[2][c][i] += (float)cur.dl[c][i];
             }
             o = pin(o);
             if (nv[c]) stg8<true>(a.g.p + og + e0, o);           // nothing reads G again
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 g[c][i] = (float)o[i];
-                df[c][i] = (float)rdf[c][i];
+                df[c][i] = (float)cur.df[c][i];
                 s1 += g[c][i];
                 s2 = __fmaf_rn(g[c][i], df[c][i], s2);
             }
@@ -98,7 +118,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
         s2 = wave_sum(s2);
         const float c1 = s1 * is * invn;
         const float c2 = s2 * is * is * is * invn;
-        const long oa = view_offset(a.d_ln_in, ix), ob = view_offset(a.d_drop_in, ix);
+        const long oa = view_offset(a.d_ln_in, cur.ix), ob = view_offset(a.d_drop_in, cur.ix);
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
             const int e0 = (c * WAVE + lane) * 8;
@@ -109,12 +129,13 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
             x = pin(x);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                y[i] = rmk[c][i] != (half_t)0.0f ? x[i] : (half_t)0.0f;
+                y[i] = cur.mk[c][i] != (half_t)0.0f ? x[i] : (half_t)0.0f;
                 if (EXT) acc[3][c][i] += (float)y[i];
             }
             stg8<false>(a.d_ln_in.p + oa + e0, x);
             stg8<false>(a.d_drop_in.p + ob + e0, y);
         }
+        if (more) cur = nxt;
     }
     // One partial row per block and sum: ws[(s * gridDim.x + block) * R + feature].
 #pragma unroll
