@@ -20,26 +20,30 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
     return n < 0 ? 0 : (n > 8 ? 8 : n);
 }
 
-// VPL: 8-packs per lane (row length <= 512*VPL).  RPW: rows per wave per step.
-// FAST: all views vectorisable (see ld8).
-template <int VPL, int RPW, bool FAST>
+// VPL: 8-packs per lane (row length <= 8*GRP*VPL).  RPW: rows per lane group per
+// step.  FAST: all views vectorisable (see ld8).  GRP: lanes per row; rows of up
+// to 256 (128) elements take half (a quarter) of a wave, so that two (four) of
+// them are processed side by side and no lane idles.
+template <int VPL, int RPW, bool FAST, int GRP = WAVE>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
                                                    View drop, float scale, PhiloxKey key, unsigned nrows) {
-    const int lane = threadIdx.x & 63;
-    const unsigned step = gridDim.x * WPB * RPW;
-    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+    constexpr int SPW = WAVE / GRP;                    // rows side by side in a wave
+    const int lane = threadIdx.x & 63, gl = lane % GRP, sub = lane / GRP;
+    const unsigned step = gridDim.x * WPB * RPW * SPW;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW * SPW; row0 < nrows; row0 += step) {
         float x[RPW][VPL][8];
         RowIdx ix[RPW];
         float m[RPW], s[RPW];
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            const bool live = row0 + r < nrows;
-            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const unsigned row = row0 + r * SPW + sub;
+            const bool live = row < nrows;
+            ix[r] = row_index(rs, live ? row : row0);
             const long ob = view_offset(beta, ix[r]);
             m[r] = -INFINITY;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
-                int e0 = (c * WAVE + lane) * 8;
+                int e0 = (c * GRP + gl) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
                 F8 f = ld8<FAST, true>(beta, ob, e0, nv, -INFINITY);
 #pragma unroll
@@ -50,7 +54,7 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
             }
         }
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) m[r] = wave_max(m[r]);
+        for (int r = 0; r < RPW; ++r) m[r] = group_max<GRP>(m[r]);
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             s[r] = 0.f;
@@ -63,19 +67,20 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
                 }
         }
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) s[r] = wave_sum(s[r]);
+        for (int r = 0; r < RPW; ++r) s[r] = group_sum<GRP>(s[r]);
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            if (row0 + r >= nrows) continue;
+            const unsigned row = row0 + r * SPW + sub;
+            if (row >= nrows) continue;
             const float inv = 1.0f / s[r];
             const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
-                int e0 = (c * WAVE + lane) * 8;
+                int e0 = (c * GRP + gl) * 8;
                 int nv = nvalid_at(rs.R, e0);
                 if (nv > 0) {
                     h8 a, d;
-                    uint32_t bits = keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0);
+                    uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) a[i] = (half_t)(x[r][c][i] * inv);
                     a = pin(a);
@@ -90,24 +95,26 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
     }
 }
 
-template <int VPL, int RPW, bool FAST>
+template <int VPL, int RPW, bool FAST, int GRP = WAVE>
 __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask, View ddrop,
                                               View dbeta, float scale, unsigned nrows) {
-    const int lane = threadIdx.x & 63;
-    const unsigned step = gridDim.x * WPB * RPW;
-    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
+    constexpr int SPW = WAVE / GRP;
+    const int lane = threadIdx.x & 63, gl = lane % GRP, sub = lane / GRP;
+    const unsigned step = gridDim.x * WPB * RPW * SPW;
+    for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW * SPW; row0 < nrows; row0 += step) {
         float a[RPW][VPL][8], g[RPW][VPL][8];
         RowIdx ix[RPW];
         float s[RPW];
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            const bool live = row0 + r < nrows;
-            ix[r] = row_index(rs, live ? row0 + r : row0);
+            const unsigned row = row0 + r * SPW + sub;
+            const bool live = row < nrows;
+            ix[r] = row_index(rs, live ? row : row0);
             const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(ddrop, ix[r]);
             s[r] = 0.f;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
-                int e0 = (c * WAVE + lane) * 8;
+                int e0 = (c * GRP + gl) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
                 F8 fa = ld8<FAST, true>(alpha, oa, e0, nv), fm = ld8<FAST, true>(mask, om, e0, nv), fd = ld8<FAST, true>(ddrop, od, e0, nv);
 #pragma unroll
@@ -119,14 +126,14 @@ __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask
             }
         }
 #pragma unroll
-        for (int r = 0; r < RPW; ++r) s[r] = wave_sum(s[r]);
+        for (int r = 0; r < RPW; ++r) s[r] = group_sum<GRP>(s[r]);
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
-            if (row0 + r >= nrows) continue;
+            if (row0 + r * SPW + sub >= nrows) continue;
             const long oo = view_offset(dbeta, ix[r]);
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
-                int e0 = (c * WAVE + lane) * 8;
+                int e0 = (c * GRP + gl) * 8;
                 int nv = nvalid_at(rs.R, e0);
                 if (nv > 0) {
                     h8 o;
@@ -347,6 +354,17 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax");
     bool fast = beta.vec && alpha.vec && mask.vec && drop.vec;
+    if (fast && rs.R <= 256 && nrows >= 256u * 16u * 4u) {
+        // short rows: two or four side by side in every wave
+        if (rs.R <= 128)
+            hipLaunchKernelGGL((k_softmax<1, 4, true, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs,
+                               beta, alpha, mask, drop, scale, key, nrows);
+        else
+            hipLaunchKernelGGL((k_softmax<1, 4, true, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs,
+                               beta, alpha, mask, drop, scale, key, nrows);
+        check_launch("softmax");
+        return;
+    }
     SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, scale, key, nrows);
     check_launch("softmax");
 }
@@ -357,6 +375,16 @@ void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax backward");
     bool fast = alpha.vec && mask.vec && ddrop.vec && dbeta.vec;
+    if (fast && rs.R <= 256 && nrows >= 256u * 16u * 4u) {
+        if (rs.R <= 128)
+            hipLaunchKernelGGL((k_bs<1, 4, true, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs, alpha,
+                               mask, ddrop, dbeta, scale, nrows);
+        else
+            hipLaunchKernelGGL((k_bs<1, 4, true, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs, alpha,
+                               mask, ddrop, dbeta, scale, nrows);
+        check_launch("softmax backward");
+        return;
+    }
     SUB_ROW_DISPATCH(k_bs, vpl, fast, rs, alpha, mask, ddrop, dbeta, scale, nrows);
     check_launch("softmax backward");
 }

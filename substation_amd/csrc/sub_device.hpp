@@ -188,6 +188,30 @@ __device__ __forceinline__ float wave_max(float x) {
     return fmaxf(fmaxf(a, b), fmaxf(c, d));
 }
 
+// Reductions over aligned groups of GRP lanes (64, 32 or 16): short rows sit
+// side by side in one wave.  Every lane of a group ends up with the group's
+// value (the four DPP steps above already total each 16-lane row).
+template <int GRP>
+__device__ __forceinline__ float group_sum(float x) {
+    if (GRP == 64) return wave_sum(x);
+    x += dpp<0xB1>(x);
+    x += dpp<0x4E>(x);
+    x += dpp<0x141>(x);
+    x += dpp<0x140>(x);
+    if (GRP == 32) x += __shfl_xor(x, 16);
+    return x;
+}
+template <int GRP>
+__device__ __forceinline__ float group_max(float x) {
+    if (GRP == 64) return wave_max(x);
+    x = fmaxf(x, dpp<0xB1>(x));
+    x = fmaxf(x, dpp<0x4E>(x));
+    x = fmaxf(x, dpp<0x141>(x));
+    x = fmaxf(x, dpp<0x140>(x));
+    if (GRP == 32) x = fmaxf(x, __shfl_xor(x, 16));
+    return x;
+}
+
 // Makes a rounded fp16 pack opaque to the optimiser, so that a second output
 // derived from it (value * {0,1} mask) is bit-identical to it rather than
 // recomputed through a differently rounded (fused) conversion.

@@ -39,7 +39,9 @@ def _perms(canon, keep=None, limit=4):
 SIZES = [(2, 16, 2, 32), (3, 24, 2, 48), (2, 128, 4, 512)]
 
 
-@pytest.mark.parametrize('B,L,H,E', SIZES + [(1, 520, 1, 8)])
+# the last four: short rows, several side by side in a wave (needs >= 16384 rows)
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(1, 520, 1, 8), (8, 128, 16, 64), (4, 256, 16, 64),
+                                            (9, 120, 16, 32), (6, 200, 16, 32)])
 @pytest.mark.parametrize('p', [0.0, 0.5])
 def test_softmax_and_backward(B, L, H, E, p):
     o = _ops(B, L, H, E)
