@@ -38,16 +38,15 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91621893, 'QKT': 84086417, 'softmax': 268701348,
-    'gamma': 84090513, 'out': 33751434, 'bdrln1': 59106304,
-    'lin1': 99703334, 'bad': 134437888, 'lin2': 109241083,
-    'bdrln2': 59105728, 'bsb': 26412177, 'blnrd1': 42148836,
-    'dXlin2': 100605894, 'dWlin2': 109277047, 'bdrlb': 135210466,
-    'dXlin1': 109264486, 'dWlin1': 109276901, 'ebsb': 43702960,
-    'blnrd2': 42148434, 'baob': 9025049, 'dWout': 129458241,
-    'dXout': 33775166, 'dX1gamma': 84086545, 'dX2gamma': 84086362,
-    'bs': 268534218, 'dX1QKT': 84087478, 'dX2QKT': 84084698,
-    'dXQKV-fused': 92489041, 'dWQKV-fused': 115567343, 'baib': 26066282,
+    'QKV-fused': 88458950, 'QKT': 84224724, 'softmax': 268732372,
+    'gamma': 84147253, 'out': 33775479, 'bdrln1': 59009319,
+    'lin1': 84251840, 'bad': 134581848, 'lin2': 109264877,
+    'bdrln2': 59011257, 'bsb+blnrd1': 61022809, 'dXlin2': 84238401,
+    'dWlin2': 109275336, 'bdrlb': 135394697, 'dXlin1': 109260544,
+    'dWlin1': 109274879, 'ebsb+blnrd2+baob': 79940520, 'dWout': 129206807,
+    'dXout': 33771073, 'dX1gamma': 84224523, 'dX2gamma': 84110521,
+    'bs': 268534489, 'dX1QKT': 84096442, 'dX2QKT': 84093078,
+    'dXQKV-fused': 92485074, 'dWQKV-fused': 115565462, 'baib': 25997175,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
