@@ -1,0 +1,122 @@
+"""Layout search: operator graph consistency and the descent on a synthetic
+cost table (CPU), one short search on the device with parity of the layer
+under the layouts it returns (GPU)."""
+import io
+import itertools
+
+import numpy as np
+import pytest
+
+from substation_amd import layouts as L
+from substation_amd import layout_search as ls
+from substation_amd import opgraph as og
+
+
+def test_operator_graph_names_every_tensor_once_known():
+    names = set(L.CANONICAL)
+    used = set()
+    for op, which, tensors in og.OPERATORS:
+        assert which in ('fwd', 'bwd')
+        for t in tensors:
+            assert t in names, (op, t)
+        used.update(tensors)
+    # every tensor of the pickle is touched by some launch, except the per-feature vectors
+    assert names - used <= {'BO', 'S1', 'B1', 'LINB1', 'S2', 'B2', 'LINB2'}
+    for group in og.ALTERNATIVES:
+        for op in group:
+            assert op in og.OP_TENSORS
+    # the 18 contractions are operators of the graph and their operands resolve
+    t = og.operand_layouts(L.mi355x_layouts())
+    for name, (a, b, c) in og.EINSUMS.items():
+        assert name in og.OP_TENSORS
+        assert a in t and b in t and c in t
+
+
+def test_candidate_layouts_respect_the_stacking_dim():
+    assert og.candidate_layouts('X') == [''.join(p) for p in itertools.permutations('BJI')]
+    for name in ('KKQQVV', 'DKKQQVV', 'WKKWQQWVV', 'WKQV', 'BKQV'):
+        c = og.candidate_layouts(name)
+        assert all(l[0] == 'Q' for l in c) and len(set(c)) == len(c)
+        assert sorted(c[0]) == sorted(L.CANONICAL[name])
+    assert len(og.candidate_layouts('KKQQVV')) == 24
+    assert 'BO' not in og.searchable_tensors()
+    changed = og.with_layouts(L.mi355x_layouts(), {'X': 'JBI', 'LINW1': 'IU', 'DATT': 'IBJ'})
+    t = og.tensor_layouts(L.validate(changed))
+    assert (t['X'], t['LINW1'], t['DATT'], t['SB2']) == ('JBI', 'IU', 'IBJ', 'BJI')
+
+
+class _SyntheticTimer:
+    """Every operator costs 1 us plus 1 us per tensor that is not in its preferred
+    layout; the fused-away launches are not reported (as on the device)."""
+    SKIP = {'aib', 'bei', 'bsb', 'blnrd1', 'ebsb', 'blnrd2', 'baob'}
+
+    def __init__(self, preferred, forbidden=()):
+        self.preferred, self.forbidden, self.runs = preferred, set(forbidden), 0
+
+    def usable(self, layouts):
+        t = og.tensor_layouts(layouts)
+        return not any((n, t[n]) in self.forbidden for n in t)
+
+    def measure(self, layouts):
+        self.runs += 1
+        t = og.tensor_layouts(layouts)
+        return {op: 1e-6 * (1 + sum(t[n] != self.preferred.get(n, t[n]) for n in tensors))
+                for op, _, tensors in og.OPERATORS if op not in self.SKIP}
+
+
+def test_descent_finds_the_preferred_layouts():
+    start = L.mi355x_layouts()
+    preferred = {'X': 'JBI', 'SB2': 'JBI', 'SB1': 'IBJ', 'LINW1': 'IU', 'BETA': 'BHJK', 'KKQQVV': 'QHBJP',
+                 'DLIN1': 'UBJ'}
+    timer = _SyntheticTimer(preferred)
+    log = io.StringIO()
+    s = ls.LayoutSearch(timer, start, log=log, out=io.StringIO())
+    c0 = s.cost(start)
+    best = s.run(sweeps=3)
+    t = og.tensor_layouts(best)
+    for name, lay in preferred.items():
+        assert t[name] == lay, (name, t[name])
+    assert s.cost(best) < c0
+    assert t['X'] == t['SB2']                      # input and output stay tied
+    L.validate(best)
+    # the table log is in the reference's "k = v ... time = X s" format
+    line = log.getvalue().splitlines()[0].split()
+    assert line[:3] == ['op', '=', 'QKV-fused'] and line[-4] == 'time' and line[-1] == 's'
+    # everything was answered from the table in the end
+    runs = timer.runs
+    s.cost(best)
+    assert timer.runs == runs
+
+
+def test_descent_respects_fixed_tensors_and_unusable_configurations():
+    start = L.mi355x_layouts()
+    preferred = {'SB1': 'IBJ', 'LINW1': 'IU', 'DLIN1': 'UBJ'}
+    timer = _SyntheticTimer(preferred, forbidden=[('DLIN1', 'UBJ')])
+    s = ls.LayoutSearch(timer, start, fixed=['SB1'], out=io.StringIO())
+    t = og.tensor_layouts(s.run(sweeps=2))
+    assert t['SB1'] == 'BJI'            # fixed
+    assert t['DLIN1'] != 'UBJ'          # never usable
+    assert t['LINW1'] == 'IU'
+
+
+@pytest.mark.gpu
+def test_search_on_device_returns_layouts_that_keep_parity(tmp_path):
+    """A short search at a small size (few tensors free, one sweep), then the
+    whole layer under the returned layouts against the oracle."""
+    from tests.test_encoder_gpu import run_layer, _compare
+    dims = (2, 64, 4, 256)
+    timer = ls.LayerTimer(*dims, iters=2, warmup=1)
+    free = {'LINW1', 'LINW2', 'SB1', 'DATT', 'GAMMA'}
+    fixed = [n for n in og.searchable_tensors() if n not in free]
+    log = io.StringIO()
+    s = ls.LayoutSearch(timer, L.reference_layouts('bert-b96-l128-h16-e1024'), fixed=fixed, log=log,
+                        out=io.StringIO(), min_gain=0.01)
+    best = s.run(sweeps=1)
+    assert s.evaluations >= 10 and len(s.table) > len(og.OPERATORS) - 8
+    assert np.isfinite(s.cost(best))
+    path = tmp_path / 'found.pickle'
+    L.save_layouts(best, str(path))
+    again = L.load_layouts(str(path))
+    assert og.tensor_layouts(again) == og.tensor_layouts(best)
+    want, got = run_layer(*dims, again, 0.1, 'relu', seed_data=21)
+    _compare(want, got)
