@@ -202,19 +202,24 @@ def test_fused_ln_backward_matches_separate(dims, act):
     _compare(w0, sep)
 
 
-@pytest.mark.parametrize('which', ['mi355x', 'bert-b8-l512-h16-e1024'])
-def test_fused_epilogues_match_unfused(which):
+@pytest.mark.parametrize('which,dims,act', [
+    ('mi355x', (2, 64, 2, 128), 'relu'), ('mi355x', (2, 64, 2, 128), 'gelu'),
+    ('bert-b8-l512-h16-e1024', (2, 64, 2, 128), 'relu'),
+    ('mi355x', (3, 40, 3, 120), 'relu'),             # edge tiles
+    ('mi355x', (8, 512, 16, 1024), 'relu'),          # the bench size: 256x256 asynchronous tiles
+])
+def test_fused_epilogues_match_unfused(which, dims, act):
     """Without debug capture the QKV bias add and the DX residual add run inside
     the GEMM epilogues (where the layouts allow it).  Both roundings are kept, so
     outputs and gradients must be bit-identical to the unfused operator sequence."""
     from substation_amd import Encoder
     lay = _layouts(which)
-    B, L, H, E = 2, 64, 2, 128
+    B, L, H, E = dims
     outs = []
     for debug in (True, False):
         torch.manual_seed(0)
         enc = Encoder('unused', B, L, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, enable_debug=debug,
-                      seed=SEED).cuda()
+                      seed=SEED, activation=act).cuda()
         enc.set_rng(SEED, 0)
         with torch.no_grad():
             for p in enc.parameters():
