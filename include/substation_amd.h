@@ -107,6 +107,15 @@ int sub_set_stream(void* handle, void* hip_stream);  /* hipStream_t */
 /* Dropout masks are a pure function of (seed, site, step, element); step is
  * incremented by every encoder_forward (blocks.cuh:48-51 advances an offset). */
 int sub_set_rng(void* handle, uint64_t seed, uint32_t step);
+/* No counterpart in the reference (its generator state lives in device memory
+ * already, blocks.cuh:24-51).  For callers that record the launches in a HIP
+ * graph: kernel arguments, the step included, are frozen at capture, so replays
+ * would repeat the captured masks.  With a counter in device memory set here
+ * (one uint32, owned by the caller, NULL to switch off), the step a kernel uses
+ * is the host step of sub_set_rng plus *device_step read when the kernel runs,
+ * and encoder_forward advances *device_step on the stream instead of the host
+ * step. */
+int sub_set_rng_counter(void* handle, uint32_t* device_step);
 const char* sub_last_error(void);
 
 /* Options.  SUB_OPT_FUSE_EPILOGUES (default 1): add BKQV in the epilogue of the

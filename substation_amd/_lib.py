@@ -50,6 +50,7 @@ SIGNATURES = {
     'sub_configure': (_I, [_VP, ctypes.POINTER(SubConfig)]),
     'sub_set_stream': (_I, [_VP, _VP]),
     'sub_set_rng': (_I, [_VP, _U64, _U32]),
+    'sub_set_rng_counter': (_I, [_VP, _VP]),
     'sub_last_error': (_CP, []),
     'sub_set_option': (_I, [_VP, _I, _I]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
@@ -161,6 +162,9 @@ class Handle:
 
     def set_rng(self, seed, step=0):
         check(self.lib.sub_set_rng(self.ptr, seed, step), 'sub_set_rng')
+
+    def set_rng_counter(self, device_ptr):
+        check(self.lib.sub_set_rng_counter(self.ptr, ctypes.c_void_p(device_ptr or 0)), 'sub_set_rng_counter')
 
     def set_option(self, option, value):
         check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')

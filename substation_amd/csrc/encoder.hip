@@ -177,15 +177,22 @@ struct Handle {
     float* gws = nullptr;         // split-k partials of the small-output contractions
     size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
+    uint32_t* step_dev = nullptr;     // optional device-side dropout step (HIP-graph replays)
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
     ~Handle() {
+        // A handle may be destroyed (e.g. by a garbage collector) while some other
+        // stream of the process is being captured into a HIP graph; freeing this
+        // handle's own scratch must not invalidate that capture.
+        hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+        const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
         if (ws) (void)hipFree(ws);
         if (gws) (void)hipFree(gws);
         for (auto& e : prof) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+        if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
     }
 };
 
@@ -197,6 +204,7 @@ PhiloxKey make_key(const Handle& h, uint32_t site, float p) {
     PhiloxKey k;
     k.k0 = (uint32_t)h.seed; k.k1 = (uint32_t)(h.seed >> 32);
     k.site = site; k.step = h.step; k.thr = threshold16(p);
+    k.step_dev = h.step_dev;
     return k;
 }
 
@@ -218,8 +226,18 @@ struct ProfScope {
     void cancel() { if (e) { --h.prof_used; e = nullptr; } }     // nothing was launched
 };
 
+// Allocations happen on the first call of a handle; that call cannot be part
+// of a graph capture.
+void refuse_capture(const Handle& h, const char* what) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(h.stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+        fail(std::string(what) + ": the scratch buffers are allocated by the first forward/backward call, "
+             "run one outside the graph capture first");
+}
+
 void ensure_ws(Handle& h, size_t floats) {
     if (floats <= h.ws_floats) return;
+    refuse_capture(h, "column-sum workspace");
     if (h.ws) hip_check(hipFree(h.ws), "hipFree");
     h.ws = nullptr; h.ws_floats = 0;
     hip_check(hipMalloc((void**)&h.ws, floats * sizeof(float)), "hipMalloc(workspace)");
@@ -385,6 +403,7 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
         for (int i = 0; i < 3; ++i) ep.sbb[i] = p.sb[i];
     }
     if (h.gws_need > h.gws_floats) {
+        refuse_capture(h, "split-k workspace");
         if (h.gws) hip_check(hipFree(h.gws), "hipFree");
         h.gws = nullptr; h.gws_floats = 0;
         hip_check(hipMalloc((void**)&h.gws, h.gws_need * sizeof(float)), "hipMalloc(split-k workspace)");
@@ -582,6 +601,11 @@ half_t* sub_q(void* base, const Handle& h, int q) {
     return (half_t*)base + (int64_t)q * n;
 }
 
+// Advances the device-side dropout step (a vector store by one lane).
+__global__ void k_step_increment(uint32_t* step) {
+    if (threadIdx.x == 0) step[0] = step[0] + 1u;
+}
+
 void forward(Handle& h, const FwdPtrs& t) {
     if (!h.configured) fail("encoder_forward: handle is not configured");
     h.prof_used = 0;
@@ -622,7 +646,12 @@ void forward(Handle& h, const FwdPtrs& t) {
                  F[LIN2], h.lf[LIN2], F[DROP3MASK], h.lf[DROP3MASK], F[LN2DIFF], h.lf[LN2DIFF],
                  F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2);
     }
-    h.step += 1;
+    if (h.step_dev) {
+        hipLaunchKernelGGL(k_step_increment, dim3(1), dim3(64), 0, h.stream, h.step_dev);
+        check_launch("dropout step increment");
+    } else {
+        h.step += 1;
+    }
 }
 
 void backward(Handle& h, const BwdPtrs& t) {
@@ -813,6 +842,10 @@ int sub_set_stream(void* handle, void* hip_stream) {
 
 int sub_set_rng(void* handle, uint64_t seed, uint32_t step) {
     return guarded([&] { Handle& h = as_handle(handle); h.seed = seed; h.step = step; });
+}
+
+int sub_set_rng_counter(void* handle, uint32_t* device_step) {
+    return guarded([&] { as_handle(handle).step_dev = device_step; });
 }
 
 int sub_encoder_forward(void* handle, void* const* ptrs, int n) {
@@ -1048,7 +1081,7 @@ int sub_einsum_classify(void* handle, const char* l_A, const char* l_B, const ch
 int sub_philox_fields_host(uint64_t seed, uint32_t site, uint32_t step, uint64_t start, uint64_t n,
                            uint16_t* out) {
     return guarded([&] {
-        PhiloxKey k; k.k0 = (uint32_t)seed; k.k1 = (uint32_t)(seed >> 32); k.site = site; k.step = step; k.thr = 0;
+        PhiloxKey k{}; k.k0 = (uint32_t)seed; k.k1 = (uint32_t)(seed >> 32); k.site = site; k.step = step; k.thr = 0;
         for (uint64_t i = 0; i < n; ++i) {
             uint64_t e = start + i;
             U4 r = philox_group(k, e >> 3);

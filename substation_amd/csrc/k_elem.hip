@@ -38,8 +38,9 @@ __device__ __forceinline__ Chunk chunk_of(const RowSpace& rs, unsigned idx, unsi
 
 template <bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, View lin, View mask,
-                                               View out, int act, PhiloxKey key, unsigned nchunks,
+                                               View out, int act, PhiloxKey key_, unsigned nchunks,
                                                unsigned cpr) {
+    const PhiloxKey key = resolved(key_);
     const unsigned stride = gridDim.x * BLOCK;
     for (unsigned base = blockIdx.x * BLOCK + threadIdx.x; base < nchunks; base += stride * UNROLL) {
         Chunk c[UNROLL];

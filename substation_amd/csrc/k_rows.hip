@@ -26,7 +26,8 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
 // them are processed side by side and no lane idles.
 template <int VPL, int RPW, bool FAST, int GRP = WAVE>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
-                                                   View drop, float scale, PhiloxKey key, unsigned nrows) {
+                                                   View drop, float scale, PhiloxKey key_, unsigned nrows) {
+    const PhiloxKey key = resolved(key_);
     constexpr int SPW = WAVE / GRP;                    // rows side by side in a wave
     const int lane = threadIdx.x & 63, gl = lane % GRP, sub = lane / GRP;
     const unsigned step = gridDim.x * WPB * RPW * SPW;
@@ -150,7 +151,8 @@ template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resid, View lin_bias,
                                                  View scale, View bias, View lin, View mask,
                                                  View diff, View normed, View out, View istd,
-                                                 PhiloxKey key, float eps, unsigned nrows) {
+                                                 PhiloxKey key_, float eps, unsigned nrows) {
+    const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63;
     const unsigned step = gridDim.x * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;

@@ -147,6 +147,13 @@ __device__ __forceinline__ void st8h(const View& t, long base, int e0, int nvali
     }
 }
 
+// The key a kernel works with: the device-side step counter, if any, folded in.
+__device__ __forceinline__ PhiloxKey resolved(PhiloxKey k) {
+    if (k.step_dev) k.step += *k.step_dev;
+    k.step_dev = nullptr;
+    return k;
+}
+
 // d(LN input) of one element: g * istd - c1 - diff * c2, with the contraction
 // into FMAs spelled out so that every kernel that evaluates it rounds alike.
 __device__ __forceinline__ float ln_bwd_value(float g, float diff, float istd, float c1, float c2) {

@@ -23,6 +23,10 @@ struct PhiloxKey {
     uint32_t k0, k1;     // seed
     uint32_t site, step; // counter words 2 and 3
     uint32_t thr;        // drop threshold on a 16-bit field, 0..65536
+    // Optional step counter in device memory, added to `step` when a kernel
+    // starts: launches recorded in a HIP graph then draw new masks on every
+    // replay (their arguments, `step` included, are frozen at capture).
+    const uint32_t* step_dev = nullptr;
 };
 
 struct U4 { uint32_t x, y, z, w; };

@@ -157,6 +157,24 @@ class Encoder(torch.nn.Module):
         self.seed = seed
         self._handle.set_rng(seed, step)
 
+    def use_device_step(self, counter=None):
+        """Keeps the dropout step in device memory (a one-element int32 CUDA tensor,
+        created at zero when not given) so that forward calls recorded in a HIP
+        graph draw new masks on every replay: the step a kernel uses is the host
+        step of ``set_rng`` plus this counter, which every forward advances on
+        the stream.  Returns the tensor; ``use_device_step(False)`` switches back."""
+        if counter is False:
+            self._step_counter = None
+            self._handle.set_rng_counter(0)
+            return None
+        if counter is None:
+            counter = torch.zeros(1, dtype=torch.int32, device='cuda')
+        if not (counter.is_cuda and counter.dtype == torch.int32 and counter.numel() == 1):
+            raise ValueError('the step counter is a one-element int32 CUDA tensor')
+        self._step_counter = counter          # keeps the memory alive
+        self._handle.set_rng_counter(counter.data_ptr())
+        return counter
+
     def profile(self):
         """Per-operator times in ms of the last forward or backward call
         (``profiling=True`` only); the counterpart of the NVTX ranges of

@@ -235,3 +235,77 @@ def test_fused_epilogues_match_unfused(which, dims, act):
     for a, b in zip(*outs):
         assert torch.isfinite(a.float()).all()
         assert torch.equal(a, b)
+
+
+def test_hip_graph_replays_match_eager_and_draw_new_masks():
+    """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
+    the library's one-time allocations) and replayed with eager work in between:
+    every replay must equal the eager run at the same dropout step bit for bit.
+    With the step counter in device memory, each replay draws the next step's
+    masks, although the kernel arguments were frozen at capture."""
+    from substation_amd import Encoder, layouts as L
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = 2, 64, 4, 256
+
+    def make(device_step):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED).cuda()
+        with torch.no_grad():
+            for p in enc.parameters():
+                p.mul_(0.1)
+        enc.set_rng(SEED, 0)
+        return enc, (enc.use_device_step() if device_step else None)
+
+    g0 = torch.Generator().manual_seed(9)
+    X = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
+    DY = torch.randn(B, Ls, E, generator=g0).half().cuda()
+
+    def collect(enc, Y):
+        return [Y.detach().clone(), X.grad.clone()] + [p.grad.clone() for p in enc.parameters()]
+
+    def clear(enc):
+        X.grad = None
+        for p in enc.parameters():
+            p.grad = None
+
+    enc, counter = make(True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):                       # warm-up: steps 0 and 1
+            clear(enc)
+            enc(X).backward(DY)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert int(counter.item()) == 2
+    clear(enc)
+    # a module that was never run cannot be captured: its scratch is allocated by the first call
+    fresh, _ = make(False)
+    with pytest.raises(Exception):
+        with torch.cuda.graph(torch.cuda.CUDAGraph()):
+            with torch.no_grad():
+                fresh(X)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        Y = enc(X)
+        Y.backward(DY)
+    assert int(counter.item()) == 2              # capture runs nothing
+    replays = []
+    for r in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        replays.append(collect(enc, Y))
+        assert int(counter.item()) == 3 + r
+        _ = (torch.randn(1 << 20, device='cuda') * 2).sum().item()      # eager work between replays
+
+    ref, _ = make(False)
+    for r in range(3):
+        ref.set_rng(SEED, 2 + r)
+        clear(ref)
+        Yr = ref(X)
+        Yr.backward(DY)
+        torch.cuda.synchronize()
+        for a, b in zip(replays[r], collect(ref, Yr)):
+            assert torch.equal(a, b), f'replay {r} differs from the eager run at step {2 + r}'
+    assert not torch.equal(replays[0][0], replays[1][0])     # new masks on every replay
