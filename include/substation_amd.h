@@ -117,6 +117,14 @@ int sub_set_rng(void* handle, uint64_t seed, uint32_t step);
  * step. */
 int sub_set_rng_counter(void* handle, uint32_t* device_step);
 const char* sub_last_error(void);
+/* Masked self-attention: the layer of substation/transformer.py:443-546
+ * (`decoder`), i.e. the encoder layer with an additive [J,K] mask on the
+ * attention scores (fp16 device tensor owned by the caller, layout "JK" or
+ * "KJ"; -inf above the diagonal for a causal layer).  As in
+ * substation/attention.py:65-68 the mask is added to the raw scores, before the
+ * 1/sqrt(P) scaling.  encoder_forward uses it until it is cleared with NULL;
+ * encoder_backward needs nothing (masked positions have zero probability). */
+int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layout);
 
 /* Options.  SUB_OPT_FUSE_EPILOGUES (default 1): add BKQV in the epilogue of the
  * QKV projection and DRESID1 in the epilogue of the input-gradient projection,
@@ -157,6 +165,14 @@ int sub_profile_read(void* handle, int cap, const char** names, float* ms);
 int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alpha,
                    const char* l_alpha, void* mask, const char* l_mask, void* drop,
                    const char* l_drop, float scale, float p, uint32_t site);
+/* The same with an additive attention mask over (query, key) positions
+ * (substation/attention.py:65-68, mask of transformer.py:151-157):
+ * alpha = softmax(beta * scale + attn_mask * mask_scale); attn_mask is a [J,K]
+ * fp16 tensor in layout "JK" or "KJ", shared by all heads and samples. */
+int sub_op_softmax_masked(void* handle, const void* beta, const char* l_beta, void* alpha,
+                          const char* l_alpha, void* mask, const char* l_mask, void* drop,
+                          const char* l_drop, const void* attn_mask, const char* l_attn_mask,
+                          float scale, float mask_scale, float p, uint32_t site);
 /* block_bs.cuh:107-156 */
 int sub_op_bs(void* handle, const void* alpha, const char* l_alpha, const void* mask,
               const char* l_mask, const void* ddrop, const char* l_ddrop, void* dbeta,

@@ -163,11 +163,18 @@ def softmax_backward_data(y, dy, dim=-1):
 # multi-head attention                           substation/attention.py:31-179
 # --------------------------------------------------------------------------
 
-def attn_forward(q, k, v, wq, wk, wv, wo, in_b, out_b, scale, softmax_mask=None):
+def gen_attn_mask(lq, lk, dtype=np.float64):
+    """Causal additive mask, transformer.py:151-157: -inf above the diagonal."""
+    return np.triu(np.full((lq, lk), float('-inf'), dtype=dtype), k=1)
+
+
+def attn_forward(q, k, v, wq, wk, wv, wo, in_b, out_b, scale, softmax_mask=None, attn_mask=None):
     """attention.py:31-79, plus the softmax-output dropout of encoder.cu:120.
 
     q,k,v [B,L,E]; wq,wk,wv [H,P,E]; wo [E,H*P]; in_b [3,H,P] in (q,k,v) order;
-    softmax_mask [B,H,Lq,Lk] of {0,1} or None.  Same per-sample loop of
+    softmax_mask [B,H,Lq,Lk] of {0,1} or None (dropout of the softmax output);
+    attn_mask [Lq,Lk] additive or None, added to the raw scores BEFORE the
+    scaling as at attention.py:65-68 (a 0/-inf mask is indifferent to that).  Same per-sample loop of
     ``np.matmul`` over the head axis as the reference.  Returns
     (out [B,Lq,E], concat, proj_q, proj_k, proj_v, alpha, attn_drop) with the
     five/six intermediates as per-sample lists like the reference's.
@@ -179,6 +186,8 @@ def attn_forward(q, k, v, wq, wk, wv, wo, in_b, out_b, scale, softmax_mask=None)
         proj_k = np.matmul(k[b], wk.transpose(0, 2, 1)) + np.expand_dims(in_b[1], axis=1)
         proj_v = np.matmul(v[b], wv.transpose(0, 2, 1)) + np.expand_dims(in_b[2], axis=1)
         scores = np.matmul(proj_q, proj_k.transpose(0, 2, 1))       # [H,Lq,Lk]
+        if attn_mask is not None:
+            scores = scores + attn_mask
         alpha = softmax(scale * scores, dim=-1)
         attn_drop = dropout(alpha, None if softmax_mask is None else softmax_mask[b])
         weighted = np.matmul(attn_drop, proj_v)                      # [H,Lq,P]
@@ -243,8 +252,12 @@ def encoder(x, attn_wq, attn_wk, attn_wv, attn_wo, attn_in_b, attn_out_b, attn_s
             norm1_scale, norm1_bias, norm2_scale, norm2_bias,
             linear1_w, linear1_b, linear2_w, linear2_b,
             softmax_mask=None, attn_dropout_mask=None, linear1_dropout_mask=None,
-            ff_dropout_mask=None, activation='relu', ln_mode='rsqrt'):
-    """Post-LN encoder layer forward, transformer.py:176-209.
+            ff_dropout_mask=None, activation='relu', ln_mode='rsqrt', attn_mask=None):
+    """Post-LN encoder layer forward, transformer.py:176-209; with ``attn_mask``
+    [L,L] (additive) it is the masked-self-attention layer ``decoder`` of
+    transformer.py:443-476.  The backward pass does not see the mask
+    (transformer.py:478-546 passes it on, attention.py:82-179 never reads it:
+    a masked position has alpha = 0, hence no gradient).
 
     Masks: softmax_mask [B,H,L,L], attn_dropout_mask [B,L,E],
     linear1_dropout_mask [B,L,U], ff_dropout_mask [B,L,E]; None = no dropout.
@@ -254,7 +267,7 @@ def encoder(x, attn_wq, attn_wk, attn_wv, attn_wo, attn_in_b, attn_out_b, attn_s
     act = _ACT[activation][0]
     (attn, attn_concat, proj_q, proj_k, proj_v, alpha, attn_drop) = attn_forward(
         x, x, x, attn_wq, attn_wk, attn_wv, attn_wo, attn_in_b, attn_out_b, attn_scale,
-        softmax_mask)
+        softmax_mask, attn_mask)
     attn_resid = dropout(attn, attn_dropout_mask) + x
     normed1, norm1_mean, norm1_std, norm1_normed = layer_norm(
         attn_resid, norm1_scale, norm1_bias, ln_mode=ln_mode)
@@ -364,7 +377,8 @@ def module_params_to_numpy(p):
         linear2_w=np.ascontiguousarray(p['LINW2'].T), linear2_b=p['LINB2'])
 
 
-def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', relu_gate=None):
+def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', relu_gate=None,
+              attn_mask=None):
     """Forward + backward with device-module naming.
 
     params: dict name -> array in canonical dim order (CANONICAL); X, DY [B,J,I];
@@ -384,7 +398,7 @@ def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', rel
     f = encoder(X, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], a['attn_in_b'],
                 a['attn_out_b'], scale, a['norm1_scale'], a['norm1_bias'], a['norm2_scale'],
                 a['norm2_bias'], a['linear1_w'], a['linear1_b'], a['linear2_w'], a['linear2_b'],
-                activation=activation, ln_mode=ln_mode, **mk)
+                activation=activation, ln_mode=ln_mode, attn_mask=attn_mask, **mk)
     g = encoder_backward(X, DY, f, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], scale,
                          a['norm1_scale'], a['norm2_scale'], a['linear1_w'], a['linear1_b'],
                          a['linear2_w'], a['linear2_b'], activation=activation,

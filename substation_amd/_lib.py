@@ -58,6 +58,8 @@ SIGNATURES = {
     'sub_profile_enable': (_I, [_VP, _I]),
     'sub_profile_read': (_I, [_VP, _I, ctypes.POINTER(_CP), ctypes.POINTER(_F)]),
     'sub_op_softmax': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _U32]),
+    'sub_op_softmax_masked': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _F, _U32]),
+    'sub_set_attention_mask': (_I, [_VP, _VP, _CP]),
     'sub_op_bs': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_bdrln': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP, _CP, _VP, _CP, _VP, _CP,
                           _VP, _CP, _VP, _CP, _VP, _CP, _F, _U32]),
@@ -165,6 +167,10 @@ class Handle:
 
     def set_rng_counter(self, device_ptr):
         check(self.lib.sub_set_rng_counter(self.ptr, ctypes.c_void_p(device_ptr or 0)), 'sub_set_rng_counter')
+
+    def set_attention_mask(self, device_ptr, layout='JK'):
+        check(self.lib.sub_set_attention_mask(self.ptr, ctypes.c_void_p(device_ptr or 0), layout.encode()),
+              'sub_set_attention_mask')
 
     def set_option(self, option, value):
         check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')

@@ -178,6 +178,8 @@ struct Handle {
     size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
     uint32_t* step_dev = nullptr;     // optional device-side dropout step (HIP-graph replays)
+    const void* attn_mask = nullptr;  // optional additive [J,K] attention mask (caller-owned)
+    Layout l_attn_mask;
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
     std::vector<ProfEntry> prof;
@@ -417,12 +419,21 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 void op_softmax(Handle& h, const void* beta, const Layout& lb, void* alpha, const Layout& la,
                 void* mask, const Layout& lm, void* drop, const Layout& ld, float scale, float p,
-                uint32_t site) {
+                uint32_t site, const void* amask = nullptr, const Layout* lam = nullptr,
+                float mscale = 1.f) {
     Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
     View vb = make_view(beta, lb, sp), va = make_view(alpha, la, sp), vm = make_view(mask, lm, sp),
          vd = make_view(drop, ld, sp);
-    flatten(sp.rs, {&vb, &va, &vm, &vd});
-    launch_softmax(sp.rs, vb, va, vm, vd, scale, make_key(h, site, p), h.stream);
+    View vam; vam.p = nullptr; vam.s0 = vam.s1 = vam.s2 = vam.s3 = 0; vam.sr = 0; vam.vec = 0;
+    if (amask) {
+        if (!lam || lam->rank != 2 || !lam->has[dJ] || !lam->has[dK])
+            fail("softmax: the attention mask is a [J,K] tensor (layout JK or KJ)");
+        vam = make_view(amask, *lam, sp);       // strides 0 along heads and samples
+        flatten(sp.rs, {&vb, &va, &vm, &vd, &vam});
+    } else {
+        flatten(sp.rs, {&vb, &va, &vm, &vd});
+    }
+    launch_softmax(sp.rs, vb, va, vm, vd, vam, scale, mscale, make_key(h, site, p), h.stream);
 }
 
 void op_bs(Handle& h, const void* alpha, const Layout& la, const void* mask, const Layout& lm,
@@ -623,7 +634,8 @@ void forward(Handle& h, const FwdPtrs& t) {
     {
         ProfScope ps(h, "softmax");
         op_softmax(h, F[BETA], h.lf[BETA], F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK],
-                   F[ATTN_DROP], h.lf[ATTN_DROP], 1.0f, h.p_softmax, SUB_SITE_SOFTMAX);
+                   F[ATTN_DROP], h.lf[ATTN_DROP], 1.0f, h.p_softmax, SUB_SITE_SOFTMAX, h.attn_mask,
+                   &h.l_attn_mask, h.gemm[G_QKT].alpha);
     }
     run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
     run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
@@ -938,6 +950,28 @@ int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alp
         Handle& h = as_handle(handle); need_cfg(h);
         op_softmax(h, beta, L(h, l_beta), alpha, L(h, l_alpha), mask, L(h, l_mask), drop, L(h, l_drop),
                    scale, p, site);
+    });
+}
+
+int sub_op_softmax_masked(void* handle, const void* beta, const char* l_beta, void* alpha,
+                          const char* l_alpha, void* mask, const char* l_mask, void* drop,
+                          const char* l_drop, const void* attn_mask, const char* l_attn_mask,
+                          float scale, float mask_scale, float p, uint32_t site) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        Layout lam = L(h, l_attn_mask);
+        op_softmax(h, beta, L(h, l_beta), alpha, L(h, l_alpha), mask, L(h, l_mask), drop, L(h, l_drop),
+                   scale, p, site, attn_mask, &lam, mask_scale);
+    });
+}
+
+int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layout) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        if (!attn_mask) { h.attn_mask = nullptr; return; }
+        Layout l = L(h, layout);
+        if (l.rank != 2 || !l.has[dJ] || !l.has[dK]) fail("sub_set_attention_mask: layout must be JK or KJ");
+        h.attn_mask = attn_mask; h.l_attn_mask = l;
     });
 }
 

@@ -24,9 +24,13 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
 // step.  FAST: all views vectorisable (see ld8).  GRP: lanes per row; rows of up
 // to 256 (128) elements take half (a quarter) of a wave, so that two (four) of
 // them are processed side by side and no lane idles.
+// amask (optional, p == nullptr when absent): additive attention mask indexed by
+// (query position, key position) only, x = beta * scale + amask * mscale
+// (substation/attention.py:65-68 adds it before the scaling, hence mscale).
 template <int VPL, int RPW, bool FAST, int GRP = WAVE>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
-                                                   View drop, float scale, PhiloxKey key_, unsigned nrows) {
+                                                   View drop, View amask, float scale, float mscale,
+                                                   PhiloxKey key_, unsigned nrows) {
     const PhiloxKey key = resolved(key_);
     constexpr int SPW = WAVE / GRP;                    // rows side by side in a wave
     const int lane = threadIdx.x & 63, gl = lane % GRP, sub = lane / GRP;
@@ -41,15 +45,25 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
             const bool live = row < nrows;
             ix[r] = row_index(rs, live ? row : row0);
             const long ob = view_offset(beta, ix[r]);
+            const long oam = amask.p ? view_offset(amask, ix[r]) : 0;
             m[r] = -INFINITY;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * GRP + gl) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
                 F8 f = ld8<FAST, true>(beta, ob, e0, nv, -INFINITY);
+                if (amask.p) {
+                    // every (head, sample) re-reads the mask: plain loads, it stays in cache
+                    F8 am = load8(amask, oam, e0, nv, 0.f);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f.v[i] = f.v[i] * scale + am.v[i] * mscale;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) f.v[i] = f.v[i] * scale;
+                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    x[r][c][i] = f.v[i] * scale;
+                    x[r][c][i] = f.v[i];
                     m[r] = fmaxf(m[r], x[r][c][i]);
                 }
             }
@@ -350,8 +364,8 @@ inline unsigned check_rows(const RowSpace& rs, const char* what) {
         }                                                                          \
     } while (0)
 
-void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, float scale,
-                    PhiloxKey key, hipStream_t st) {
+void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, View amask,
+                    float scale, float mscale, PhiloxKey key, hipStream_t st) {
     unsigned nrows = check_rows(rs, "softmax");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax");
@@ -360,14 +374,14 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
         // short rows: two or four side by side in every wave
         if (rs.R <= 128)
             hipLaunchKernelGGL((k_softmax<1, 4, true, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs,
-                               beta, alpha, mask, drop, scale, key, nrows);
+                               beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
         else
             hipLaunchKernelGGL((k_softmax<1, 4, true, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs,
-                               beta, alpha, mask, drop, scale, key, nrows);
+                               beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
         check_launch("softmax");
         return;
     }
-    SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, scale, key, nrows);
+    SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
     check_launch("softmax");
 }
 

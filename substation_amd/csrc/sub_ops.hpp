@@ -16,8 +16,9 @@ inline void check_launch(const char* what) {
 }
 
 // --- row operators (one wave per row, row held in registers) -----------------
-void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, float scale,
-                    PhiloxKey key, hipStream_t st);
+// amask: optional additive attention mask over (query, key) positions (p == nullptr: none)
+void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, View amask,
+                    float scale, float mscale, PhiloxKey key, hipStream_t st);
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st);
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,

@@ -20,6 +20,11 @@ from . import layouts as _lay
 _SUPPORTED_DTYPES = (torch.float16,)
 
 
+def causal_mask(seq_len, device='cuda', dtype=torch.float16):
+    """-inf above the diagonal, 0 elsewhere (gen_attn_mask, substation/transformer.py:151-157)."""
+    return torch.triu(torch.full((seq_len, seq_len), float('-inf'), dtype=dtype, device=device), diagonal=1)
+
+
 class Encoder(torch.nn.Module):
     """Optimized BERT encoder layer (pytorch_module/encoder.py:19-162)."""
 
@@ -156,6 +161,23 @@ class Encoder(torch.nn.Module):
         every forward call advances ``step`` by one."""
         self.seed = seed
         self._handle.set_rng(seed, step)
+
+    def set_attention_mask(self, mask, layout='JK'):
+        """Masked self-attention (the ``decoder`` layer of
+        substation/transformer.py:443-546): ``mask`` is an additive [L, L] fp16 CUDA
+        tensor over (query, key) positions, e.g. ``causal_mask(L)``; ``None``
+        clears it.  It is added to the raw scores, before the 1/sqrt(P) scaling
+        (substation/attention.py:65-68)."""
+        if mask is None:
+            self._attn_mask = None
+            self._handle.set_attention_mask(0)
+            return
+        L = self.max_seq_len
+        if not (mask.is_cuda and mask.dtype == self.torch_dtype and tuple(mask.shape) == (L, L)
+                and mask.is_contiguous()):
+            raise ValueError(f'the attention mask is a contiguous [{L}, {L}] fp16 CUDA tensor')
+        self._attn_mask = mask                 # keeps the memory alive
+        self._handle.set_attention_mask(mask.data_ptr(), layout)
 
     def use_device_step(self, counter=None):
         """Keeps the dropout step in device memory (a one-element int32 CUDA tensor,

@@ -49,7 +49,12 @@ class Ops:
         self.handle.set_rng(seed, step)
 
     def softmax(self, beta, l_beta, alpha, l_alpha, mask, l_mask, drop, l_drop, scale=1.0, p=0.0,
-                site=0):
+                site=0, attn_mask=None, l_attn_mask='JK', mask_scale=1.0):
+        if attn_mask is not None:
+            _lib.check(self.lib.sub_op_softmax_masked(
+                self._pre(), _p(beta), _s(l_beta), _p(alpha), _s(l_alpha), _p(mask), _s(l_mask), _p(drop),
+                _s(l_drop), _p(attn_mask), _s(l_attn_mask), scale, mask_scale, p, site), 'softmax')
+            return
         _lib.check(self.lib.sub_op_softmax(self._pre(), _p(beta), _s(l_beta), _p(alpha), _s(l_alpha),
                                            _p(mask), _s(l_mask), _p(drop), _s(l_drop), scale, p, site),
                    'softmax')

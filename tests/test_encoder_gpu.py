@@ -29,7 +29,7 @@ def _all_layouts(lay):
 
 
 def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params_np=None,
-              X_np=None, DY_np=None, options=()):
+              X_np=None, DY_np=None, options=(), attn_mask=None):
     """Builds the module, runs forward+backward, returns (oracle dict, device dict)."""
     from substation_amd import Encoder
     lay = _layouts(which)
@@ -39,6 +39,8 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
     enc.set_rng(SEED, step)
     for option, value in options:
         enc._handle.set_option(option, value)
+    if attn_mask is not None:
+        enc.set_attention_mask(torch.from_numpy(attn_mask).half().cuda())
     sz = enc.sizes
     rng = np.random.default_rng(seed_data)
     if params_np is None:
@@ -85,7 +87,7 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
     # pre-activation that fp16 rounds across 0 would otherwise flip whole
     # gradient elements (see oracle.encoder_ref.encoder_backward).
     gate = (got['LIN1'] > 0).astype(np.float64) if act == 'relu' else None
-    want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate)
+    want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate, attn_mask=attn_mask)
     if gate is not None:
         flips = (gate != (want['LIN1'] > 0)).mean()
         assert flips < 1e-3, f'{flips:.2e} of the ReLU gates differ from the oracle forward'
@@ -142,6 +144,21 @@ def test_layer_random_layouts(seed):
     lay = _random_layouts(100 + seed)
     want, got = run_layer(2, 32, 2, 64, lay, 0.1, 'relu' if seed % 2 else 'gelu', seed_data=10 + seed)
     _compare(want, got)
+
+
+@pytest.mark.parametrize('which', ['mi355x', 'bert-b8-l512-h16-e1024'])
+def test_layer_with_causal_attention_mask(which):
+    """Masked self-attention layer (`decoder`, substation/transformer.py:443-546):
+    the encoder layer with an additive causal mask on the scores."""
+    L = 32
+    mask = ref.gen_attn_mask(L, L)
+    want, got = run_layer(2, L, 2, 64, which, 0.1, 'gelu', seed_data=31, attn_mask=mask)
+    iu = np.triu_indices(L, 1)
+    assert (got['ALPHA'][..., iu[0], iu[1]] == 0).all()
+    _compare(want, got)
+    # the unmasked layer on the same inputs differs: the mask is really applied
+    _, plain = run_layer(2, L, 2, 64, which, 0.1, 'gelu', seed_data=31)
+    assert np.abs(plain['SB2'] - got['SB2']).max() > 1e-2
 
 
 def test_layer_odd_sizes_scalar_paths():

@@ -72,6 +72,33 @@ def test_softmax_and_backward(B, L, H, E, p):
                      name='DBETA ' + lin)
 
 
+@pytest.mark.parametrize('B,L,H,E', [(2, 16, 2, 32), (2, 128, 4, 512), (8, 128, 16, 64), (3, 40, 2, 16)])
+def test_softmax_with_attention_mask(B, L, H, E):
+    """alpha = softmax(scale * beta + mask_scale * attn_mask) with a causal mask
+    plus finite entries, in both mask layouts; the backward operator needs no mask."""
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(2)
+    beta = h16(rng.normal(size=(H, B, L, L)) * 2)
+    am = h16(np.triu(np.full((L, L), -np.inf), k=1) + np.tril(rng.normal(size=(L, L))))
+    scale, mscale, p = 0.25, 0.5, 0.3
+    want_mask = ph.dropout_mask((H, B, L, L), p, SEED, ph.SITE_SOFTMAX, step=1)
+    x = scale * beta + mscale * am[None, None]
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    alpha_w = e / e.sum(axis=-1, keepdims=True)
+    for lay, lam in (('HBJK', 'JK'), ('BHJK', 'KJ'), ('JBHK', 'JK')):
+        o.set_rng(SEED, 1)
+        a, m, d = o.empty(lay), o.empty(lay), o.empty(lay)
+        t_am = torch.from_numpy(am if lam == 'JK' else am.T.copy()).half().cuda()
+        o.softmax(to_layout(beta, 'HBJK', lay), lay, a, lay, m, lay, d, lay, scale=scale, p=p, site=0,
+                  attn_mask=t_am, l_attn_mask=lam, mask_scale=mscale)
+        torch.cuda.synchronize()
+        got = from_layout(a, 'HBJK', lay)
+        assert (from_layout(m, 'HBJK', lay) == want_mask).all()
+        assert (got[..., np.triu_indices(L, 1)[0], np.triu_indices(L, 1)[1]] == 0).all()   # future positions
+        assert_close(got, alpha_w, name='ALPHA masked ' + lay)
+        assert (from_layout(d, 'HBJK', lay) == got * want_mask).all()
+
+
 @pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 8, 1, 1024), (1, 4, 1, 4096), (2, 3, 1, 20)])
 @pytest.mark.parametrize('p', [0.0, 0.3])
 def test_bdrln_and_blnrd(B, L, H, E, p):

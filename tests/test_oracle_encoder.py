@@ -18,7 +18,8 @@ def _np(d):
 
 
 @pytest.mark.parametrize('activation', ['relu', 'gelu'])
-def test_encoder_matches_torch_transformer_layer(activation):
+@pytest.mark.parametrize('masked', [False, True])
+def test_encoder_matches_torch_transformer_layer(activation, masked):
     params, X, DY = tg.make_inputs(B, L, H, E, seed=11, w_std=0.3, b_std=0.3)
     a = ref.module_params_to_numpy(_np(params))
     P = E // H
@@ -41,14 +42,23 @@ def test_encoder_matches_torch_transformer_layer(activation):
         layer.norm2.weight.copy_(params['S2']); layer.norm2.bias.copy_(params['B2'])
     x = X.clone().requires_grad_(True)
     layer.train()
-    y = layer(x)
+    scale = 1.0 / np.sqrt(P)
+    attn_mask = None
+    if masked:
+        # causal, plus finite entries below the diagonal so that the place where the
+        # mask enters (raw scores, before the scaling: attention.py:65-68) is pinned;
+        # torch adds its mask after the scaling
+        rng = np.random.default_rng(5)
+        attn_mask = ref.gen_attn_mask(L, L) + np.tril(rng.normal(size=(L, L)))
+        y = layer(x, src_mask=torch.from_numpy(scale * attn_mask))
+    else:
+        y = layer(x)
     y.backward(DY)
 
-    scale = 1.0 / np.sqrt(P)
     f = ref.encoder(X.numpy(), a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'],
                     a['attn_in_b'], a['attn_out_b'], scale, a['norm1_scale'], a['norm1_bias'],
                     a['norm2_scale'], a['norm2_bias'], a['linear1_w'], a['linear1_b'],
-                    a['linear2_w'], a['linear2_b'], activation=activation)
+                    a['linear2_w'], a['linear2_b'], activation=activation, attn_mask=attn_mask)
     g = ref.encoder_backward(X.numpy(), DY.numpy(), f, a['attn_wq'], a['attn_wk'], a['attn_wv'],
                              a['attn_wo'], scale, a['norm1_scale'], a['norm2_scale'],
                              a['linear1_w'], a['linear1_b'], a['linear2_w'], a['linear2_b'],
