@@ -27,7 +27,7 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
 // amask (optional, p == nullptr when absent): additive attention mask indexed by
 // (query position, key position) only, x = beta * scale + amask * mscale
 // (substation/attention.py:65-68 adds it before the scaling, hence mscale).
-template <int VPL, int RPW, bool FAST, int GRP = WAVE>
+template <int VPL, int RPW, bool FAST, int GRP = WAVE, bool MASKED = false>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
                                                    View drop, View amask, float scale, float mscale,
                                                    PhiloxKey key_, unsigned nrows) {
@@ -45,14 +45,14 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
             const bool live = row < nrows;
             ix[r] = row_index(rs, live ? row : row0);
             const long ob = view_offset(beta, ix[r]);
-            const long oam = amask.p ? view_offset(amask, ix[r]) : 0;
+            const long oam = MASKED ? view_offset(amask, ix[r]) : 0;
             m[r] = -INFINITY;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * GRP + gl) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
                 F8 f = ld8<FAST, true>(beta, ob, e0, nv, -INFINITY);
-                if (amask.p) {
+                if (MASKED) {
                     // every (head, sample) re-reads the mask: plain loads, it stays in cache
                     F8 am = load8(amask, oam, e0, nv, 0.f);
 #pragma unroll
@@ -370,14 +370,30 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax");
     bool fast = beta.vec && alpha.vec && mask.vec && drop.vec;
+    const bool masked = amask.p != nullptr;
     if (fast && rs.R <= 256 && nrows >= 256u * 16u * 4u) {
         // short rows: two or four side by side in every wave
-        if (rs.R <= 128)
-            hipLaunchKernelGGL((k_softmax<1, 4, true, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs,
-                               beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
-        else
-            hipLaunchKernelGGL((k_softmax<1, 4, true, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs,
-                               beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
+#define SUB_SM_SHORT(G, RPS, M)                                                                        \
+        hipLaunchKernelGGL((k_softmax<1, 4, true, G, M>), dim3(row_grid(nrows, RPS)), dim3(BLOCK), 0, st, rs, \
+                           beta, alpha, mask, drop, amask, scale, mscale, key, nrows)
+        if (rs.R <= 128) { if (masked) SUB_SM_SHORT(16, 16, true); else SUB_SM_SHORT(16, 16, false); }
+        else { if (masked) SUB_SM_SHORT(32, 8, true); else SUB_SM_SHORT(32, 8, false); }
+#undef SUB_SM_SHORT
+        check_launch("softmax");
+        return;
+    }
+    if (masked) {
+        // one row per wave; the mask rows are re-read by every head and sample from cache
+#define SUB_SM_MASKED(V, F)                                                                            \
+        hipLaunchKernelGGL((k_softmax<V, 1, F, WAVE, true>), dim3(row_grid(nrows, 1)), dim3(BLOCK), 0, st, rs, \
+                           beta, alpha, mask, drop, amask, scale, mscale, key, nrows)
+        switch (vpl) {
+            case 1: if (fast) SUB_SM_MASKED(1, true); else SUB_SM_MASKED(1, false); break;
+            case 2: if (fast) SUB_SM_MASKED(2, true); else SUB_SM_MASKED(2, false); break;
+            case 4: if (fast) SUB_SM_MASKED(4, true); else SUB_SM_MASKED(4, false); break;
+            default: if (fast) SUB_SM_MASKED(8, true); else SUB_SM_MASKED(8, false); break;
+        }
+#undef SUB_SM_MASKED
         check_launch("softmax");
         return;
     }
