@@ -166,6 +166,22 @@ def test_layer_odd_sizes_scalar_paths():
     _compare(want, got)
 
 
+@pytest.mark.parametrize('dims,act', [((8, 512, 16, 1024), 'relu'),      # BASELINE configs[2], the bench workload
+                                      ((96, 128, 16, 1024), 'relu'),     # configs[3]
+                                      ((1, 256, 32, 4096), 'gelu')])     # configs[4] widths (P=128, FF=16384), shorter
+def test_layer_full_size_configs(dims, act):
+    """The BASELINE workloads at their real sizes against the oracle, every tensor
+    (about 15 s and 11 GB of host memory each)."""
+    want, got = run_layer(*dims, 'mi355x', 0.1, act, seed_data=7, w_std=0.02 if dims[3] < 4096 else 0.01)
+    _compare(want, got)
+    # size-independent properties of the same run
+    assert np.abs(got['ALPHA'].sum(axis=-1) - 1).max() < 4e-3                 # softmax rows sum to 1
+    assert (got['ATTN_DROP'] == got['ALPHA'] * got['ATTN_DROP_MASK']).all()   # dropout is a product with the mask
+    assert np.abs(got['DBETA'].sum(axis=-1)).max() < 5e-2 * np.abs(got['DBETA']).max() * np.sqrt(dims[1])
+    n1 = got['LN1DIFF'] * got['LN1STD'][..., None]                            # normalised rows
+    assert np.abs(n1.mean(axis=-1)).max() < 2e-3 and np.abs(n1.var(axis=-1) - 1).max() < 2e-2
+
+
 def test_layer_config1_shape():
     """BASELINE config 1 shape (B=2, L=128, H=12, E=768) in fp16."""
     want, got = run_layer(2, 128, 12, 768, 'mi355x', 0.1, 'relu', seed_data=3, w_std=0.02)

@@ -72,6 +72,31 @@ def test_softmax_and_backward(B, L, H, E, p):
                      name='DBETA ' + lin)
 
 
+def test_softmax_baseline_config_full_size():
+    """BASELINE configs[1]: scores [H=16,B=8,J=512,K=512] ~ N(0,1), scale 1/sqrt(64),
+    p=0.1 seeded, forward plus softmax backward with dY ~ N(0,1), at full size."""
+    B, L, H, E = 8, 512, 16, 1024
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(1002)
+    beta = h16(rng.normal(size=(H, B, L, L)))
+    ddrop = h16(rng.normal(size=(H, B, L, L)))
+    scale, p, lay = 0.125, 0.1, 'HBJK'
+    want_mask = ph.dropout_mask((H, B, L, L), p, SEED, ph.SITE_SOFTMAX, step=0)
+    o.set_rng(SEED, 0)
+    a, m, d, db = o.empty(lay), o.empty(lay), o.empty(lay), o.empty(lay)
+    o.softmax(to_layout(beta, lay, lay), lay, a, lay, m, lay, d, lay, scale=scale, p=p, site=0)
+    o.bs(a, lay, m, lay, to_layout(ddrop, lay, lay), lay, db, lay, scale=scale)
+    torch.cuda.synchronize()
+    alpha_w, drop_w = ref.op_softmax(beta, want_mask, scale)
+    alpha16 = from_layout(a, lay, lay)
+    assert (from_layout(m, lay, lay) == want_mask).all()
+    assert 0.099 < 1 - want_mask.mean() < 0.101
+    assert_close(alpha16, alpha_w, name='ALPHA')
+    assert (from_layout(d, lay, lay) == alpha16 * want_mask).all()
+    assert_close(from_layout(db, lay, lay), ref.op_bs(alpha16, want_mask, ddrop, scale), name='DBETA')
+    assert np.abs(alpha16.sum(axis=-1) - 1).max() < 4e-3
+
+
 @pytest.mark.parametrize('B,L,H,E', [(2, 16, 2, 32), (2, 128, 4, 512), (8, 128, 16, 64), (3, 40, 2, 16)])
 def test_softmax_with_attention_mask(B, L, H, E):
     """alpha = softmax(scale * beta + mask_scale * attn_mask) with a causal mask
