@@ -717,15 +717,21 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
 }
 
 // Block tile for a problem: 22 = 128x128, 42 = 256x128, 44 = 256x256, 21 = 128x64.
-int pick_tile(const GemmArgs& a, long batch) {
+int pick_tile(const GemmArgs& a, long batch, bool akc, bool bkc) {
     if (a.N <= 64) return 21;      // head-size wide outputs of the attention products
     // 256x256 tiles halve the L2->LDS traffic per flop; they pay once the output
-    // alone has enough of them for most of the 256 CUs (asynchronous kernel only:
-    // whole tiles, no split contraction).
-    static const int min44 = [] { const char* e = getenv("SUB_GEMM_MIN44"); return e ? atoi(e) : 192; }();
-    if (a.M % 256 == 0 && a.N % 256 == 0 && a.K1 % BK == 0 && a.splits == 1 &&
-        (long)(a.M / 256) * (a.N / 256) * batch >= min44)
-        return 44;
+    // alone has enough of them to keep most of the 256 CUs busy in every round of
+    // tiles (asynchronous kernel only: whole tiles, no split contraction).  With
+    // an operand that is read through the slower LDS transpose path the bar is
+    // higher: three quarters of a round is not enough then (measured).
+    static const int min44 = [] { const char* e = getenv("SUB_GEMM_MIN44"); return e ? atoi(e) : 0; }();
+    if (a.M % 256 == 0 && a.N % 256 == 0 && a.K1 % BK == 0 && a.splits == 1) {
+        const long tiles = (long)(a.M / 256) * (a.N / 256) * batch;
+        const long rounds = (tiles + 255) / 256;
+        const double fill = (double)tiles / (double)(rounds * 256);
+        const bool ok = min44 > 0 ? tiles >= min44 : fill >= ((akc && bkc) ? 0.7 : 0.9);
+        if (ok) return 44;
+    }
     return 22;
 }
 
@@ -818,7 +824,7 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             c.a.splits = pick_splits(c.a, batch, ws_floats);
             c.a.partial = ws;
         }
-        const int tile = force ? force : pick_tile(c.a, batch);
+        const int tile = force ? force : pick_tile(c.a, batch, akc, bkc);
         const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
         if (tile == 44) launch_mfma<4, 4, true>(c.a, akc, bkc, batch, true, st);
         else if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
