@@ -88,7 +88,9 @@ def algorithmic_work(B, L, H, E):
 def make_encoder(cfg, layouts_name, profiling=False, seed=0x5EED):
     import torch
     from substation_amd import Encoder, layouts as L
-    lay = (L.mi355x_layouts() if layouts_name == 'mi355x'
+    shipped = {(8, 512): 'bert-b8-l512-h16-e1024', (96, 128): 'bert-b96-l128-h16-e1024'}
+    lay = (L.mi355x_layouts(shipped.get((cfg['B'], cfg['L'])) if cfg['E'] == 1024 else None)
+           if layouts_name == 'mi355x'
            else L.reference_layouts('bert-b8-l512-h16-e1024' if cfg['L'] >= 512 else 'bert-b96-l128-h16-e1024'))
     enc = Encoder('unused', cfg['B'], cfg['L'], cfg['H'], cfg['E'], lay, torch.float16,
                   0.1, 0.1, 0.1, 0.1, profiling=profiling, activation=cfg['act'], seed=seed)
