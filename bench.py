@@ -68,6 +68,10 @@ def algorithmic_work(B, L, H, E):
         # single-launch forms: the scaled gradient is written but not read back
         # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
         'bsb+blnrd1': ('hbm', 7 * bji * 2), 'ebsb+blnrd2+baob': ('hbm', 9 * bji * 2),
+        # scores formed in place: the score tensor itself is neither written nor read
+        # (QKT + softmax: Q, K in, three score-sized tensors out; dX1gamma + bs: dO, V
+        # and two score-sized tensors in, one out)
+        'QKT+softmax': ('hbm', (3 * hbjk + 2 * bji) * 2), 'dX1gamma+bs': ('hbm', (3 * hbjk + 2 * bji) * 2),
     }
     tok = B * L
     proj = (2 * tok * 3 * E * E, 2 * (tok * E + 3 * E * E + 3 * tok * E))

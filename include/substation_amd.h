@@ -142,6 +142,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * intermediates; the bias / scale gradients are summed in a different order
  * (fp32), so results can differ from the separate launches in the last bit. */
 #define SUB_OPT_FUSE_LN_BACKWARD 2
+/* SUB_OPT_FUSE_SCORES (default 1): form the attention scores inside the softmax
+ * kernel (QK^T, encoder.cu:104-121) and the gradient of the dropped softmax
+ * inside the softmax-backward kernel (dO.V^T, encoder.cu:228-247), for sequence
+ * lengths 512 and 1024, head sizes 64 and 128 and feature-contiguous
+ * projections.  BETA and DATTN_DROP, which only those kernels consume, are then
+ * left unwritten; every other tensor is unchanged.  Set to 0 to materialise
+ * them (the Python module does so for debug capture). */
+#define SUB_OPT_FUSE_SCORES 3
 int sub_set_option(void* handle, int option, int value);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same

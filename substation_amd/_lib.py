@@ -16,6 +16,7 @@ ABI_VERSION = 1
 ACTIVATIONS = {'relu': 0, 'gelu': 1}
 OPT_FUSE_EPILOGUES = 1
 OPT_FUSE_LN_BACKWARD = 2
+OPT_FUSE_SCORES = 3
 
 
 class SubConfig(ctypes.Structure):

@@ -182,6 +182,7 @@ struct Handle {
     Layout l_attn_mask;
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
+    bool fuse_scores = true;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -515,6 +516,43 @@ void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     launch_baob(sp.rs, make_view(datt, l, sp), ColOut{(half_t*)dbo}, ws, h.stream, defer_of(h));
 }
 
+// Score rows straight from the projections: `ln` lays out the query-side rows
+// ([B,J,H,P]-like), `lm` the key-side rows (its sequence dim is K).
+bool score_args(const Handle& h, const void* rows_n, const Layout& ln, const void* rows_m, const Layout& lm,
+                float alpha, ScoreArgs& a) {
+    if (ln.rank != 4 || lm.rank != 4 || !ln.has[dP] || !lm.has[dP] || ln.stride[dP] != 1 || lm.stride[dP] != 1)
+        return false;
+    if (!ln.has[dJ] || !lm.has[dK] || !ln.has[dH] || !lm.has[dH] || !ln.has[dB] || !lm.has[dB]) return false;
+    a.rows_n = (const half_t*)rows_n; a.rows_m = (const half_t*)rows_m;
+    a.n_sh = ln.stride[dH]; a.n_sb = ln.stride[dB]; a.n_sr = ln.stride[dJ];
+    a.m_sh = lm.stride[dH]; a.m_sb = lm.stride[dB]; a.m_sr = lm.stride[dK];
+    a.alpha = alpha;
+    (void)h;
+    return true;
+}
+
+// QK^T + softmax + dropout in one launch (BETA is not written).
+bool op_scores_softmax(Handle& h, const void* qq, const void* kk, void* alpha, const Layout& la, void* mask,
+                       const Layout& lm, void* drop, const Layout& ld) {
+    if (h.attn_mask) return false;
+    ScoreArgs a;
+    if (!score_args(h, qq, h.lQQ, kk, h.lKK, h.gemm[G_QKT].alpha, a)) return false;
+    Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
+    View va = make_view(alpha, la, sp), vm = make_view(mask, lm, sp), vd = make_view(drop, ld, sp);
+    return launch_scores_softmax(sp.rs, a, (int)h.sz.n[dP], va, vm, vd,
+                                 make_key(h, SUB_SITE_SOFTMAX, h.p_softmax), h.stream);
+}
+
+// dO.V^T + softmax backward in one launch (DATTN_DROP is not written).
+bool op_dscores_bs(Handle& h, const void* dgamma, const void* vv, const void* alpha, const Layout& la,
+                   const void* mask, const Layout& lm, void* dbeta, const Layout& lo) {
+    ScoreArgs a;
+    if (!score_args(h, dgamma, h.lb[DGAMMA], vv, h.lKK, 1.f, a)) return false;
+    Space sp = make_space(h.sz, {dH, dB, dJ}, dK);
+    View va = make_view(alpha, la, sp), vm = make_view(mask, lm, sp), vo = make_view(dbeta, lo, sp);
+    return launch_dscores_bs(sp.rs, a, (int)h.sz.n[dP], va, vm, vo, h.stream);
+}
+
 // bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
 // false, having done nothing, when the shape or the layouts rule the fused
 // kernel out; the caller then runs the separate operators.
@@ -630,8 +668,15 @@ void forward(Handle& h, const FwdPtrs& t) {
         op_aib(h, F[WKKWQQWVV], h.lf[WKKWQQWVV], W[BKQV], h.lp[BKQV], F[KKQQVV], h.lf[KKQQVV]);
     }
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
-    run_gemm(h, G_QKT, KK, QQ, F[BETA], "QKT");
-    {
+    bool fused_scores = false;
+    if (h.fuse_scores) {
+        ProfScope ps(h, "QKT+softmax");
+        fused_scores = op_scores_softmax(h, QQ, KK, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK],
+                                         h.lf[ATTN_DROP_MASK], F[ATTN_DROP], h.lf[ATTN_DROP]);
+        if (!fused_scores) ps.cancel();
+    }
+    if (!fused_scores) {
+        run_gemm(h, G_QKT, KK, QQ, F[BETA], "QKT");
         ProfScope ps(h, "softmax");
         op_softmax(h, F[BETA], h.lf[BETA], F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK],
                    F[ATTN_DROP], h.lf[ATTN_DROP], 1.0f, h.p_softmax, SUB_SITE_SOFTMAX, h.attn_mask,
@@ -737,9 +782,16 @@ void backward(Handle& h, const BwdPtrs& t) {
     run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
-    run_gemm(h, G_DX1GAMMA, VV, D[DGAMMA], D[DATTN_DROP], "dX1gamma");
     run_gemm(h, G_DX2GAMMA, D[DGAMMA], F[ATTN_DROP], DVV, "dX2gamma");
-    {
+    bool fused_scores = false;
+    if (h.fuse_scores) {
+        ProfScope ps(h, "dX1gamma+bs");
+        fused_scores = op_dscores_bs(h, D[DGAMMA], VV, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK],
+                                     h.lf[ATTN_DROP_MASK], D[DBETA], h.lb[DBETA]);
+        if (!fused_scores) ps.cancel();
+    }
+    if (!fused_scores) {
+        run_gemm(h, G_DX1GAMMA, VV, D[DGAMMA], D[DATTN_DROP], "dX1gamma");
         ProfScope ps(h, "bs");
         op_bs(h, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK], D[DATTN_DROP],
               h.lb[DATTN_DROP], D[DBETA], h.lb[DBETA], 1.0f);
@@ -919,6 +971,7 @@ int sub_set_option(void* handle, int option, int value) {
         Handle& h = as_handle(handle);
         if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
         else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
+        else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
         else fail("sub_set_option: unknown option");
     });
 }

@@ -1,0 +1,264 @@
+// Attention scores without their round trip through memory.
+//
+// The reference forms the scaled scores with a batched GEMM, writes them out
+// and reads them back in the softmax kernel (pytorch_module/encoder.cu:104-121:
+// Einsum -> BETA, then Softmax), and likewise in the backward pass writes
+// d(dropped softmax) and reads it back in BackwardSoftmax (encoder.cu:228-247).
+// A row of scores is only head_size long in its contraction, so a workgroup can
+// form a block of 32 complete rows with MFMA straight from the projections
+// (operand fragments are loaded from global memory in MFMA layout, no LDS),
+// park it in LDS as fp16 -- the same rounding the stored tensor would get -- and
+// run the row operator on it.  Everything the row operator writes is written as
+// before; only the score tensor itself (BETA, resp. DATTN_DROP) is not.
+//
+//   forward : S = alpha * Q.K^T        -> softmax + dropout -> ALPHA, mask, ATTN_DROP
+//   backward: G = dO.V^T               -> softmax backward  -> DBETA
+#include "sub_ops.hpp"
+
+namespace sub {
+
+namespace {
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+constexpr int BLOCK = 256;
+constexpr int WPB = BLOCK / WAVE;
+constexpr int ROWS = 32;                  // score rows per workgroup (one MFMA tile high)
+constexpr float LOG2E = 1.4426950408889634f;
+
+// 32 rows (queries j0..j0+31 of one head and sample) x R keys of scores into
+// `stage` ([32][R + 8] fp16).  Each wave forms the columns of its quarter of the
+// keys: NT MFMA tiles of 32 keys, contraction over the P features of a head.
+template <int P, int NT>
+__device__ __forceinline__ void score_block(const ScoreArgs& a, unsigned h, unsigned b, unsigned j0, int wave,
+                                            int lane, half_t* stage, int pitch) {
+    constexpr int KS = P / 16;
+    const int l32 = lane & 31, hi = lane >> 5;
+    f16v acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
+    // B operand: lane holds 8 consecutive features of query row j0 + l32
+    const half_t* qrow = a.rows_n + (long)h * a.n_sh + (long)b * a.n_sb + (long)(j0 + l32) * a.n_sr + hi * 8;
+    h8 fq[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) fq[ks] = *reinterpret_cast<const h8*>(qrow + ks * 16);
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        // A operand: lane holds 8 consecutive features of key row (wave's tile t) + l32
+        const half_t* krow = a.rows_m + (long)h * a.m_sh + (long)b * a.m_sb +
+                             (long)((wave * NT + t) * 32 + l32) * a.m_sr + hi * 8;
+        h8 fk[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) fk[ks] = *reinterpret_cast<const h8*>(krow + ks * 16);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], acc[t], 0, 0, 0);
+    }
+    // D[key, query]: lane = query row l32, registers = keys q*8 + hi*4 + 0..3 of the tile
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            h4 w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[t][q * 4 + e] * a.alpha);
+            *reinterpret_cast<h4*>(stage + l32 * pitch + (wave * NT + t) * 32 + q * 8 + hi * 4) = w;
+        }
+}
+
+// grid.x = (heads * samples * queries) / 32.  Row numbering is the canonical one
+// of the [H,B,J,K] tensors (rs = {1, H, B, J} x K, not merged).
+template <int P, int NT>
+__global__ __launch_bounds__(BLOCK) void k_scores_softmax(RowSpace rs, ScoreArgs a, View alpha, View mask,
+                                                          View drop, PhiloxKey key_) {
+    constexpr int R = 128 * NT;
+    constexpr int VPL = (R + 511) / 512;
+    constexpr int PITCH = R + 8;
+    constexpr int RPW = ROWS / WPB;          // 8 rows per wave, taken 4 at a time
+    __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
+    const PhiloxKey key = resolved(key_);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned row_base = blockIdx.x * ROWS;
+    {
+        const RowIdx ix0 = row_index(rs, row_base);
+        score_block<P, NT>(a, ix0.i1, ix0.i2, ix0.i3, wave, lane, stage, PITCH);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int half_ = 0; half_ < RPW / 4; ++half_) {
+        float x[4][VPL][8];
+        float m[4], s[4];
+        RowIdx ix[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int rl = wave * RPW + half_ * 4 + r;
+            ix[r] = row_index(rs, row_base + rl);
+            m[r] = -INFINITY;
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                const int e0 = (c * WAVE + lane) * 8;
+                if (e0 < R) {
+                    h8 v = *reinterpret_cast<const h8*>(stage + rl * PITCH + e0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) { x[r][c][i] = (float)v[i]; m[r] = fmaxf(m[r], x[r][c][i]); }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) x[r][c][i] = -INFINITY;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m[r] = wave_max(m[r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            s[r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VPL; ++c)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    x[r][c][i] = __builtin_amdgcn_exp2f((x[r][c][i] - m[r]) * LOG2E);
+                    s[r] += x[r][c][i];
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const unsigned row = row_base + wave * RPW + half_ * 4 + r;
+            const float inv = 1.0f / s[r];
+            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                const int e0 = (c * WAVE + lane) * 8;
+                if (e0 >= R) continue;
+                h8 al, d;
+                const uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)R + (uint64_t)e0);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) al[i] = (half_t)(x[r][c][i] * inv);
+                al = pin(al);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) d[i] = ((bits >> i) & 1u) ? al[i] : (half_t)0.0f;
+                stg8<true>(alpha.p + oa + e0, al);
+                stg8<true>(mask.p + om + e0, mask_h8(bits));
+                stg8<false>(drop.p + od + e0, d);
+            }
+        }
+    }
+}
+
+template <int P, int NT>
+__global__ __launch_bounds__(BLOCK) void k_dscores_bs(RowSpace rs, ScoreArgs a, View alpha, View mask, View dbeta) {
+    constexpr int R = 128 * NT;
+    constexpr int VPL = (R + 511) / 512;
+    constexpr int PITCH = R + 8;
+    constexpr int RPW = ROWS / WPB;
+    __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned row_base = blockIdx.x * ROWS;
+    {
+        const RowIdx ix0 = row_index(rs, row_base);
+        score_block<P, NT>(a, ix0.i1, ix0.i2, ix0.i3, wave, lane, stage, PITCH);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int half_ = 0; half_ < RPW / 4; ++half_) {
+        float al[4][VPL][8], g[4][VPL][8];
+        float s[4];
+        RowIdx ix[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int rl = wave * RPW + half_ * 4 + r;
+            ix[r] = row_index(rs, row_base + rl);
+            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]);
+            s[r] = 0.f;
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                const int e0 = (c * WAVE + lane) * 8;
+                h8 va = (h8)(half_t)0.0f, vm = (h8)(half_t)0.0f, vd = (h8)(half_t)0.0f;
+                if (e0 < R) {
+                    va = ldg8<true>(alpha.p + oa + e0);
+                    vm = ldg8<true>(mask.p + om + e0);
+                    vd = *reinterpret_cast<const h8*>(stage + rl * PITCH + e0);
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    al[r][c][i] = (float)va[i];
+                    g[r][c][i] = (float)vm[i] * (float)vd[i];
+                    s[r] += al[r][c][i] * g[r][c][i];
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const long oo = view_offset(dbeta, ix[r]);
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                const int e0 = (c * WAVE + lane) * 8;
+                if (e0 >= R) continue;
+                h8 o;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) o[i] = (half_t)(1.0f * al[r][c][i] * (g[r][c][i] - s[r]));
+                stg8<false>(dbeta.p + oo + e0, o);
+            }
+        }
+    }
+}
+
+template <int P>
+bool dispatch_fwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
+                  View drop, PhiloxKey key) {
+    switch (R) {
+        case 512: hipLaunchKernelGGL((k_scores_softmax<P, 4>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, drop, key); return true;
+        case 1024: hipLaunchKernelGGL((k_scores_softmax<P, 8>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, drop, key); return true;
+        default: return false;
+    }
+}
+template <int P>
+bool dispatch_bwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
+                  View dbeta) {
+    switch (R) {
+        case 512: hipLaunchKernelGGL((k_dscores_bs<P, 4>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, dbeta); return true;
+        case 1024: hipLaunchKernelGGL((k_dscores_bs<P, 8>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, dbeta); return true;
+        default: return false;
+    }
+}
+
+}  // namespace
+
+bool scores_fusable(const RowSpace& rs, const ScoreArgs& a, int P, std::initializer_list<const View*> views) {
+    if (rs.n0 != 1 || rs.flat) return false;                       // rows numbered over (H, B, J)
+    if (rs.R != 512 && rs.R != 1024) return false;
+    if (P != 64 && P != 128) return false;
+    if (rs.n3 % ROWS != 0) return false;                           // a block of rows shares head and sample
+    if (rs.rows() <= 0 || rs.rows() / ROWS > 0x7fffffffL) return false;
+    for (const View* v : views) if (!v->vec) return false;
+    auto al = [](const void* p, long s1, long s2, long s3) {
+        return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && s1 % 8 == 0 && s2 % 8 == 0 && s3 % 8 == 0;
+    };
+    return al(a.rows_n, a.n_sh, a.n_sb, a.n_sr) && al(a.rows_m, a.m_sh, a.m_sb, a.m_sr);
+}
+
+bool launch_scores_softmax(const RowSpace& rs, const ScoreArgs& a, int P, View alpha, View mask, View drop,
+                           PhiloxKey key, hipStream_t st) {
+    if (!scores_fusable(rs, a, P, {&alpha, &mask, &drop})) return false;
+    dim3 grid((unsigned)(rs.rows() / ROWS));
+    bool ok = P == 64 ? dispatch_fwd<64>(rs.R, grid, st, rs, a, alpha, mask, drop, key)
+                      : dispatch_fwd<128>(rs.R, grid, st, rs, a, alpha, mask, drop, key);
+    if (ok) check_launch("scores + softmax");
+    return ok;
+}
+
+bool launch_dscores_bs(const RowSpace& rs, const ScoreArgs& a, int P, View alpha, View mask, View dbeta,
+                       hipStream_t st) {
+    if (!scores_fusable(rs, a, P, {&alpha, &mask, &dbeta})) return false;
+    dim3 grid((unsigned)(rs.rows() / ROWS));
+    bool ok = P == 64 ? dispatch_bwd<64>(rs.R, grid, st, rs, a, alpha, mask, dbeta)
+                      : dispatch_bwd<128>(rs.R, grid, st, rs, a, alpha, mask, dbeta);
+    if (ok) check_launch("d(scores) + softmax backward");
+    return ok;
+}
+
+}  // namespace sub

@@ -87,6 +87,24 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
 // Row sums: out[row-group] = sum over (n3, R) for each (n0,n1,n2): baib.
 void launch_baib(const RowSpace& rs, View d, View out, hipStream_t st);
 
+// --- attention scores formed in place (no round trip of the score tensor) -----
+// rows_n: one row of head_size features per query position, rows_m: per key
+// position; strides over (head, sample, position); the feature dim is contiguous.
+struct ScoreArgs {
+    const half_t* rows_n; const half_t* rows_m;
+    long n_sh, n_sb, n_sr;
+    long m_sh, m_sb, m_sr;
+    float alpha;                 // scores = alpha * rows_n . rows_m^T, rounded to fp16
+};
+// Both return false, having launched nothing, when the shape or the layouts rule
+// the fused kernel out.  rs: rows over (H, B, J), row length K, not merged.
+// scores -> softmax -> dropout: writes alpha, mask, drop.
+bool launch_scores_softmax(const RowSpace& rs, const ScoreArgs& a, int head_size, View alpha, View mask,
+                           View drop, PhiloxKey key, hipStream_t st);
+// d(dropped softmax) = rows_n . rows_m^T -> softmax backward: writes dbeta.
+bool launch_dscores_bs(const RowSpace& rs, const ScoreArgs& a, int head_size, View alpha, View mask,
+                       View dbeta, hipStream_t st);
+
 // --- tensor contraction ------------------------------------------------------
 // Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
 // that broadcasts along M or N, or a whole tensor (a residual).

@@ -79,6 +79,7 @@ class Encoder(torch.nn.Module):
             # debug capture promises every named intermediate: keep the separate
             # aib / bei operators instead of fusing them into GEMM epilogues
             self._handle.set_option(_lib.OPT_FUSE_EPILOGUES, 0)
+            self._handle.set_option(_lib.OPT_FUSE_SCORES, 0)
         handle = self._handle
         lib = handle.lib
         module = self

@@ -17,6 +17,7 @@ from . import layouts as _lay
 OPERATORS = [
     ('QKV-fused', 'fwd', ('X', 'WKQV', 'BKQV', 'WKKWQQWVV', 'KKQQVV')),
     ('aib', 'fwd', ('WKKWQQWVV', 'BKQV', 'KKQQVV')),
+    ('QKT+softmax', 'fwd', ('KKQQVV', 'BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP')),
     ('QKT', 'fwd', ('KKQQVV', 'BETA')),
     ('softmax', 'fwd', ('BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP')),
     ('gamma', 'fwd', ('KKQQVV', 'ATTN_DROP', 'GAMMA')),
@@ -41,6 +42,7 @@ OPERATORS = [
     ('baob', 'bwd', ('DATT',)),
     ('dWout', 'bwd', ('GAMMA', 'DATT', 'WO')),
     ('dXout', 'bwd', ('WO', 'DATT', 'DGAMMA')),
+    ('dX1gamma+bs', 'bwd', ('KKQQVV', 'DGAMMA', 'DATTN_DROP', 'ALPHA', 'ATTN_DROP_MASK', 'DBETA')),
     ('dX1gamma', 'bwd', ('KKQQVV', 'DGAMMA', 'DATTN_DROP')),
     ('dX2gamma', 'bwd', ('DGAMMA', 'ATTN_DROP', 'DKKQQVV')),
     ('bs', 'bwd', ('ALPHA', 'ATTN_DROP_MASK', 'DATTN_DROP', 'DBETA')),
@@ -60,6 +62,8 @@ OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused', 'bei'),
+    ('QKT+softmax', 'QKT', 'softmax'),
+    ('dX1gamma+bs', 'dX1gamma', 'bs'),
     ('bsb+blnrd1', 'bsb', 'blnrd1'),
     ('ebsb+blnrd2+baob', 'ebsb', 'blnrd2', 'baob'),
 ]
