@@ -20,70 +20,86 @@ namespace sub {
 namespace {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
-constexpr int BLOCK = 256;
-constexpr int WPB = BLOCK / WAVE;
 constexpr int ROWS = 32;                  // score rows per workgroup (one MFMA tile high)
 constexpr float LOG2E = 1.4426950408889634f;
 
-// 32 rows (queries j0..j0+31 of one head and sample) x R keys of scores into
-// `stage` ([32][R + 8] fp16).  Each wave forms the columns of its quarter of the
-// keys: NT MFMA tiles of 32 keys, contraction over the P features of a head.
+// The key-side MFMA operand of one wave: its quarter of the keys (NT tiles of 32),
+// all P features, kept in registers and reused for every block of query rows the
+// workgroup goes through (lane = key row, 8 consecutive features per k-step).
 template <int P, int NT>
-__device__ __forceinline__ void score_block(const ScoreArgs& a, unsigned h, unsigned b, unsigned j0, int wave,
-                                            int lane, half_t* stage, int pitch) {
-    constexpr int KS = P / 16;
+__device__ __forceinline__ void load_keys(const ScoreArgs& a, unsigned h, unsigned b, int wave, int lane,
+                                          h8 (&fk)[NT][P / 16]) {
     const int l32 = lane & 31, hi = lane >> 5;
-    f16v acc[NT];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[t][v] = 0.f;
-    // B operand: lane holds 8 consecutive features of query row j0 + l32
-    const half_t* qrow = a.rows_n + (long)h * a.n_sh + (long)b * a.n_sb + (long)(j0 + l32) * a.n_sr + hi * 8;
-    h8 fq[KS];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) fq[ks] = *reinterpret_cast<const h8*>(qrow + ks * 16);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        // A operand: lane holds 8 consecutive features of key row (wave's tile t) + l32
         const half_t* krow = a.rows_m + (long)h * a.m_sh + (long)b * a.m_sb +
                              (long)((wave * NT + t) * 32 + l32) * a.m_sr + hi * 8;
-        h8 fk[KS];
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) fk[ks] = *reinterpret_cast<const h8*>(krow + ks * 16);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-            acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], acc[t], 0, 0, 0);
+        for (int ks = 0; ks < P / 16; ++ks) fk[t][ks] = *reinterpret_cast<const h8*>(krow + ks * 16);
     }
-    // D[key, query]: lane = query row l32, registers = keys q*8 + hi*4 + 0..3 of the tile
+}
+
+template <int P>
+__device__ __forceinline__ void load_queries(const ScoreArgs& a, unsigned h, unsigned b, unsigned j0, int lane,
+                                             h8 (&fq)[P / 16]) {
+    const int l32 = lane & 31, hi = lane >> 5;
+    const half_t* qrow = a.rows_n + (long)h * a.n_sh + (long)b * a.n_sb + (long)(j0 + l32) * a.n_sr + hi * 8;
 #pragma unroll
-    for (int t = 0; t < NT; ++t)
+    for (int ks = 0; ks < P / 16; ++ks) fq[ks] = *reinterpret_cast<const h8*>(qrow + ks * 16);
+}
+
+// 32 query rows x R keys of scores into `stage` ([32][R + 8] fp16): each wave
+// forms the columns of its quarter of the keys, contraction over the P features.
+template <int P, int NT>
+__device__ __forceinline__ void score_tile(const h8 (&fk)[NT][P / 16], const h8 (&fq)[P / 16], float alpha,
+                                           int wave, int lane, half_t* stage, int pitch) {
+    const int l32 = lane & 31, hi = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        f16v acc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < P / 16; ++ks)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[t][ks], fq[ks], acc, 0, 0, 0);
+        // D[key, query]: lane = query row l32, registers = keys q*8 + hi*4 + 0..3 of the tile
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             h4 w;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[t][q * 4 + e] * a.alpha);
+            for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[q * 4 + e] * alpha);
             *reinterpret_cast<h4*>(stage + l32 * pitch + (wave * NT + t) * 32 + q * 8 + hi * 4) = w;
         }
+    }
 }
 
-// grid.x = (heads * samples * queries) / 32.  Row numbering is the canonical one
+// Rows per workgroup: TILES blocks of 32 query rows of one head and sample, gone
+// through one after the other with the key fragments held in registers.
+constexpr int TILES = 4;
+
+// grid.x = (heads * samples * queries) / (32 * TILES).  Row numbering is the canonical one
 // of the [H,B,J,K] tensors (rs = {1, H, B, J} x K, not merged).
-template <int P, int NT>
-__global__ __launch_bounds__(BLOCK) void k_scores_softmax(RowSpace rs, ScoreArgs a, View alpha, View mask,
-                                                          View drop, PhiloxKey key_) {
-    constexpr int R = 128 * NT;
+// NW waves per workgroup, each forming NT tiles of 32 keys: R = 32 * NT * NW.
+template <int P, int NT, int NW>
+__global__ __launch_bounds__(NW * WAVE) void k_scores_softmax(RowSpace rs, ScoreArgs a, View alpha, View mask,
+                                                              View drop, PhiloxKey key_) {
+    constexpr int R = 32 * NT * NW;
+    constexpr int WPB = NW;
     constexpr int VPL = (R + 511) / 512;
     constexpr int PITCH = R + 8;
-    constexpr int RPW = ROWS / WPB;          // 8 rows per wave, taken 4 at a time
+    constexpr int RPW = ROWS / WPB;          // rows per wave, taken 4 at a time
     __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
     const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned row_base = blockIdx.x * ROWS;
-    {
-        const RowIdx ix0 = row_index(rs, row_base);
-        score_block<P, NT>(a, ix0.i1, ix0.i2, ix0.i3, wave, lane, stage, PITCH);
-    }
+    const RowIdx ixb = row_index(rs, blockIdx.x * (ROWS * TILES));
+    h8 fk[NT][P / 16], fq[P / 16];
+    load_keys<P, NT>(a, ixb.i1, ixb.i2, wave, lane, fk);
+    load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3, lane, fq);
+    for (int tile = 0; tile < TILES; ++tile) {
+    const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
+    if (tile) __syncthreads();                 // the previous tile's rows have been read
+    score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
+    if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
     __syncthreads();
 #pragma unroll
     for (int half_ = 0; half_ < RPW / 4; ++half_) {
@@ -145,21 +161,27 @@ __global__ __launch_bounds__(BLOCK) void k_scores_softmax(RowSpace rs, ScoreArgs
             }
         }
     }
+    }
 }
 
-template <int P, int NT>
-__global__ __launch_bounds__(BLOCK) void k_dscores_bs(RowSpace rs, ScoreArgs a, View alpha, View mask, View dbeta) {
-    constexpr int R = 128 * NT;
+template <int P, int NT, int NW>
+__global__ __launch_bounds__(NW * WAVE) void k_dscores_bs(RowSpace rs, ScoreArgs a, View alpha, View mask, View dbeta) {
+    constexpr int R = 32 * NT * NW;
+    constexpr int WPB = NW;
     constexpr int VPL = (R + 511) / 512;
     constexpr int PITCH = R + 8;
     constexpr int RPW = ROWS / WPB;
     __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const unsigned row_base = blockIdx.x * ROWS;
-    {
-        const RowIdx ix0 = row_index(rs, row_base);
-        score_block<P, NT>(a, ix0.i1, ix0.i2, ix0.i3, wave, lane, stage, PITCH);
-    }
+    const RowIdx ixb = row_index(rs, blockIdx.x * (ROWS * TILES));
+    h8 fk[NT][P / 16], fq[P / 16];
+    load_keys<P, NT>(a, ixb.i1, ixb.i2, wave, lane, fk);
+    load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3, lane, fq);
+    for (int tile = 0; tile < TILES; ++tile) {
+    const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
+    if (tile) __syncthreads();
+    score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
+    if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
     __syncthreads();
 #pragma unroll
     for (int half_ = 0; half_ < RPW / 4; ++half_) {
@@ -205,14 +227,15 @@ __global__ __launch_bounds__(BLOCK) void k_dscores_bs(RowSpace rs, ScoreArgs a, 
             }
         }
     }
+    }
 }
 
 template <int P>
 bool dispatch_fwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
                   View drop, PhiloxKey key) {
     switch (R) {
-        case 512: hipLaunchKernelGGL((k_scores_softmax<P, 4>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, drop, key); return true;
-        case 1024: hipLaunchKernelGGL((k_scores_softmax<P, 8>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, drop, key); return true;
+        case 512: hipLaunchKernelGGL((k_scores_softmax<P, 4, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
+        case 1024: hipLaunchKernelGGL((k_scores_softmax<P, 8, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
         default: return false;
     }
 }
@@ -220,8 +243,8 @@ template <int P>
 bool dispatch_bwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
                   View dbeta) {
     switch (R) {
-        case 512: hipLaunchKernelGGL((k_dscores_bs<P, 4>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, dbeta); return true;
-        case 1024: hipLaunchKernelGGL((k_dscores_bs<P, 8>), grid, dim3(BLOCK), 0, st, rs, a, alpha, mask, dbeta); return true;
+        case 512: hipLaunchKernelGGL((k_dscores_bs<P, 4, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
+        case 1024: hipLaunchKernelGGL((k_dscores_bs<P, 8, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
         default: return false;
     }
 }
@@ -232,8 +255,8 @@ bool scores_fusable(const RowSpace& rs, const ScoreArgs& a, int P, std::initiali
     if (rs.n0 != 1 || rs.flat) return false;                       // rows numbered over (H, B, J)
     if (rs.R != 512 && rs.R != 1024) return false;
     if (P != 64 && P != 128) return false;
-    if (rs.n3 % ROWS != 0) return false;                           // a block of rows shares head and sample
-    if (rs.rows() <= 0 || rs.rows() / ROWS > 0x7fffffffL) return false;
+    if (rs.n3 % (ROWS * TILES) != 0) return false;                 // a workgroup's rows share head and sample
+    if (rs.rows() <= 0 || rs.rows() / (ROWS * TILES) > 0x7fffffffL) return false;
     for (const View* v : views) if (!v->vec) return false;
     auto al = [](const void* p, long s1, long s2, long s3) {
         return (reinterpret_cast<uintptr_t>(p) & 15) == 0 && s1 % 8 == 0 && s2 % 8 == 0 && s3 % 8 == 0;
@@ -244,7 +267,7 @@ bool scores_fusable(const RowSpace& rs, const ScoreArgs& a, int P, std::initiali
 bool launch_scores_softmax(const RowSpace& rs, const ScoreArgs& a, int P, View alpha, View mask, View drop,
                            PhiloxKey key, hipStream_t st) {
     if (!scores_fusable(rs, a, P, {&alpha, &mask, &drop})) return false;
-    dim3 grid((unsigned)(rs.rows() / ROWS));
+    dim3 grid((unsigned)(rs.rows() / (ROWS * TILES)));
     bool ok = P == 64 ? dispatch_fwd<64>(rs.R, grid, st, rs, a, alpha, mask, drop, key)
                       : dispatch_fwd<128>(rs.R, grid, st, rs, a, alpha, mask, drop, key);
     if (ok) check_launch("scores + softmax");
@@ -254,7 +277,7 @@ bool launch_scores_softmax(const RowSpace& rs, const ScoreArgs& a, int P, View a
 bool launch_dscores_bs(const RowSpace& rs, const ScoreArgs& a, int P, View alpha, View mask, View dbeta,
                        hipStream_t st) {
     if (!scores_fusable(rs, a, P, {&alpha, &mask, &dbeta})) return false;
-    dim3 grid((unsigned)(rs.rows() / ROWS));
+    dim3 grid((unsigned)(rs.rows() / (ROWS * TILES)));
     bool ok = P == 64 ? dispatch_bwd<64>(rs.R, grid, st, rs, a, alpha, mask, dbeta)
                       : dispatch_bwd<128>(rs.R, grid, st, rs, a, alpha, mask, dbeta);
     if (ok) check_launch("d(scores) + softmax backward");
