@@ -79,154 +79,159 @@ constexpr int TILES = 4;
 
 // grid.x = (heads * samples * queries) / (32 * TILES).  Row numbering is the canonical one
 // of the [H,B,J,K] tensors (rs = {1, H, B, J} x K, not merged).
+// How the rows of a block are gone through by a wave: rows of up to 128 (256)
+// elements take a quarter (half) of a wave, so four (two) sit side by side.
+template <int R>
+struct RowPlan {
+    static constexpr int GRP = R >= 512 ? WAVE : R / 8;        // lanes per row
+    static constexpr int SPW = WAVE / GRP;                     // rows side by side
+    static constexpr int VPL = R > 512 ? R / 512 : 1;          // 8-packs per lane
+    static constexpr int RP = SPW == 1 ? 4 : (SPW == 2 ? 4 : 2);   // rows per lane group and pass
+    static constexpr int PER_PASS = RP * SPW;
+};
+
 // NW waves per workgroup, each forming NT tiles of 32 keys: R = 32 * NT * NW.
 template <int P, int NT, int NW>
 __global__ __launch_bounds__(NW * WAVE) void k_scores_softmax(RowSpace rs, ScoreArgs a, View alpha, View mask,
                                                               View drop, PhiloxKey key_) {
     constexpr int R = 32 * NT * NW;
-    constexpr int WPB = NW;
-    constexpr int VPL = (R + 511) / 512;
+    using RPn = RowPlan<R>;
+    constexpr int GRP = RPn::GRP, SPW = RPn::SPW, VPL = RPn::VPL, RP = RPn::RP;
     constexpr int PITCH = R + 8;
-    constexpr int RPW = ROWS / WPB;          // rows per wave, taken 4 at a time
+    constexpr int RPW = ROWS / NW;           // rows per wave
+    static_assert(RPW % RPn::PER_PASS == 0, "rows per wave must be whole passes");
     __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
     const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gl = lane % GRP, sub = lane / GRP;
     const RowIdx ixb = row_index(rs, blockIdx.x * (ROWS * TILES));
     h8 fk[NT][P / 16], fq[P / 16];
     load_keys<P, NT>(a, ixb.i1, ixb.i2, wave, lane, fk);
     load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3, lane, fq);
     for (int tile = 0; tile < TILES; ++tile) {
-    const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
-    if (tile) __syncthreads();                 // the previous tile's rows have been read
-    score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
-    if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
-    __syncthreads();
+        const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
+        if (tile) __syncthreads();                 // the previous tile's rows have been read
+        score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
+        if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
+        __syncthreads();
 #pragma unroll
-    for (int half_ = 0; half_ < RPW / 4; ++half_) {
-        float x[4][VPL][8];
-        float m[4], s[4];
-        RowIdx ix[4];
+        for (int pass = 0; pass < RPW / RPn::PER_PASS; ++pass) {
+            float x[RP][VPL][8];
+            float m[RP], s[RP];
+            RowIdx ix[RP];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int rl = wave * RPW + half_ * 4 + r;
-            ix[r] = row_index(rs, row_base + rl);
-            m[r] = -INFINITY;
+            for (int r = 0; r < RP; ++r) {
+                const int rl = wave * RPW + pass * RPn::PER_PASS + r * SPW + sub;
+                ix[r] = row_index(rs, row_base + rl);
+                m[r] = -INFINITY;
 #pragma unroll
-            for (int c = 0; c < VPL; ++c) {
-                const int e0 = (c * WAVE + lane) * 8;
-                if (e0 < R) {
+                for (int c = 0; c < VPL; ++c) {
+                    const int e0 = (c * GRP + gl) * 8;
                     h8 v = *reinterpret_cast<const h8*>(stage + rl * PITCH + e0);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) { x[r][c][i] = (float)v[i]; m[r] = fmaxf(m[r], x[r][c][i]); }
-                } else {
+                }
+            }
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) x[r][c][i] = -INFINITY;
+            for (int r = 0; r < RP; ++r) m[r] = group_max<GRP>(m[r]);
+#pragma unroll
+            for (int r = 0; r < RP; ++r) {
+                s[r] = 0.f;
+#pragma unroll
+                for (int c = 0; c < VPL; ++c)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        x[r][c][i] = __builtin_amdgcn_exp2f((x[r][c][i] - m[r]) * LOG2E);
+                        s[r] += x[r][c][i];
+                    }
+            }
+#pragma unroll
+            for (int r = 0; r < RP; ++r) s[r] = group_sum<GRP>(s[r]);
+#pragma unroll
+            for (int r = 0; r < RP; ++r) {
+                const unsigned row = row_base + wave * RPW + pass * RPn::PER_PASS + r * SPW + sub;
+                const float inv = 1.0f / s[r];
+                const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
+#pragma unroll
+                for (int c = 0; c < VPL; ++c) {
+                    const int e0 = (c * GRP + gl) * 8;
+                    h8 al, d;
+                    const uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)R + (uint64_t)e0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) al[i] = (half_t)(x[r][c][i] * inv);
+                    al = pin(al);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) d[i] = ((bits >> i) & 1u) ? al[i] : (half_t)0.0f;
+                    stg8<true>(alpha.p + oa + e0, al);
+                    stg8<true>(mask.p + om + e0, mask_h8(bits));
+                    stg8<false>(drop.p + od + e0, d);
                 }
             }
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) m[r] = wave_max(m[r]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            s[r] = 0.f;
-#pragma unroll
-            for (int c = 0; c < VPL; ++c)
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    x[r][c][i] = __builtin_amdgcn_exp2f((x[r][c][i] - m[r]) * LOG2E);
-                    s[r] += x[r][c][i];
-                }
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const unsigned row = row_base + wave * RPW + half_ * 4 + r;
-            const float inv = 1.0f / s[r];
-            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
-#pragma unroll
-            for (int c = 0; c < VPL; ++c) {
-                const int e0 = (c * WAVE + lane) * 8;
-                if (e0 >= R) continue;
-                h8 al, d;
-                const uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)R + (uint64_t)e0);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) al[i] = (half_t)(x[r][c][i] * inv);
-                al = pin(al);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) d[i] = ((bits >> i) & 1u) ? al[i] : (half_t)0.0f;
-                stg8<true>(alpha.p + oa + e0, al);
-                stg8<true>(mask.p + om + e0, mask_h8(bits));
-                stg8<false>(drop.p + od + e0, d);
-            }
-        }
-    }
     }
 }
 
 template <int P, int NT, int NW>
 __global__ __launch_bounds__(NW * WAVE) void k_dscores_bs(RowSpace rs, ScoreArgs a, View alpha, View mask, View dbeta) {
     constexpr int R = 32 * NT * NW;
-    constexpr int WPB = NW;
-    constexpr int VPL = (R + 511) / 512;
+    using RPn = RowPlan<R>;
+    constexpr int GRP = RPn::GRP, SPW = RPn::SPW, VPL = RPn::VPL, RP = RPn::RP;
     constexpr int PITCH = R + 8;
-    constexpr int RPW = ROWS / WPB;
+    constexpr int RPW = ROWS / NW;
+    static_assert(RPW % RPn::PER_PASS == 0, "rows per wave must be whole passes");
     __shared__ __attribute__((aligned(16))) half_t stage[ROWS * PITCH];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int gl = lane % GRP, sub = lane / GRP;
     const RowIdx ixb = row_index(rs, blockIdx.x * (ROWS * TILES));
     h8 fk[NT][P / 16], fq[P / 16];
     load_keys<P, NT>(a, ixb.i1, ixb.i2, wave, lane, fk);
     load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3, lane, fq);
     for (int tile = 0; tile < TILES; ++tile) {
-    const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
-    if (tile) __syncthreads();
-    score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
-    if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
-    __syncthreads();
+        const unsigned row_base = (blockIdx.x * TILES + tile) * ROWS;
+        if (tile) __syncthreads();
+        score_tile<P, NT>(fk, fq, a.alpha, wave, lane, stage, PITCH);
+        if (tile + 1 < TILES) load_queries<P>(a, ixb.i1, ixb.i2, ixb.i3 + (tile + 1) * ROWS, lane, fq);
+        __syncthreads();
 #pragma unroll
-    for (int half_ = 0; half_ < RPW / 4; ++half_) {
-        float al[4][VPL][8], g[4][VPL][8];
-        float s[4];
-        RowIdx ix[4];
+        for (int pass = 0; pass < RPW / RPn::PER_PASS; ++pass) {
+            float al[RP][VPL][8], g[RP][VPL][8];
+            float s[RP];
+            RowIdx ix[RP];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int rl = wave * RPW + half_ * 4 + r;
-            ix[r] = row_index(rs, row_base + rl);
-            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]);
-            s[r] = 0.f;
+            for (int r = 0; r < RP; ++r) {
+                const int rl = wave * RPW + pass * RPn::PER_PASS + r * SPW + sub;
+                ix[r] = row_index(rs, row_base + rl);
+                const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]);
+                s[r] = 0.f;
 #pragma unroll
-            for (int c = 0; c < VPL; ++c) {
-                const int e0 = (c * WAVE + lane) * 8;
-                h8 va = (h8)(half_t)0.0f, vm = (h8)(half_t)0.0f, vd = (h8)(half_t)0.0f;
-                if (e0 < R) {
-                    va = ldg8<true>(alpha.p + oa + e0);
-                    vm = ldg8<true>(mask.p + om + e0);
-                    vd = *reinterpret_cast<const h8*>(stage + rl * PITCH + e0);
+                for (int c = 0; c < VPL; ++c) {
+                    const int e0 = (c * GRP + gl) * 8;
+                    const h8 va = ldg8<true>(alpha.p + oa + e0);
+                    const h8 vm = ldg8<true>(mask.p + om + e0);
+                    const h8 vd = *reinterpret_cast<const h8*>(stage + rl * PITCH + e0);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        al[r][c][i] = (float)va[i];
+                        g[r][c][i] = (float)vm[i] * (float)vd[i];
+                        s[r] += al[r][c][i] * g[r][c][i];
+                    }
                 }
+            }
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    al[r][c][i] = (float)va[i];
-                    g[r][c][i] = (float)vm[i] * (float)vd[i];
-                    s[r] += al[r][c][i] * g[r][c][i];
+            for (int r = 0; r < RP; ++r) s[r] = group_sum<GRP>(s[r]);
+#pragma unroll
+            for (int r = 0; r < RP; ++r) {
+                const long oo = view_offset(dbeta, ix[r]);
+#pragma unroll
+                for (int c = 0; c < VPL; ++c) {
+                    const int e0 = (c * GRP + gl) * 8;
+                    h8 o;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) o[i] = (half_t)(1.0f * al[r][c][i] * (g[r][c][i] - s[r]));
+                    stg8<false>(dbeta.p + oo + e0, o);
                 }
             }
         }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) s[r] = wave_sum(s[r]);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const long oo = view_offset(dbeta, ix[r]);
-#pragma unroll
-            for (int c = 0; c < VPL; ++c) {
-                const int e0 = (c * WAVE + lane) * 8;
-                if (e0 >= R) continue;
-                h8 o;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) o[i] = (half_t)(1.0f * al[r][c][i] * (g[r][c][i] - s[r]));
-                stg8<false>(dbeta.p + oo + e0, o);
-            }
-        }
-    }
     }
 }
 
@@ -234,6 +239,8 @@ template <int P>
 bool dispatch_fwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
                   View drop, PhiloxKey key) {
     switch (R) {
+        case 128: hipLaunchKernelGGL((k_scores_softmax<P, 1, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
+        case 256: hipLaunchKernelGGL((k_scores_softmax<P, 2, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
         case 512: hipLaunchKernelGGL((k_scores_softmax<P, 4, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
         case 1024: hipLaunchKernelGGL((k_scores_softmax<P, 8, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, drop, key); return true;
         default: return false;
@@ -243,6 +250,8 @@ template <int P>
 bool dispatch_bwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const ScoreArgs& a, View alpha, View mask,
                   View dbeta) {
     switch (R) {
+        case 128: hipLaunchKernelGGL((k_dscores_bs<P, 1, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
+        case 256: hipLaunchKernelGGL((k_dscores_bs<P, 2, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
         case 512: hipLaunchKernelGGL((k_dscores_bs<P, 4, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
         case 1024: hipLaunchKernelGGL((k_dscores_bs<P, 8, 4>), grid, dim3(256), 0, st, rs, a, alpha, mask, dbeta); return true;
         default: return false;
@@ -253,7 +262,7 @@ bool dispatch_bwd(int R, dim3 grid, hipStream_t st, const RowSpace& rs, const Sc
 
 bool scores_fusable(const RowSpace& rs, const ScoreArgs& a, int P, std::initializer_list<const View*> views) {
     if (rs.n0 != 1 || rs.flat) return false;                       // rows numbered over (H, B, J)
-    if (rs.R != 512 && rs.R != 1024) return false;
+    if (rs.R != 128 && rs.R != 256 && rs.R != 512 && rs.R != 1024) return false;
     if (P != 64 && P != 128) return false;
     if (rs.n3 % (ROWS * TILES) != 0) return false;                 // a workgroup's rows share head and sample
     if (rs.rows() <= 0 || rs.rows() / (ROWS * TILES) > 0x7fffffffL) return false;

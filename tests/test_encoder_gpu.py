@@ -19,7 +19,9 @@ def _layouts(which):
     from substation_amd import layouts as L
     if isinstance(which, dict):
         return which
-    return L.mi355x_layouts() if which == 'mi355x' else L.reference_layouts(which)
+    if which.startswith('mi355x'):
+        return L.mi355x_layouts(which[7:] or None)
+    return L.reference_layouts(which)
 
 
 def _all_layouts(lay):
@@ -243,6 +245,9 @@ def test_fused_ln_backward_matches_separate(dims, act):
     ('bert-b8-l512-h16-e1024', (2, 64, 2, 128), 'relu'),
     ('mi355x', (3, 40, 3, 120), 'relu'),             # edge tiles
     ('mi355x', (8, 512, 16, 1024), 'relu'),          # the bench size: 256x256 asynchronous tiles
+    ('mi355x', (2, 128, 2, 128), 'relu'),            # fused score kernels, four rows per wave
+    ('mi355x', (2, 256, 2, 256), 'gelu'),            # two rows per wave, head size 128
+    ('mi355x:bert-b96-l128-h16-e1024', (16, 128, 16, 1024), 'relu'),# short rows at a size where they run side by side
 ])
 def test_fused_epilogues_match_unfused(which, dims, act):
     """Without debug capture the QKV bias add and the DX residual add run inside
