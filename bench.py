@@ -82,6 +82,12 @@ def algorithmic_work(B, L, H, E):
         w[n] = ('mfma',) + proj
     for n in ('QKT', 'gamma', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT'):
         w[n] = ('mfma',) + attn
+    # attention with the scores in registers: 2 / 3 / 4 products of the size of QKT
+    # (the backward launches form the scores again); bytes: the projections, the
+    # output or gradients, one keep bit per score
+    w['attention'] = ('mfma', 2 * attn[0], 2 * 4 * bji + hbjk // 8)
+    w['attention-bwd-dQ'] = ('mfma', 3 * attn[0], 2 * 6 * bji + hbjk // 8)
+    w['attention-bwd-dKdV'] = ('mfma', 4 * attn[0], 2 * 6 * bji + hbjk // 8)
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

@@ -150,6 +150,22 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * left unwritten; every other tensor is unchanged.  Set to 0 to materialise
  * them (the Python module does so for debug capture). */
 #define SUB_OPT_FUSE_SCORES 3
+/* SUB_OPT_FUSE_ATTENTION (default 1): run the whole self-attention -- scores,
+ * softmax, dropout and the weighted sum of the values (encoder.cu:104-131), and
+ * in the backward pass everything between DGAMMA and the gradients of the
+ * projections (encoder.cu:222-262) -- with the scores kept in registers.  None
+ * of BETA, ALPHA, ATTN_DROP_MASK, ATTN_DROP, DATTN_DROP and DBETA is then
+ * produced; the ALPHA buffer holds two fp32 statistics per score row and the
+ * ATTN_DROP_MASK buffer one keep bit per score instead (both buffers must be
+ * the ones handed to the matching backward call, as in the reference).  The
+ * dropout mask is the same counter-based one as in the separate operators.
+ * Needs head size 64 or 128, sequence lengths that are multiples of 128,
+ * feature-contiguous projections and no attention mask; otherwise, or with 0,
+ * the operators run separately (results then agree to fp16 rounding, not bit
+ * for bit, because probabilities are no longer rounded before the weighted sum).
+ * Set the option before the forward call and leave it until after the matching
+ * backward call. */
+#define SUB_OPT_FUSE_ATTENTION 4
 int sub_set_option(void* handle, int option, int value);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same

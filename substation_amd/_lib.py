@@ -17,6 +17,7 @@ ACTIVATIONS = {'relu': 0, 'gelu': 1}
 OPT_FUSE_EPILOGUES = 1
 OPT_FUSE_LN_BACKWARD = 2
 OPT_FUSE_SCORES = 3
+OPT_FUSE_ATTENTION = 4
 
 
 class SubConfig(ctypes.Structure):

@@ -183,6 +183,7 @@ struct Handle {
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
     bool fuse_scores = true;
+    bool fuse_attention = true;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -553,6 +554,44 @@ bool op_dscores_bs(Handle& h, const void* dgamma, const void* vv, const void* al
     return launch_dscores_bs(sp.rs, a, (int)h.sz.n[dP], va, vm, vo, h.stream);
 }
 
+half_t* sub_q(void* base, const Handle& h, int q) {
+    int64_t n = h.sz.n[dP] * h.sz.n[dH] * h.sz.n[dB] * h.sz.n[dJ];
+    return (half_t*)base + (int64_t)q * n;
+}
+
+// Whole self-attention (scores, softmax, dropout, weighted sum) with the scores
+// kept in registers.  The ALPHA buffer then holds, instead of probabilities, two
+// fp32 values per score row (log-sum-exp, and in the backward pass the row sum of
+// dO o O), and the ATTN_DROP_MASK buffer one keep bit per score.
+bool attn_side(const void* p, const Layout& l, int pos_dim, AttnSide& s) {
+    if (l.rank != 4 || !l.has[dP] || l.stride[dP] != 1 || !l.has[dH] || !l.has[dB] || !l.has[pos_dim]) return false;
+    s.p = (const half_t*)p; s.sh = l.stride[dH]; s.sb = l.stride[dB]; s.sr = l.stride[pos_dim];
+    return true;
+}
+
+// Decided from what the forward pass sees, so that both passes take the same path.
+bool attention_fused(const Handle& h, void* const* F, AttnArgs& a) {
+    if (!h.fuse_attention || h.attn_mask) return false;
+    const Sizes& z = h.sz;
+    if (!mha_shape_ok(z.n[dH], z.n[dB], z.n[dJ], z.n[dK], z.n[dP])) return false;
+    a.H = (int)z.n[dH]; a.B = (int)z.n[dB]; a.J = (int)z.n[dJ]; a.K = (int)z.n[dK];
+    a.alpha = h.gemm[G_QKT].alpha;
+    half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
+    if (!attn_side(QQ, h.lQQ, dJ, a.q) || !attn_side(KK, h.lKK, dK, a.k) || !attn_side(VV, h.lKK, dK, a.v) ||
+        !attn_side(F[GAMMA], h.lf[GAMMA], dJ, a.o))
+        return false;
+    // the backward pass's tensors must qualify too (layouts only; pointers are checked there)
+    AttnSide t;
+    if (!attn_side(nullptr, h.lb[DGAMMA], dJ, t) || !attn_side(nullptr, h.lDQQ, dJ, t) ||
+        !attn_side(nullptr, h.lDKK, dK, t))
+        return false;
+    const size_t rows = (size_t)a.H * a.B * a.J;
+    if (mha_stat_bytes(a.H, a.B, a.J) > rows * a.K * sizeof(half_t)) return false;
+    a.lse = (float*)F[ALPHA]; a.dsum = a.lse + rows;
+    a.keep = (uint32_t*)F[ATTN_DROP_MASK];
+    return mha_forward_ok(a, (int)z.n[dP]);
+}
+
 // bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
 // false, having done nothing, when the shape or the layouts rule the fused
 // kernel out; the caller then runs the separate operators.
@@ -645,11 +684,6 @@ struct BwdPtrs {
     void* X; void* DX;
 };
 
-half_t* sub_q(void* base, const Handle& h, int q) {
-    int64_t n = h.sz.n[dP] * h.sz.n[dH] * h.sz.n[dB] * h.sz.n[dJ];
-    return (half_t*)base + (int64_t)q * n;
-}
-
 // Advances the device-side dropout step (a vector store by one lane).
 __global__ void k_step_increment(uint32_t* step) {
     if (threadIdx.x == 0) step[0] = step[0] + 1u;
@@ -668,8 +702,14 @@ void forward(Handle& h, const FwdPtrs& t) {
         op_aib(h, F[WKKWQQWVV], h.lf[WKKWQQWVV], W[BKQV], h.lp[BKQV], F[KKQQVV], h.lf[KKQQVV]);
     }
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
-    bool fused_scores = false;
-    if (h.fuse_scores) {
+    AttnArgs at;
+    const bool fused_attention = attention_fused(h, F, at);
+    if (fused_attention) {
+        ProfScope ps(h, "attention");
+        launch_mha_forward(at, (int)h.sz.n[dP], make_key(h, SUB_SITE_SOFTMAX, h.p_softmax), h.stream);
+    }
+    bool fused_scores = fused_attention;
+    if (!fused_attention && h.fuse_scores) {
         ProfScope ps(h, "QKT+softmax");
         fused_scores = op_scores_softmax(h, QQ, KK, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK],
                                          h.lf[ATTN_DROP_MASK], F[ATTN_DROP], h.lf[ATTN_DROP]);
@@ -682,7 +722,7 @@ void forward(Handle& h, const FwdPtrs& t) {
                    F[ATTN_DROP], h.lf[ATTN_DROP], 1.0f, h.p_softmax, SUB_SITE_SOFTMAX, h.attn_mask,
                    &h.l_attn_mask, h.gemm[G_QKT].alpha);
     }
-    run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
+    if (!fused_attention) run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
     run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
     {
         ProfScope ps(h, "bdrln1");   // adds BO to ATT in place (encoder.cu:134-135)
@@ -782,22 +822,35 @@ void backward(Handle& h, const BwdPtrs& t) {
     run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
-    run_gemm(h, G_DX2GAMMA, D[DGAMMA], F[ATTN_DROP], DVV, "dX2gamma");
-    bool fused_scores = false;
-    if (h.fuse_scores) {
-        ProfScope ps(h, "dX1gamma+bs");
-        fused_scores = op_dscores_bs(h, D[DGAMMA], VV, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK],
-                                     h.lf[ATTN_DROP_MASK], D[DBETA], h.lb[DBETA]);
-        if (!fused_scores) ps.cancel();
+    AttnArgs at;
+    if (attention_fused(h, F, at)) {
+        if (!attn_side(D[DGAMMA], h.lb[DGAMMA], dJ, at.d_o) || !attn_side(DQQ, h.lDQQ, dJ, at.dq) ||
+            !attn_side(DKK, h.lDKK, dK, at.dk) || !attn_side(DVV, h.lDKK, dK, at.dv))
+            fail("encoder_backward: attention layouts changed since the forward pass");
+        {
+            ProfScope ps(h, "attention-bwd-dQ");
+            launch_mha_backward_dq(at, (int)h.sz.n[dP], h.stream);
+        }
+        ProfScope ps(h, "attention-bwd-dKdV");
+        launch_mha_backward_dkv(at, (int)h.sz.n[dP], h.stream);
+    } else {
+        run_gemm(h, G_DX2GAMMA, D[DGAMMA], F[ATTN_DROP], DVV, "dX2gamma");
+        bool fused_scores = false;
+        if (h.fuse_scores) {
+            ProfScope ps(h, "dX1gamma+bs");
+            fused_scores = op_dscores_bs(h, D[DGAMMA], VV, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK],
+                                         h.lf[ATTN_DROP_MASK], D[DBETA], h.lb[DBETA]);
+            if (!fused_scores) ps.cancel();
+        }
+        if (!fused_scores) {
+            run_gemm(h, G_DX1GAMMA, VV, D[DGAMMA], D[DATTN_DROP], "dX1gamma");
+            ProfScope ps(h, "bs");
+            op_bs(h, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK], D[DATTN_DROP],
+                  h.lb[DATTN_DROP], D[DBETA], h.lb[DBETA], 1.0f);
+        }
+        run_gemm(h, G_DX1QKT, KK, D[DBETA], DQQ, "dX1QKT");
+        run_gemm(h, G_DX2QKT, QQ, D[DBETA], DKK, "dX2QKT");
     }
-    if (!fused_scores) {
-        run_gemm(h, G_DX1GAMMA, VV, D[DGAMMA], D[DATTN_DROP], "dX1gamma");
-        ProfScope ps(h, "bs");
-        op_bs(h, F[ALPHA], h.lf[ALPHA], F[ATTN_DROP_MASK], h.lf[ATTN_DROP_MASK], D[DATTN_DROP],
-              h.lb[DATTN_DROP], D[DBETA], h.lb[DBETA], 1.0f);
-    }
-    run_gemm(h, G_DX1QKT, KK, D[DBETA], DQQ, "dX1QKT");
-    run_gemm(h, G_DX2QKT, QQ, D[DBETA], DKK, "dX2QKT");
     const bool fuse_dx = h.fuse_epilogues && h.gemm[G_DXQKV_RESID].ok && aligned16(D[DRESID1]) &&
                          aligned16(t.DX);
     if (fuse_dx) {
@@ -972,6 +1025,7 @@ int sub_set_option(void* handle, int option, int value) {
         if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
         else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
         else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
+        else if (option == SUB_OPT_FUSE_ATTENTION) h.fuse_attention = value != 0;
         else fail("sub_set_option: unknown option");
     });
 }

@@ -105,6 +105,34 @@ bool launch_scores_softmax(const RowSpace& rs, const ScoreArgs& a, int head_size
 bool launch_dscores_bs(const RowSpace& rs, const ScoreArgs& a, int head_size, View alpha, View mask,
                        View dbeta, hipStream_t st);
 
+// --- self-attention with the scores kept in registers -------------------------
+// One of Q, K, V, the output or a gradient of these: rows of head_size contiguous
+// features, strided over (head, sample, position).
+struct AttnSide {
+    const half_t* p = nullptr;
+    long sh = 0, sb = 0, sr = 0;
+};
+struct AttnArgs {
+    AttnSide q, k, v;          // projections (read)
+    AttnSide o;                // forward: the output (written); backward: read
+    AttnSide d_o;              // backward: gradient of the output (read)
+    AttnSide dq, dk, dv;       // backward: gradients of the projections (written)
+    float* lse = nullptr;      // [H*B*J]  log2-domain log-sum-exp of each score row
+    float* dsum = nullptr;     // [H*B*J]  row sums of dO o O (written by the dQ launch, read by the dK/dV one)
+    uint32_t* keep = nullptr;  // [H*B*J][K/32]  keep bits of the softmax dropout, bit k%32 of word k/32
+    int H = 0, B = 0, J = 0, K = 0;
+    float alpha = 1.f;         // score scale
+};
+// head_size 64 or 128, J and K multiples of 128
+bool mha_shape_ok(long H, long B, long J, long K, long head_size);
+size_t mha_stat_bytes(long H, long B, long J);          // lse followed by dsum
+size_t mha_keep_bytes(long H, long B, long J, long K);
+bool mha_forward_ok(const AttnArgs& a, int head_size);
+bool mha_backward_ok(const AttnArgs& a, int head_size);
+void launch_mha_forward(const AttnArgs& a, int head_size, PhiloxKey key, hipStream_t st);
+void launch_mha_backward_dq(const AttnArgs& a, int head_size, hipStream_t st);
+void launch_mha_backward_dkv(const AttnArgs& a, int head_size, hipStream_t st);
+
 // --- tensor contraction ------------------------------------------------------
 // Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
 // that broadcasts along M or N, or a whole tensor (a residual).

@@ -80,6 +80,7 @@ class Encoder(torch.nn.Module):
             # aib / bei operators instead of fusing them into GEMM epilogues
             self._handle.set_option(_lib.OPT_FUSE_EPILOGUES, 0)
             self._handle.set_option(_lib.OPT_FUSE_SCORES, 0)
+            self._handle.set_option(_lib.OPT_FUSE_ATTENTION, 0)
         handle = self._handle
         lib = handle.lib
         module = self

@@ -261,6 +261,7 @@ def test_fused_epilogues_match_unfused(which, dims, act):
         torch.manual_seed(0)
         enc = Encoder('unused', B, L, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, enable_debug=debug,
                       seed=SEED, activation=act).cuda()
+        enc._handle.set_option(4, 0)      # the attention kernels are compared separately (rounding differs)
         enc.set_rng(SEED, 0)
         with torch.no_grad():
             for p in enc.parameters():
@@ -276,6 +277,48 @@ def test_fused_epilogues_match_unfused(which, dims, act):
     for a, b in zip(*outs):
         assert torch.isfinite(a.float()).all()
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize('which,dims,act,p', [
+    ('mi355x', (2, 128, 2, 128), 'gelu', 0.1),
+    ('mi355x', (2, 128, 2, 128), 'gelu', 0.0),
+    ('mi355x', (3, 384, 2, 128), 'gelu', 0.5),           # three blocks of 128 positions
+    ('mi355x', (2, 256, 2, 256), 'gelu', 0.1),           # head size 128
+    ('bert-b8-l512-h16-e1024', (2, 128, 2, 128), 'gelu', 0.1),   # the reference's layouts: falls back, still equal
+    ('mi355x:bert-b96-l128-h16-e1024', (16, 128, 16, 1024), 'gelu', 0.1),
+    ('mi355x', (8, 512, 16, 1024), 'gelu', 0.1),
+])
+def test_attention_in_registers_matches_separate_operators(which, dims, act, p):
+    """The attention kernels that keep the scores in registers (default) against
+    the separate operators (QKT, softmax, gamma and their backward counterparts):
+    same inputs, same dropout masks, outputs and all gradients within the parity
+    bound of each other (observed: 4e-3 at the bench size, where weight gradients
+    sum 4096 fp16-rounded terms).  A wrong mask bit, a transposed tile or a wrong
+    log-sum-exp would be an error of order one.  GELU throughout: with ReLU, a
+    pre-activation that rounds to the other side of zero flips whole gradient
+    elements, which says nothing about the attention kernels."""
+    from substation_amd import Encoder
+    lay = _layouts(which)
+    B, L, H, E = dims
+    outs = []
+    for fused in (0, 1):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, L, H, E, lay, torch.float16, p, 0.1, 0.1, 0.1, seed=SEED, activation=act).cuda()
+        enc._handle.set_option(4, fused)
+        enc.set_rng(SEED, 0)
+        with torch.no_grad():
+            for q in enc.parameters():
+                q.mul_(0.1)
+        g = torch.Generator().manual_seed(5)
+        shape = tuple(enc.sizes[d] for d in lay['input'][1])
+        X = torch.randn(shape, generator=g).half().cuda().requires_grad_(True)
+        DY = torch.randn(shape, generator=g).half().cuda()
+        Y = enc(X)
+        Y.backward(DY)
+        torch.cuda.synchronize()
+        outs.append([('Y', Y.detach()), ('DX', X.grad)] + [(n, q.grad) for n, q in enc.named_parameters()])
+    for (name, a), (_, b) in zip(*outs):
+        assert_close(b.float().cpu().numpy(), a.float().cpu().numpy(), tol=1e-2, name=name)
 
 
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
