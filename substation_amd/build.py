@@ -20,6 +20,10 @@ SOURCES = ['encoder.hip', 'k_rows.hip', 'k_elem.hip', 'k_cols.hip', 'k_lnbwd.hip
 FLAGS = ['--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-Wall', '-Wno-unused-function',
          # packed-fp32 VALU forms are switched off for every kernel of this library
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']
+# The attention kernels work on the MFMA results with vector instructions right
+# away: keep those results in ordinary vector registers (the default puts them
+# in accumulator registers and copies every value out and back in).
+EXTRA_FLAGS = {'k_mha.hip': ['-mllvm', '-amdgpu-mfma-vgpr-form=1']}
 
 
 def _hipcc():
@@ -45,7 +49,7 @@ def build(verbose=False, jobs=8):
 
     def compile_one(src):
         obj = os.path.join(OBJ, src.replace('.hip', '.o'))
-        out = _run([hipcc, *FLAGS, '-c', os.path.join(CSRC, src), '-o', obj])
+        out = _run([hipcc, *FLAGS, *EXTRA_FLAGS.get(src, []), '-c', os.path.join(CSRC, src), '-o', obj])
         if verbose and out.strip():
             print(out)
         return obj

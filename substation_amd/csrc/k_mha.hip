@@ -33,14 +33,25 @@ typedef short s4v __attribute__((ext_vector_type(4)));
 typedef short s8v __attribute__((ext_vector_type(8)));
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int QB = 128;           // positions per workgroup: 4 waves x 32
+constexpr float RESCALE_SLACK = 8.f;   // unnormalised probabilities stay below 2^8
 
 template <int P>
 struct Geo {
     static constexpr int NKS = P / 16;             // k-steps of a contraction over the features
     static constexpr int NPT = P / 32;             // 32-wide tiles of the feature dim
-    static constexpr int PITCH = P + 8;            // halves per row of an LDS tile
-    static constexpr int TILE = 32 * PITCH;        // 32 positions
+    static constexpr int TILE = 32 * P;            // halves of an LDS tile of 32 positions
     static constexpr int VL = (32 * (P / 8)) / 256; // 16-byte words per thread and tile
+
+    // LDS tiles are [position][feature] without padding; the index of a 16-byte
+    // chunk within its row is xor-ed with a function of the row chosen so that both
+    // ways of reading a tile are free of bank conflicts: 16 consecutive rows at one
+    // chunk (the features as contraction index, ds_read_b128) and 4 consecutive
+    // rows x 4 adjacent chunks (the positions as contraction index, transposing read).
+    static __device__ __forceinline__ int swz(int row) {
+        return P == 64 ? ((((row >> 1) & 1) << 2) | ((row >> 2) & 3)) : (((row & 3) << 2) | ((row >> 2) & 3));
+    }
+    // offset in halves of chunk c of a row
+    static __device__ __forceinline__ int at(int row, int c) { return row * P + ((c ^ swz(row)) << 3); }
 };
 
 // Fragment of 32 rows (one per lane%32) with the features as contraction index:
@@ -53,12 +64,12 @@ __device__ __forceinline__ void row_frags(const AttnSide& t, unsigned h, unsigne
     for (int ks = 0; ks < P / 16; ++ks) f[ks] = *reinterpret_cast<const h8*>(p + ks * 16);
 }
 
-// The same fragment from an LDS tile [32 positions][P].
+// The same fragment from an LDS tile.
 template <int P>
 __device__ __forceinline__ void row_frags_lds(const half_t* tile, int l32, int hi, h8 (&f)[P / 16]) {
 #pragma unroll
     for (int ks = 0; ks < P / 16; ++ks)
-        f[ks] = *reinterpret_cast<const h8*>(tile + l32 * Geo<P>::PITCH + hi * 8 + ks * 16);
+        f[ks] = *reinterpret_cast<const h8*>(tile + Geo<P>::at(l32, 2 * ks + hi));
 }
 
 // A tile of 32 positions x P features: global -> registers -> LDS, all threads.
@@ -77,7 +88,7 @@ __device__ __forceinline__ void tile_put(half_t* tile, int tid, const h8 (&r)[Ge
 #pragma unroll
     for (int i = 0; i < Geo<P>::VL; ++i) {
         const int id = tid + i * 256, row = id / (P / 8), c = id % (P / 8);
-        *reinterpret_cast<h8*>(tile + row * Geo<P>::PITCH + c * 8) = r[i];
+        *reinterpret_cast<h8*>(tile + Geo<P>::at(row, c)) = r[i];
     }
 }
 
@@ -85,16 +96,24 @@ __device__ __forceinline__ void tile_put(half_t* tile, int tid, const h8 (&r)[Ge
 // m0 + lane%32, elements = positions in the register order of a score tile.
 // ds_read_b64_tr_b16: within 16 lanes, lane i receives T[k0 + 0..3][m0 + i] when
 // lane l addresses T[k0 + l/4][m0 + 4*(l%4)].
-__device__ __forceinline__ h8 tr_frag(const half_t* tile, int pitch, int m0, int s, int lane) {
+template <int P>
+__device__ __forceinline__ h8 tr_frag(const half_t* tile, int m0, int s, int lane) {
     const int g = lane >> 4, l = lane & 15;
     const int k = 16 * s + 4 * (g >> 1) + (l >> 2);
     const int m = m0 + 16 * (g & 1) + 4 * (l & 3);
-    const half_t* p = tile + k * pitch + m;
     typedef s4v __attribute__((address_space(3))) * lds_s4;
-    s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p));
-    s4v up = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(p + 8 * pitch));
+    s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(tile + Geo<P>::at(k, m >> 3) + (m & 7)));
+    s4v up = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4)(tile + Geo<P>::at(k + 8, m >> 3) + (m & 7)));
     s8v r = __builtin_shufflevector(lo, up, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(h8, r);
+}
+
+// Workgroups are dealt to the 8 XCDs (each with its own L2) in turn.  Renumbered
+// so that consecutive logical blocks -- the blocks of one head and sample, which
+// read the same K, V (or Q, dO) -- run on one XCD and share its L2.
+__device__ __forceinline__ unsigned logical_block() {
+    const unsigned n = gridDim.x, bid = blockIdx.x;
+    return (n % 8u) ? bid : (bid % 8u) * (n / 8u) + bid / 8u;
 }
 
 // Position (within a tile of 32) that accumulator register v of a lane holds.
@@ -116,6 +135,41 @@ __device__ __forceinline__ void store_rows(const AttnSide& t, unsigned h, unsign
         }
 }
 
+// x ^ y ^ k in one instruction (k uniform).
+__device__ __forceinline__ uint32_t xor3(uint32_t x, uint32_t y, uint32_t k) {
+    uint32_t r;
+    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0x96" : "=v"(r) : "v"(x), "v"(y), "s"(k));
+    return r;
+}
+
+// philox_group() of sub_philox.hpp, bit for bit, with the two xors of each
+// half-round folded into one instruction.
+__device__ __forceinline__ U4 philox_group_dev(const PhiloxKey& k, uint64_t g) {
+    U4 c;
+    c.x = (uint32_t)g; c.y = (uint32_t)(g >> 32); c.z = k.site; c.w = k.step;
+    uint32_t k0 = k.k0, k1 = k.k1;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        uint32_t hi0, lo0, hi1, lo1;
+        mulhilo(0xD2511F53u, c.x, hi0, lo0);
+        mulhilo(0xCD9E8D57u, c.z, hi1, lo1);
+        U4 n;
+        n.x = xor3(hi1, c.y, k0);
+        n.y = lo1;
+        n.z = xor3(hi0, c.w, k1);
+        n.w = lo0;
+        c = n;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return c;
+}
+
+// x where bit `pos` of `bits` is set, else +0.0
+__device__ __forceinline__ float keep_if(float x, uint32_t bits, int pos) {
+    return __int_as_float(__float_as_int(x) & __builtin_amdgcn_sbfe((int)bits, pos, 1));
+}
+
 __device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
     uint32_t b = 0;
 #pragma unroll
@@ -124,98 +178,144 @@ __device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
 }
 
 // ---------------------------------------------------------------------------
+// All three kernels stream tiles of 32 positions through a ring of three LDS
+// buffers: while tile t is worked on, tile t+1 already lies in LDS (its row
+// fragments are read ahead, during the vector work on tile t) and tile t+2 is on
+// its way from memory in registers.  One barrier per tile.
+// ---------------------------------------------------------------------------
+constexpr int RING = 3;
+
+// Every load issued so far has arrived.  Placed before a main loop: a load of the
+// prologue whose first use is inside the loop would otherwise put its wait there,
+// where on every later pass it waits for the loads that pass has just issued.
+__device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
+
+// ---------------------------------------------------------------------------
 // forward.  grid = H * B * (J / 128); wave = 32 queries.
 // ---------------------------------------------------------------------------
 template <int P>
 __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
     using G = Geo<P>;
-    __shared__ __attribute__((aligned(16))) half_t vt[2][G::TILE];
+    __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
+    __shared__ __attribute__((aligned(16))) half_t vt[RING][G::TILE];
     const PhiloxKey key = resolved(key_);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned qblocks = a.J / QB;
-    const unsigned qb = blockIdx.x % qblocks, hb = blockIdx.x / qblocks;
+    const unsigned lb = logical_block();
+    const unsigned qb = lb % qblocks, hb = lb / qblocks;
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned j = qb * QB + wave * 32 + l32;                    // this lane's query
     const unsigned row = (h * a.B + b) * a.J + j;                    // its score row
     const unsigned nt = a.K / 32;
     const float c = a.alpha * LOG2E;
 
-    h8 fq[G::NKS], fk[G::NKS], vr[G::VL];
-    row_frags<P>(a.q, h, b, j, hi, fq);
-    row_frags<P>(a.k, h, b, l32, hi, fk);
-    tile_fetch<P>(a.v, h, b, 0, tid, vr);
-    tile_put<P>(vt[0], tid, vr);
+    h8 fq[G::NKS], fk[G::NKS], kr[G::VL], vr[G::VL];
+    {   // the first two tiles and the query rows: all loads in flight together
+        h8 kr1[G::VL], vr1[G::VL];
+        tile_fetch<P>(a.k, h, b, 0, tid, kr);
+        tile_fetch<P>(a.v, h, b, 0, tid, vr);
+        tile_fetch<P>(a.k, h, b, 32, tid, kr1);
+        tile_fetch<P>(a.v, h, b, 32, tid, vr1);
+        row_frags<P>(a.q, h, b, j, hi, fq);
+        tile_put<P>(kt[0], tid, kr);
+        tile_put<P>(vt[0], tid, vr);
+        tile_put<P>(kt[1], tid, kr1);
+        tile_put<P>(vt[1], tid, vr1);
+    }
     __syncthreads();
+    row_frags_lds<P>(kt[0], l32, hi, fk);
 
     f16v o[G::NPT];
 #pragma unroll
     for (int pt = 0; pt < G::NPT; ++pt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[pt][v] = 0.f;
-    float m_run = -INFINITY, l_run = 0.f;                            // l_run: this lane's keys only
+    float m_ref = -INFINITY, l_run = 0.f;                            // l_run: this lane's keys only
+    const float slack = RESCALE_SLACK / c;
+    int cur = 0, nxt = 1, nn = 2;
+    wait_loads();
 
     for (unsigned t = 0; t < nt; ++t) {
-        h8 fkn[G::NKS];
-        const bool more = t + 1 < nt;
-        if (more) {
-            row_frags<P>(a.k, h, b, (t + 1) * 32 + l32, hi, fkn);
-            tile_fetch<P>(a.v, h, b, (t + 1) * 32, tid, vr);
+        const bool fetch = t + 2 < nt;
+        if (fetch) {
+            tile_fetch<P>(a.k, h, b, (t + 2) * 32, tid, kr);
+            tile_fetch<P>(a.v, h, b, (t + 2) * 32, tid, vr);
         }
         f16v s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
+        // fragments for the second product of this tile and the first of the next
+        h8 va[2][G::NPT];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int pt = 0; pt < G::NPT; ++pt) va[st][pt] = tr_frag<P>(vt[cur], pt * 32, st, lane);
+        row_frags_lds<P>(kt[nxt], l32, hi, fk);
 
         // keep bits of the 32 scores (this query, keys of tile t): each half of the
         // wave draws two of the four groups of 8 and the halves trade them
         uint32_t word = 0xffffffffu;
         if (key.thr) {
             const uint64_t g0 = (uint64_t)row * (a.K / 8) + 4 * t + 2 * hi;
-            const uint32_t mine = keep8(philox_group(key, g0), key.thr) |
-                                  (keep8(philox_group(key, g0 + 1), key.thr) << 8);
+            const uint32_t mine = keep8(philox_group_dev(key, g0), key.thr) |
+                                  (keep8(philox_group_dev(key, g0 + 1), key.thr) << 8);
             const uint32_t other = (uint32_t)__shfl_xor((int)mine, 32);
             word = hi ? (other | (mine << 16)) : (mine | (other << 16));
         }
         if (hi == 0) a.keep[(size_t)row * nt + t] = word;
         const uint32_t nib = word >> (hi * 4);                       // bit reg_pos(v, 0) of nib = keep of register v
 
-        float mt = -INFINITY;
+        // Running softmax with a reference value per query that trails the running
+        // maximum by up to RESCALE_SLACK (in log2 units): the accumulators are only
+        // rescaled when some query of the wave outgrows its reference by more, which
+        // after the first tiles is rare.  Scores and reference are in raw units.
+        float mt = s[0];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { s[v] *= c; mt = fmaxf(mt, s[v]); }
+        for (int v = 1; v < 16; ++v) mt = fmaxf(mt, s[v]);
         mt = fmaxf(mt, __shfl_xor(mt, 32));
-        const float m_new = fmaxf(m_run, mt);
-        const float corr = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        l_run *= corr;
+        if (__builtin_amdgcn_ballot_w64(mt > m_ref + slack) != 0) {
+            const float m_new = fmaxf(m_ref, mt);
+            const float corr = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+            m_ref = m_new;
+            l_run *= corr;
 #pragma unroll
-        for (int pt = 0; pt < G::NPT; ++pt)
+            for (int pt = 0; pt < G::NPT; ++pt)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) o[pt][v] *= corr;
+                for (int v = 0; v < 16; ++v) o[pt][v] *= corr;
+        }
+        const float mc = -m_ref * c;
         h8 pb[2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const float p = __builtin_amdgcn_exp2f(s[v] - m_new);
-            l_run += p;
-            pb[v >> 3][v & 7] = ((nib >> reg_pos(v, 0)) & 1u) ? (half_t)p : (half_t)0.0f;
+        for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], c, mc);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v]);
+        {   // four partial sums: a single one would be a chain of 16 dependent additions
+            float l4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int v = 0; v < 16; ++v) l4[v & 3] += s[v];
+            l_run += (l4[0] + l4[1]) + (l4[2] + l4[3]);
         }
-        const half_t* vtile = vt[t & 1];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = keep_if(s[v], nib, reg_pos(v, 0));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) pb[v >> 3][v & 7] = (half_t)s[v];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int pt = 0; pt < G::NPT; ++pt)
-                o[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(tr_frag(vtile, G::PITCH, pt * 32, st, lane), pb[st],
-                                                               o[pt], 0, 0, 0);
-        if (more) {
-            tile_put<P>(vt[(t + 1) & 1], tid, vr);
-#pragma unroll
-            for (int ks = 0; ks < G::NKS; ++ks) fk[ks] = fkn[ks];
+                o[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[st][pt], pb[st], o[pt], 0, 0, 0);
+        if (fetch) {
+            tile_put<P>(kt[nn], tid, kr);
+            tile_put<P>(vt[nn], tid, vr);
         }
         __syncthreads();
+        const int x = cur; cur = nxt; nxt = nn; nn = x;
     }
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     store_rows<P>(a.o, h, b, j, hi, o, 1.0f / l_tot);
-    if (hi == 0) a.lse[row] = m_run + __builtin_amdgcn_logf(l_tot);
+    if (hi == 0) a.lse[row] = m_ref * c + __builtin_amdgcn_logf(l_tot);
 }
 
 // ---------------------------------------------------------------------------
@@ -224,23 +324,37 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
 template <int P>
 __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
     using G = Geo<P>;
-    __shared__ __attribute__((aligned(16))) half_t kt[2][G::TILE];
+    __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
+    __shared__ __attribute__((aligned(16))) half_t vt[RING][G::TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned qblocks = a.J / QB;
-    const unsigned qb = blockIdx.x % qblocks, hb = blockIdx.x / qblocks;
+    const unsigned lb = logical_block();
+    const unsigned qb = lb % qblocks, hb = lb / qblocks;
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned j = qb * QB + wave * 32 + l32;
     const unsigned row = (h * a.B + b) * a.J + j;
     const unsigned nt = a.K / 32;
     const float c = a.alpha * LOG2E;
 
-    h8 fq[G::NKS], fdo[G::NKS], fv[G::NKS], kr[G::VL];
-    row_frags<P>(a.q, h, b, j, hi, fq);
-    row_frags<P>(a.d_o, h, b, j, hi, fdo);
-    float dsum;
-    {
-        h8 fo[G::NKS];
+    h8 fq[G::NKS], fdo[G::NKS], fk[G::NKS], fv[G::NKS], kr[G::VL], vr[G::VL];
+    float dsum, lse;
+    uint32_t word;
+    {   // the first two tiles, the rows of this lane's query and its statistics: all
+        // loads in flight together
+        h8 kr1[G::VL], vr1[G::VL], fo[G::NKS];
+        tile_fetch<P>(a.k, h, b, 0, tid, kr);
+        tile_fetch<P>(a.v, h, b, 0, tid, vr);
+        tile_fetch<P>(a.k, h, b, 32, tid, kr1);
+        tile_fetch<P>(a.v, h, b, 32, tid, vr1);
+        row_frags<P>(a.q, h, b, j, hi, fq);
+        row_frags<P>(a.d_o, h, b, j, hi, fdo);
         row_frags<P>(a.o, h, b, j, hi, fo);
+        lse = a.lse[row];
+        word = a.keep[(size_t)row * nt];
+        tile_put<P>(kt[0], tid, kr);
+        tile_put<P>(vt[0], tid, vr);
+        tile_put<P>(kt[1], tid, kr1);
+        tile_put<P>(vt[1], tid, vr1);
         float part = 0.f;
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks)
@@ -249,31 +363,25 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         dsum = part + __shfl_xor(part, 32);
         if (hi == 0) a.dsum[row] = dsum;
     }
-    const float lse = a.lse[row];
-    row_frags<P>(a.v, h, b, l32, hi, fv);
-    tile_fetch<P>(a.k, h, b, 0, tid, kr);
-    tile_put<P>(kt[0], tid, kr);
-    uint32_t word = a.keep[(size_t)row * nt];
     __syncthreads();
+    row_frags_lds<P>(kt[0], l32, hi, fk);
+    row_frags_lds<P>(vt[0], l32, hi, fv);
 
     f16v dq[G::NPT];
 #pragma unroll
     for (int pt = 0; pt < G::NPT; ++pt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) dq[pt][v] = 0.f;
+    int cur = 0, nxt = 1, nn = 2;
+    wait_loads();
 
     for (unsigned t = 0; t < nt; ++t) {
-        h8 fvn[G::NKS];
-        uint32_t wordn = 0;
-        const bool more = t + 1 < nt;
-        if (more) {
-            row_frags<P>(a.v, h, b, (t + 1) * 32 + l32, hi, fvn);
-            tile_fetch<P>(a.k, h, b, (t + 1) * 32, tid, kr);
-            wordn = a.keep[(size_t)row * nt + t + 1];
+        const bool fetch = t + 2 < nt;
+        if (fetch) {
+            tile_fetch<P>(a.k, h, b, (t + 2) * 32, tid, kr);
+            tile_fetch<P>(a.v, h, b, (t + 2) * 32, tid, vr);
         }
-        const half_t* ktile = kt[t & 1];
-        h8 fk[G::NKS];
-        row_frags_lds<P>(ktile, l32, hi, fk);
+        const uint32_t wordn = t + 1 < nt ? a.keep[(size_t)row * nt + t + 1] : 0u;
         f16v s, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
@@ -281,27 +389,41 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fv[ks], fdo[ks], dp, 0, 0, 0);
+        h8 ka[2][G::NPT];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int pt = 0; pt < G::NPT; ++pt) ka[st][pt] = tr_frag<P>(kt[cur], pt * 32, st, lane);
+        row_frags_lds<P>(kt[nxt], l32, hi, fk);
+        row_frags_lds<P>(vt[nxt], l32, hi, fv);
         const uint32_t nib = word >> (hi * 4);
+        // stage by stage over the 16 scores of the lane, so that consecutive
+        // instructions do not depend on one another
         h8 ds[2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -lse));
-            const float g = ((nib >> reg_pos(v, 0)) & 1u) ? dp[v] : 0.f;
-            ds[v >> 3][v & 7] = (half_t)(p * (g - dsum));
-        }
+        for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], c, -lse);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v]);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[v] = keep_if(dp[v], nib, reg_pos(v, 0));
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dp[v] -= dsum;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] *= dp[v];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ds[v >> 3][v & 7] = (half_t)s[v];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int pt = 0; pt < G::NPT; ++pt)
-                dq[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(tr_frag(ktile, G::PITCH, pt * 32, st, lane), ds[st],
-                                                                dq[pt], 0, 0, 0);
-        if (more) {
-            tile_put<P>(kt[(t + 1) & 1], tid, kr);
-#pragma unroll
-            for (int ks = 0; ks < G::NKS; ++ks) fv[ks] = fvn[ks];
-            word = wordn;
+                dq[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[st][pt], ds[st], dq[pt], 0, 0, 0);
+        if (fetch) {
+            tile_put<P>(kt[nn], tid, kr);
+            tile_put<P>(vt[nn], tid, vr);
         }
+        word = wordn;
         __syncthreads();
+        const int x = cur; cur = nxt; nxt = nn; nn = x;
     }
     store_rows<P>(a.dq, h, b, j, hi, dq, a.alpha);
 }
@@ -323,57 +445,69 @@ struct KvStage {
 template <int P>
 __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
     using G = Geo<P>;
-    __shared__ __attribute__((aligned(16))) KvStage<P> stage[2];
+    __shared__ __attribute__((aligned(16))) KvStage<P> stage[RING];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned kblocks = a.K / QB;
-    const unsigned kb = blockIdx.x % kblocks, hb = blockIdx.x / kblocks;
+    const unsigned lb = logical_block();
+    const unsigned kb = lb % kblocks, hb = lb / kblocks;
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned kpos = kb * QB + wave * 32 + l32;                 // this lane's key
     const unsigned row0 = (h * a.B + b) * a.J;                       // score row of query 0
     const unsigned nq = a.J / 32, nkt = a.K / 32;
     const float c = a.alpha * LOG2E;
 
-    h8 fk[G::NKS], fv[G::NKS], qr[G::VL], dr[G::VL];
-    float stat = 0.f;
-    uint4 kw = make_uint4(0, 0, 0, 0);
-    row_frags<P>(a.k, h, b, kpos, hi, fk);
-    row_frags<P>(a.v, h, b, kpos, hi, fv);
-
-    auto fetch = [&](unsigned qt) {
-        tile_fetch<P>(a.q, h, b, qt * 32, tid, qr);
-        tile_fetch<P>(a.d_o, h, b, qt * 32, tid, dr);
-        const unsigned r = row0 + qt * 32 + (tid & 31);
-        if (tid < 32) stat = a.lse[r];
-        else if (tid < 64) stat = a.dsum[r];
-        else if (tid < 96) kw = *reinterpret_cast<const uint4*>(a.keep + (size_t)r * nkt + kb * 4);
+    h8 fk[G::NKS], fv[G::NKS], fq[G::NKS], fdo[G::NKS];
+    struct InFlight {             // one tile of queries on its way from memory
+        h8 q[G::VL], d_o[G::VL];
+        float stat;
+        uint4 kw;
     };
-    auto put = [&](KvStage<P>& s) {
-        tile_put<P>(s.q, tid, qr);
-        tile_put<P>(s.d_o, tid, dr);
-        if (tid < 32) s.lse[tid] = stat;
-        else if (tid < 64) s.dsum[tid - 32] = stat;
+    auto fetch = [&](unsigned qt, InFlight& f) {
+        tile_fetch<P>(a.q, h, b, qt * 32, tid, f.q);
+        tile_fetch<P>(a.d_o, h, b, qt * 32, tid, f.d_o);
+        const unsigned r = row0 + qt * 32 + (tid & 31);
+        if (tid < 32) f.stat = a.lse[r];
+        else if (tid < 64) f.stat = a.dsum[r];
+        else if (tid < 96) f.kw = *reinterpret_cast<const uint4*>(a.keep + (size_t)r * nkt + kb * 4);
+    };
+    auto put = [&](KvStage<P>& sg, const InFlight& f) {
+        tile_put<P>(sg.q, tid, f.q);
+        tile_put<P>(sg.d_o, tid, f.d_o);
+        if (tid < 32) sg.lse[tid] = f.stat;
+        else if (tid < 64) sg.dsum[tid - 32] = f.stat;
         else if (tid < 96) {
-            s.keep[0][tid - 64] = kw.x; s.keep[1][tid - 64] = kw.y;
-            s.keep[2][tid - 64] = kw.z; s.keep[3][tid - 64] = kw.w;
+            sg.keep[0][tid - 64] = f.kw.x; sg.keep[1][tid - 64] = f.kw.y;
+            sg.keep[2][tid - 64] = f.kw.z; sg.keep[3][tid - 64] = f.kw.w;
         }
     };
-    fetch(0);
-    put(stage[0]);
+    InFlight fl;
+    fl.stat = 0.f; fl.kw = make_uint4(0, 0, 0, 0);
+    {
+        InFlight f1;
+        f1.stat = 0.f; f1.kw = make_uint4(0, 0, 0, 0);
+        fetch(0, fl);
+        fetch(1, f1);
+        row_frags<P>(a.k, h, b, kpos, hi, fk);
+        row_frags<P>(a.v, h, b, kpos, hi, fv);
+        put(stage[0], fl);
+        put(stage[1], f1);
+    }
     __syncthreads();
+    row_frags_lds<P>(stage[0].q, l32, hi, fq);
+    row_frags_lds<P>(stage[0].d_o, l32, hi, fdo);
 
     f16v dk[G::NPT], dv[G::NPT];
 #pragma unroll
     for (int pt = 0; pt < G::NPT; ++pt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) { dk[pt][v] = 0.f; dv[pt][v] = 0.f; }
+    int cur = 0, nxt = 1, nn = 2;
+    wait_loads();
 
     for (unsigned qt = 0; qt < nq; ++qt) {
-        const bool more = qt + 1 < nq;
-        if (more) fetch(qt + 1);
-        const KvStage<P>& sg = stage[qt & 1];
-        h8 fq[G::NKS], fdo[G::NKS];
-        row_frags_lds<P>(sg.q, l32, hi, fq);
-        row_frags_lds<P>(sg.d_o, l32, hi, fdo);
+        const bool more = qt + 2 < nq;
+        if (more) fetch(qt + 2, fl);
+        const KvStage<P>& sg = stage[cur];
         f16v s, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
@@ -381,6 +515,16 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[ks], fk[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fdo[ks], fv[ks], dp, 0, 0, 0);
+        h8 qa[2][G::NPT], da[2][G::NPT];
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+            for (int pt = 0; pt < G::NPT; ++pt) {
+                da[st][pt] = tr_frag<P>(sg.d_o, pt * 32, st, lane);
+                qa[st][pt] = tr_frag<P>(sg.q, pt * 32, st, lane);
+            }
+        row_frags_lds<P>(stage[nxt].q, l32, hi, fq);
+        row_frags_lds<P>(stage[nxt].d_o, l32, hi, fdo);
         // D[query, key]: lane = key, register v = query reg_pos(v, hi)
         h8 pd[2], ds[2];
 #pragma unroll
@@ -394,22 +538,21 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
             for (int e = 0; e < 4; ++e) {
                 const int v = q * 4 + e;
                 const float p = __builtin_amdgcn_exp2f(fmaf(s[v], c, -lsv[e]));
-                const bool keep = (wv[e] >> l32) & 1u;
-                pd[v >> 3][v & 7] = keep ? (half_t)p : (half_t)0.0f;
-                ds[v >> 3][v & 7] = (half_t)(p * ((keep ? dp[v] : 0.f) - ddv[e]));
+                const int keep = __builtin_amdgcn_sbfe((int)wv[e], l32, 1);
+                pd[v >> 3][v & 7] = (half_t)__int_as_float(__float_as_int(p) & keep);
+                ds[v >> 3][v & 7] = (half_t)(p * (__int_as_float(__float_as_int(dp[v]) & keep) - ddv[e]));
             }
         }
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int pt = 0; pt < G::NPT; ++pt) {
-                dv[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(tr_frag(sg.d_o, G::PITCH, pt * 32, st, lane), pd[st],
-                                                                dv[pt], 0, 0, 0);
-                dk[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(tr_frag(sg.q, G::PITCH, pt * 32, st, lane), ds[st],
-                                                                dk[pt], 0, 0, 0);
+                dv[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(da[st][pt], pd[st], dv[pt], 0, 0, 0);
+                dk[pt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(qa[st][pt], ds[st], dk[pt], 0, 0, 0);
             }
-        if (more) put(stage[(qt + 1) & 1]);
+        if (more) put(stage[nn], fl);
         __syncthreads();
+        const int x = cur; cur = nxt; nxt = nn; nn = x;
     }
     store_rows<P>(a.dk, h, b, kpos, hi, dk, a.alpha);
     store_rows<P>(a.dv, h, b, kpos, hi, dv, 1.0f);
@@ -432,7 +575,7 @@ size_t mha_stat_bytes(long H, long B, long J) { return (size_t)(H * B * J) * 2 *
 size_t mha_keep_bytes(long H, long B, long J, long K) { return (size_t)(H * B * J) * (size_t)(K / 32) * 4; }
 
 bool mha_forward_ok(const AttnArgs& a, int P) {
-    return mha_shape_ok(a.H, a.B, a.J, a.K, P) && side_ok(a.q) && side_ok(a.k) && side_ok(a.v) && side_ok(a.o) &&
+    return mha_shape_ok(a.H, a.B, a.J, a.K, P) && a.alpha > 0.f && side_ok(a.q) && side_ok(a.k) && side_ok(a.v) && side_ok(a.o) &&
            a.lse && a.keep && (reinterpret_cast<uintptr_t>(a.lse) & 15) == 0 &&
            (reinterpret_cast<uintptr_t>(a.keep) & 15) == 0;
 }
