@@ -38,15 +38,12 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 88459096, 'QKT+softmax': 243621964, 'gamma': 84146854,
-    'out': 33775322, 'bdrln1': 59004898, 'lin1': 84251672,
-    'bad': 134455796, 'lin2': 109264961, 'bdrln2': 59010969,
-    'bsb+blnrd1': 61022307, 'dXlin2': 84238416, 'dWlin2': 109275401,
-    'bdrlb': 135394524, 'dXlin1': 109260573, 'dWlin1': 109274908,
-    'ebsb+blnrd2+baob': 79940187, 'dWout': 129229442, 'dXout': 33771117,
-    'dX2gamma': 84108147, 'dX1gamma+bs': 243472205, 'dX1QKT': 84108312,
-    'dX2QKT': 84090851, 'dXQKV-fused': 92485098, 'dWQKV-fused': 115565493,
-    'baib': 25997182,
+    'QKV-fused': 88458689, 'attention': 38113369, 'out': 33775290, 'bdrln1': 59014038,
+    'lin1': 84251664, 'bad': 134454950, 'lin2': 109264818, 'bdrln2': 59011094,
+    'bsb+blnrd1': 61022393, 'dXlin2': 84238426, 'dWlin2': 109275276, 'bdrlb': 135394527,
+    'dXlin1': 109260448, 'dWlin1': 109274947, 'ebsb+blnrd2+baob': 79939868, 'dWout': 101803120,
+    'dXout': 33771067, 'attention-bwd-dQ': 55131503, 'attention-bwd-dKdV': 55150951,
+    'dXQKV-fused': 92484993, 'dWQKV-fused': 115565358, 'baib': 25997151,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',

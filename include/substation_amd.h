@@ -164,8 +164,18 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * the operators run separately (results then agree to fp16 rounding, not bit
  * for bit, because probabilities are no longer rounded before the weighted sum).
  * Set the option before the forward call and leave it until after the matching
- * backward call. */
+ * backward call.  Value 2 (SUB_FUSE_REQUIRED) makes both calls fail rather
+ * than fall back: a caller that has asked sub_attention_in_registers() and got
+ * 1 may then pass token allocations (any non-null pointer) for the four tensors
+ * that are neither written nor read -- BETA, ATTN_DROP, DATTN_DROP, DBETA --
+ * and needs only 8 bytes per score row behind ALPHA and K/8 bytes per score
+ * row behind ATTN_DROP_MASK (both 16-byte aligned). */
 #define SUB_OPT_FUSE_ATTENTION 4
+#define SUB_FUSE_REQUIRED 2
+/* *planned = 1 when, with the handle's sizes, layouts, attention mask and
+ * options as they are now, self-attention runs with the scores in registers
+ * (given 16-byte aligned tensors).  No counterpart in the reference. */
+int sub_attention_in_registers(void* handle, int* planned);
 int sub_set_option(void* handle, int option, int value);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same

@@ -18,6 +18,7 @@ OPT_FUSE_EPILOGUES = 1
 OPT_FUSE_LN_BACKWARD = 2
 OPT_FUSE_SCORES = 3
 OPT_FUSE_ATTENTION = 4
+FUSE_REQUIRED = 2
 
 
 class SubConfig(ctypes.Structure):
@@ -55,6 +56,7 @@ SIGNATURES = {
     'sub_set_rng_counter': (_I, [_VP, _VP]),
     'sub_last_error': (_CP, []),
     'sub_set_option': (_I, [_VP, _I, _I]),
+    'sub_attention_in_registers': (_I, [_VP, ctypes.POINTER(_I)]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_profile_enable': (_I, [_VP, _I]),
@@ -176,6 +178,12 @@ class Handle:
 
     def set_option(self, option, value):
         check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')
+
+    def attention_in_registers(self):
+        """True when self-attention will run with the scores kept in registers."""
+        out = _I(0)
+        check(self.lib.sub_attention_in_registers(self.ptr, ctypes.byref(out)), 'sub_attention_in_registers')
+        return bool(out.value)
 
     def profile_enable(self, on=True):
         check(self.lib.sub_profile_enable(self.ptr, 1 if on else 0), 'sub_profile_enable')

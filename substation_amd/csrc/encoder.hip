@@ -183,7 +183,7 @@ struct Handle {
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
     bool fuse_scores = true;
-    bool fuse_attention = true;
+    int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -569,27 +569,40 @@ bool attn_side(const void* p, const Layout& l, int pos_dim, AttnSide& s) {
     return true;
 }
 
-// Decided from what the forward pass sees, so that both passes take the same path.
-bool attention_fused(const Handle& h, void* const* F, AttnArgs& a) {
+// What sizes, layouts and options say; tensor alignment is checked per call.
+bool attention_planned(const Handle& h) {
     if (!h.fuse_attention || h.attn_mask) return false;
     const Sizes& z = h.sz;
-    if (!mha_shape_ok(z.n[dH], z.n[dB], z.n[dJ], z.n[dK], z.n[dP])) return false;
-    a.H = (int)z.n[dH]; a.B = (int)z.n[dB]; a.J = (int)z.n[dJ]; a.K = (int)z.n[dK];
-    a.alpha = h.gemm[G_QKT].alpha;
-    half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
-    if (!attn_side(QQ, h.lQQ, dJ, a.q) || !attn_side(KK, h.lKK, dK, a.k) || !attn_side(VV, h.lKK, dK, a.v) ||
-        !attn_side(F[GAMMA], h.lf[GAMMA], dJ, a.o))
-        return false;
-    // the backward pass's tensors must qualify too (layouts only; pointers are checked there)
+    if (!mha_shape_ok(z.n[dH], z.n[dB], z.n[dJ], z.n[dK], z.n[dP]) || !(h.gemm[G_QKT].alpha > 0.f)) return false;
     AttnSide t;
-    if (!attn_side(nullptr, h.lb[DGAMMA], dJ, t) || !attn_side(nullptr, h.lDQQ, dJ, t) ||
-        !attn_side(nullptr, h.lDKK, dK, t))
-        return false;
-    const size_t rows = (size_t)a.H * a.B * a.J;
-    if (mha_stat_bytes(a.H, a.B, a.J) > rows * a.K * sizeof(half_t)) return false;
-    a.lse = (float*)F[ALPHA]; a.dsum = a.lse + rows;
-    a.keep = (uint32_t*)F[ATTN_DROP_MASK];
-    return mha_forward_ok(a, (int)z.n[dP]);
+    return attn_side(nullptr, h.lQQ, dJ, t) && attn_side(nullptr, h.lKK, dK, t) &&
+           attn_side(nullptr, h.lf[GAMMA], dJ, t) && attn_side(nullptr, h.lb[DGAMMA], dJ, t) &&
+           attn_side(nullptr, h.lDQQ, dJ, t) && attn_side(nullptr, h.lDKK, dK, t) &&
+           mha_stat_bytes(z.n[dH], z.n[dB], z.n[dJ]) <=
+               (size_t)(z.n[dH] * z.n[dB] * z.n[dJ] * z.n[dK]) * sizeof(half_t);
+}
+
+// Decided from what the forward pass sees, so that both passes take the same path.
+// With the option at SUB_FUSE_REQUIRED a caller may have handed over token-sized
+// stand-ins for the tensors this path does not touch: then there is no way back.
+bool attention_fused(const Handle& h, void* const* F, AttnArgs& a) {
+    bool ok = attention_planned(h);
+    if (ok) {
+        const Sizes& z = h.sz;
+        a.H = (int)z.n[dH]; a.B = (int)z.n[dB]; a.J = (int)z.n[dJ]; a.K = (int)z.n[dK];
+        a.alpha = h.gemm[G_QKT].alpha;
+        half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1);
+        half_t* VV = sub_q(F[KKQQVV], h, 2);
+        attn_side(QQ, h.lQQ, dJ, a.q); attn_side(KK, h.lKK, dK, a.k); attn_side(VV, h.lKK, dK, a.v);
+        attn_side(F[GAMMA], h.lf[GAMMA], dJ, a.o);
+        a.lse = (float*)F[ALPHA]; a.dsum = a.lse + (size_t)a.H * a.B * a.J;
+        a.keep = (uint32_t*)F[ATTN_DROP_MASK];
+        ok = mha_forward_ok(a, (int)z.n[dP]);
+    }
+    if (!ok && h.fuse_attention == SUB_FUSE_REQUIRED)
+        fail("attention with the scores in registers was required (SUB_OPT_FUSE_ATTENTION = 2) but the sizes, "
+             "layouts, attention mask or tensor alignment rule it out");
+    return ok;
 }
 
 // bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
@@ -1025,8 +1038,20 @@ int sub_set_option(void* handle, int option, int value) {
         if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
         else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
         else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
-        else if (option == SUB_OPT_FUSE_ATTENTION) h.fuse_attention = value != 0;
+        else if (option == SUB_OPT_FUSE_ATTENTION) {
+            if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
+            h.fuse_attention = value;
+        }
         else fail("sub_set_option: unknown option");
+    });
+}
+
+int sub_attention_in_registers(void* handle, int* planned) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        need_cfg(h);
+        if (!planned) fail("sub_attention_in_registers: null result pointer");
+        *planned = attention_planned(h) ? 1 : 0;
     });
 }
 

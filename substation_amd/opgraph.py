@@ -17,6 +17,7 @@ from . import layouts as _lay
 OPERATORS = [
     ('QKV-fused', 'fwd', ('X', 'WKQV', 'BKQV', 'WKKWQQWVV', 'KKQQVV')),
     ('aib', 'fwd', ('WKKWQQWVV', 'BKQV', 'KKQQVV')),
+    ('attention', 'fwd', ('KKQQVV', 'BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP', 'GAMMA')),
     ('QKT+softmax', 'fwd', ('KKQQVV', 'BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP')),
     ('QKT', 'fwd', ('KKQQVV', 'BETA')),
     ('softmax', 'fwd', ('BETA', 'ALPHA', 'ATTN_DROP_MASK', 'ATTN_DROP')),
@@ -42,6 +43,10 @@ OPERATORS = [
     ('baob', 'bwd', ('DATT',)),
     ('dWout', 'bwd', ('GAMMA', 'DATT', 'WO')),
     ('dXout', 'bwd', ('WO', 'DATT', 'DGAMMA')),
+    ('attention-bwd-dQ', 'bwd', ('KKQQVV', 'GAMMA', 'DGAMMA', 'DATTN_DROP', 'ALPHA', 'ATTN_DROP_MASK', 'DBETA',
+                                 'DKKQQVV')),
+    ('attention-bwd-dKdV', 'bwd', ('KKQQVV', 'DGAMMA', 'ATTN_DROP', 'DATTN_DROP', 'ALPHA', 'ATTN_DROP_MASK',
+                                   'DBETA', 'DKKQQVV')),
     ('dX1gamma+bs', 'bwd', ('KKQQVV', 'DGAMMA', 'DATTN_DROP', 'ALPHA', 'ATTN_DROP_MASK', 'DBETA')),
     ('dX1gamma', 'bwd', ('KKQQVV', 'DGAMMA', 'DATTN_DROP')),
     ('dX2gamma', 'bwd', ('DGAMMA', 'ATTN_DROP', 'DKKQQVV')),
@@ -62,8 +67,8 @@ OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused', 'bei'),
-    ('QKT+softmax', 'QKT', 'softmax'),
-    ('dX1gamma+bs', 'dX1gamma', 'bs'),
+    ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
+    ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT'),
     ('bsb+blnrd1', 'bsb', 'blnrd1'),
     ('ebsb+blnrd2+baob', 'ebsb', 'blnrd2', 'baob'),
 ]

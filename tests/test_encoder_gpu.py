@@ -321,6 +321,44 @@ def test_attention_in_registers_matches_separate_operators(which, dims, act, p):
         assert_close(b.float().cpu().numpy(), a.float().cpu().numpy(), tol=1e-2, name=name)
 
 
+def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback():
+    """compact_attention=True allocates token buffers for the score-sized tensors
+    the in-register attention never touches and a few bytes per row for the two
+    it keeps statistics and keep bits in: results are bit-identical, and anything
+    that would need the full tensors (here: an attention mask) is refused."""
+    from substation_amd import Encoder, causal_mask, layouts as L
+    from substation_amd._lib import SubstationError
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = 2, 256, 4, 256
+    outs = []
+    for compact in (False, True):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                      compact_attention=compact).cuda()
+        assert enc.compact_attention == compact
+        enc.set_rng(SEED, 0)
+        g = torch.Generator().manual_seed(5)
+        X = (0.5 * torch.randn(B, Ls, E, generator=g)).half().cuda().requires_grad_(True)
+        DY = torch.randn(B, Ls, E, generator=g).half().cuda()
+        with torch.no_grad():
+            for q in enc.parameters():
+                q.mul_(0.1)
+        for _ in range(2):                      # twice: the buffers are reallocated per call
+            X.grad = None
+            Y = enc(X)
+            Y.backward(DY)
+        torch.cuda.synchronize()
+        outs.append([Y.detach().clone(), X.grad.clone()] + [q.grad.clone() for q in enc.parameters()])
+    for a, b in zip(*outs):
+        assert torch.isfinite(a.float()).all()
+        assert torch.equal(a, b)
+    enc.set_attention_mask(causal_mask(Ls, 'cuda', torch.float16))
+    with pytest.raises(SubstationError, match='required'):
+        enc(X)
+    enc.set_attention_mask(None)
+    enc(X)
+
+
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
     """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
     the library's one-time allocations) and replayed with eager work in between:
