@@ -160,7 +160,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * the ones handed to the matching backward call, as in the reference).  The
  * dropout mask is the same counter-based one as in the separate operators.
  * Needs head size 64 or 128, sequence lengths that are multiples of 128,
- * feature-contiguous projections and no attention mask; otherwise, or with 0,
+ * and feature-contiguous projections (an attention mask set with
+ * sub_set_attention_mask is added to the score tiles); otherwise, or with 0,
  * the operators run separately (results then agree to fp16 rounding, not bit
  * for bit, because probabilities are no longer rounded before the weighted sum).
  * Set the option before the forward call and leave it until after the matching
@@ -172,8 +173,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * row behind ATTN_DROP_MASK (both 16-byte aligned). */
 #define SUB_OPT_FUSE_ATTENTION 4
 #define SUB_FUSE_REQUIRED 2
-/* *planned = 1 when, with the handle's sizes, layouts, attention mask and
- * options as they are now, self-attention runs with the scores in registers
+/* *planned = 1 when, with the handle's sizes, layouts and options as they are
+ * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */
 int sub_attention_in_registers(void* handle, int* planned);
 int sub_set_option(void* handle, int option, int value);

@@ -571,7 +571,7 @@ bool attn_side(const void* p, const Layout& l, int pos_dim, AttnSide& s) {
 
 // What sizes, layouts and options say; tensor alignment is checked per call.
 bool attention_planned(const Handle& h) {
-    if (!h.fuse_attention || h.attn_mask) return false;
+    if (!h.fuse_attention) return false;
     const Sizes& z = h.sz;
     if (!mha_shape_ok(z.n[dH], z.n[dB], z.n[dJ], z.n[dK], z.n[dP]) || !(h.gemm[G_QKT].alpha > 0.f)) return false;
     AttnSide t;
@@ -597,11 +597,15 @@ bool attention_fused(const Handle& h, void* const* F, AttnArgs& a) {
         attn_side(F[GAMMA], h.lf[GAMMA], dJ, a.o);
         a.lse = (float*)F[ALPHA]; a.dsum = a.lse + (size_t)a.H * a.B * a.J;
         a.keep = (uint32_t*)F[ATTN_DROP_MASK];
+        if (h.attn_mask) {
+            a.amask = (const half_t*)h.attn_mask;
+            a.am_sj = h.l_attn_mask.stride[dJ]; a.am_sk = h.l_attn_mask.stride[dK];
+        }
         ok = mha_forward_ok(a, (int)z.n[dP]);
     }
     if (!ok && h.fuse_attention == SUB_FUSE_REQUIRED)
         fail("attention with the scores in registers was required (SUB_OPT_FUSE_ATTENTION = 2) but the sizes, "
-             "layouts, attention mask or tensor alignment rule it out");
+             "layouts or tensor alignment rule it out");
     return ok;
 }
 

@@ -177,6 +177,27 @@ __device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
     return b;
 }
 
+// Additive attention mask (substation/attention.py:65-68: added to the raw scores,
+// before the scaling) for the 16 scores of a lane.  QUERY_LANES: the lane holds
+// one query and registers run over keys (forward, dQ); otherwise the lane holds
+// one key and registers run over queries (dK/dV).
+template <bool QUERY_LANES>
+__device__ __forceinline__ void add_mask(const AttnArgs& a, unsigned lane_pos, unsigned tile0, int hi, f16v& s) {
+    const long lane_stride = QUERY_LANES ? a.am_sj : a.am_sk, reg_stride = QUERY_LANES ? a.am_sk : a.am_sj;
+    const half_t* m = a.amask + (long)lane_pos * lane_stride + (long)tile0 * reg_stride;
+    if (reg_stride == 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const h4 w = *reinterpret_cast<const h4*>(m + q * 8 + hi * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) s[q * 4 + e] += (float)w[e];
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] += (float)m[(long)reg_pos(v, hi) * reg_stride];
+    }
+}
+
 // ---------------------------------------------------------------------------
 // All three kernels stream tiles of 32 positions through a ring of three LDS
 // buffers: while tile t is worked on, tile t+1 already lies in LDS (its row
@@ -193,7 +214,7 @@ __device__ __forceinline__ void wait_loads() { __builtin_amdgcn_s_waitcnt(0x0F70
 // ---------------------------------------------------------------------------
 // forward.  grid = H * B * (J / 128); wave = 32 queries.
 // ---------------------------------------------------------------------------
-template <int P>
+template <int P, bool MASKED>
 __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
     using G = Geo<P>;
     __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
@@ -246,6 +267,7 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
+        if (MASKED) add_mask<true>(a, j, t * 32, hi, s);
         // fragments for the second product of this tile and the first of the next
         h8 va[2][G::NPT];
 #pragma unroll
@@ -285,7 +307,8 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[pt][v] *= corr;
         }
-        const float mc = -m_ref * c;
+        // (masked: a query whose keys so far are all masked out has no reference yet)
+        const float mc = (MASKED && m_ref == -INFINITY) ? 0.f : -m_ref * c;
         h8 pb[2];
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], c, mc);
@@ -321,7 +344,7 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
 // ---------------------------------------------------------------------------
 // backward, dQ.  grid = H * B * (J / 128); wave = 32 queries.
 // ---------------------------------------------------------------------------
-template <int P>
+template <int P, bool MASKED>
 __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
     using G = Geo<P>;
     __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
@@ -389,6 +412,7 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fv[ks], fdo[ks], dp, 0, 0, 0);
+        if (MASKED) add_mask<true>(a, j, t * 32, hi, s);
         h8 ka[2][G::NPT];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
@@ -442,7 +466,7 @@ struct KvStage {
     uint32_t keep[4][32];         // [wave's key tile][query]
 };
 
-template <int P>
+template <int P, bool MASKED>
 __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
     using G = Geo<P>;
     __shared__ __attribute__((aligned(16))) KvStage<P> stage[RING];
@@ -515,6 +539,7 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[ks], fk[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fdo[ks], fv[ks], dp, 0, 0, 0);
+        if (MASKED) add_mask<false>(a, kpos, qt * 32, hi, s);
         h8 qa[2][G::NPT], da[2][G::NPT];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
@@ -558,6 +583,15 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
     store_rows<P>(a.dv, h, b, kpos, hi, dv, 1.0f);
 }
 
+// 8-byte loads of four mask values along whichever dim is contiguous
+bool mask_ok(const AttnArgs& a) {
+    if (!a.amask) return true;
+    if ((reinterpret_cast<uintptr_t>(a.amask) & 7) != 0) return false;
+    if (a.am_sk == 1) return a.am_sj % 4 == 0;
+    if (a.am_sj == 1) return a.am_sk % 4 == 0;
+    return true;
+}
+
 bool side_ok(const AttnSide& s) {
     return s.p && (reinterpret_cast<uintptr_t>(s.p) & 15) == 0 && s.sh % 8 == 0 && s.sb % 8 == 0 && s.sr % 8 == 0;
 }
@@ -577,14 +611,19 @@ size_t mha_keep_bytes(long H, long B, long J, long K) { return (size_t)(H * B * 
 bool mha_forward_ok(const AttnArgs& a, int P) {
     return mha_shape_ok(a.H, a.B, a.J, a.K, P) && a.alpha > 0.f && side_ok(a.q) && side_ok(a.k) && side_ok(a.v) && side_ok(a.o) &&
            a.lse && a.keep && (reinterpret_cast<uintptr_t>(a.lse) & 15) == 0 &&
-           (reinterpret_cast<uintptr_t>(a.keep) & 15) == 0;
+           (reinterpret_cast<uintptr_t>(a.keep) & 15) == 0 && mask_ok(a);
 }
 
 void launch_mha_forward(const AttnArgs& a, int P, PhiloxKey key, hipStream_t st) {
     if (!mha_forward_ok(a, P)) fail("attention forward: shape, strides or alignment not supported");
     dim3 grid((unsigned)(a.H * a.B * (a.J / QB)));
-    if (P == 64) hipLaunchKernelGGL(k_mha_fwd<64>, grid, dim3(256), 0, st, a, key);
-    else hipLaunchKernelGGL(k_mha_fwd<128>, grid, dim3(256), 0, st, a, key);
+    if (a.amask) {
+        if (P == 64) hipLaunchKernelGGL((k_mha_fwd<64, true>), grid, dim3(256), 0, st, a, key);
+        else hipLaunchKernelGGL((k_mha_fwd<128, true>), grid, dim3(256), 0, st, a, key);
+    } else {
+        if (P == 64) hipLaunchKernelGGL((k_mha_fwd<64, false>), grid, dim3(256), 0, st, a, key);
+        else hipLaunchKernelGGL((k_mha_fwd<128, false>), grid, dim3(256), 0, st, a, key);
+    }
     check_launch("attention forward");
 }
 
@@ -595,16 +634,26 @@ bool mha_backward_ok(const AttnArgs& a, int P) {
 void launch_mha_backward_dq(const AttnArgs& a, int P, hipStream_t st) {
     if (!mha_backward_ok(a, P)) fail("attention backward: shape, strides or alignment not supported");
     dim3 grid((unsigned)(a.H * a.B * (a.J / QB)));
-    if (P == 64) hipLaunchKernelGGL(k_mha_bwd_dq<64>, grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(k_mha_bwd_dq<128>, grid, dim3(256), 0, st, a);
+    if (a.amask) {
+        if (P == 64) hipLaunchKernelGGL((k_mha_bwd_dq<64, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((k_mha_bwd_dq<128, true>), grid, dim3(256), 0, st, a);
+    } else {
+        if (P == 64) hipLaunchKernelGGL((k_mha_bwd_dq<64, false>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((k_mha_bwd_dq<128, false>), grid, dim3(256), 0, st, a);
+    }
     check_launch("attention backward (dQ)");
 }
 
 void launch_mha_backward_dkv(const AttnArgs& a, int P, hipStream_t st) {
     if (!mha_backward_ok(a, P)) fail("attention backward: shape, strides or alignment not supported");
     dim3 grid((unsigned)(a.H * a.B * (a.K / QB)));
-    if (P == 64) hipLaunchKernelGGL(k_mha_bwd_dkv<64>, grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(k_mha_bwd_dkv<128>, grid, dim3(256), 0, st, a);
+    if (a.amask) {
+        if (P == 64) hipLaunchKernelGGL((k_mha_bwd_dkv<64, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((k_mha_bwd_dkv<128, true>), grid, dim3(256), 0, st, a);
+    } else {
+        if (P == 64) hipLaunchKernelGGL((k_mha_bwd_dkv<64, false>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((k_mha_bwd_dkv<128, false>), grid, dim3(256), 0, st, a);
+    }
     check_launch("attention backward (dK, dV)");
 }
 

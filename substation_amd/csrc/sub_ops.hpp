@@ -122,6 +122,8 @@ struct AttnArgs {
     uint32_t* keep = nullptr;  // [H*B*J][K/32]  keep bits of the softmax dropout, bit k%32 of word k/32
     int H = 0, B = 0, J = 0, K = 0;
     float alpha = 1.f;         // score scale
+    const half_t* amask = nullptr;   // optional additive mask over (query, key), added before the scaling
+    long am_sj = 0, am_sk = 0;
 };
 // head_size 64 or 128, J and K multiples of 128
 bool mha_shape_ok(long H, long B, long J, long K, long head_size);

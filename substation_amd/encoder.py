@@ -121,6 +121,9 @@ class Encoder(torch.nn.Module):
                 if tuple(X.shape) != in_shape:
                     raise ValueError(f"X has shape {tuple(X.shape)}, the configured input layout "
                                      f"{layouts['input'][1]} needs {in_shape}")
+                if module.compact_attention and not handle.attention_in_registers():
+                    raise RuntimeError('this Encoder was built with compact_attention=True but the attention '
+                                       'kernels that keep the scores in registers are switched off')
                 dev = X.device
                 X = X.contiguous()
                 # same element count as X, shaped in the output's own dimension order

@@ -279,32 +279,48 @@ def test_fused_epilogues_match_unfused(which, dims, act):
         assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize('which,dims,act,p', [
-    ('mi355x', (2, 128, 2, 128), 'gelu', 0.1),
-    ('mi355x', (2, 128, 2, 128), 'gelu', 0.0),
-    ('mi355x', (3, 384, 2, 128), 'gelu', 0.5),           # three blocks of 128 positions
-    ('mi355x', (2, 256, 2, 256), 'gelu', 0.1),           # head size 128
-    ('bert-b8-l512-h16-e1024', (2, 128, 2, 128), 'gelu', 0.1),   # the reference's layouts: falls back, still equal
-    ('mi355x:bert-b96-l128-h16-e1024', (16, 128, 16, 1024), 'gelu', 0.1),
-    ('mi355x', (8, 512, 16, 1024), 'gelu', 0.1),
+@pytest.mark.parametrize('which,dims,act,p,mask', [
+    ('mi355x', (2, 128, 2, 128), 'gelu', 0.1, None),
+    ('mi355x', (2, 128, 2, 128), 'gelu', 0.0, None),
+    ('mi355x', (3, 384, 2, 128), 'gelu', 0.5, None),           # three blocks of 128 positions
+    ('mi355x', (2, 256, 2, 256), 'gelu', 0.1, None),           # head size 128
+    ('bert-b8-l512-h16-e1024', (2, 128, 2, 128), 'gelu', 0.1, None),   # the reference's layouts: falls back, still equal
+    ('mi355x:bert-b96-l128-h16-e1024', (16, 128, 16, 1024), 'gelu', 0.1, None),
+    ('mi355x', (8, 512, 16, 1024), 'gelu', 0.1, None),
+    ('mi355x', (2, 256, 2, 128), 'gelu', 0.1, 'JK'),           # causal mask plus finite entries
+    ('mi355x', (2, 256, 2, 256), 'gelu', 0.1, 'KJ'),           # the same, stored key-major
+    ('mi355x', (2, 128, 2, 128), 'gelu', 0.1, 'late'),         # first keys masked out for every query
 ])
-def test_attention_in_registers_matches_separate_operators(which, dims, act, p):
+def test_attention_in_registers_matches_separate_operators(which, dims, act, p, mask):
     """The attention kernels that keep the scores in registers (default) against
     the separate operators (QKT, softmax, gamma and their backward counterparts):
-    same inputs, same dropout masks, outputs and all gradients within the parity
-    bound of each other (observed: 4e-3 at the bench size, where weight gradients
-    sum 4096 fp16-rounded terms).  A wrong mask bit, a transposed tile or a wrong
-    log-sum-exp would be an error of order one.  GELU throughout: with ReLU, a
-    pre-activation that rounds to the other side of zero flips whole gradient
-    elements, which says nothing about the attention kernels."""
-    from substation_amd import Encoder
+    same inputs, same dropout masks, same additive attention mask if any, outputs
+    and all gradients within the parity bound of each other (observed: 4e-3 at
+    the bench size, where weight gradients sum 4096 fp16-rounded terms).  A wrong
+    mask bit, a transposed tile or a wrong log-sum-exp would be an error of order
+    one.  GELU throughout: with ReLU, a pre-activation that rounds to the other
+    side of zero flips whole gradient elements, which says nothing about the
+    attention kernels."""
+    from substation_amd import Encoder, causal_mask
     lay = _layouts(which)
     B, L, H, E = dims
+    am, am_layout = None, 'JK'
+    if mask is not None:
+        g = torch.Generator().manual_seed(11)
+        am = causal_mask(L, 'cpu', torch.float32) + 2.0 * torch.randn(L, L, generator=g)
+        if mask == 'late':      # no query sees the first 40 keys: the running softmax starts without a reference
+            am = 2.0 * torch.randn(L, L, generator=g)
+            am[:, :40] = float('-inf')
+        elif mask == 'KJ':
+            am, am_layout = am.t().contiguous(), 'KJ'
+        am = am.half().cuda()
     outs = []
     for fused in (0, 1):
         torch.manual_seed(0)
         enc = Encoder('unused', B, L, H, E, lay, torch.float16, p, 0.1, 0.1, 0.1, seed=SEED, activation=act).cuda()
         enc._handle.set_option(4, fused)
+        if am is not None:
+            enc.set_attention_mask(am, am_layout)
         enc.set_rng(SEED, 0)
         with torch.no_grad():
             for q in enc.parameters():
@@ -325,7 +341,7 @@ def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback()
     """compact_attention=True allocates token buffers for the score-sized tensors
     the in-register attention never touches and a few bytes per row for the two
     it keeps statistics and keep bits in: results are bit-identical, and anything
-    that would need the full tensors (here: an attention mask) is refused."""
+    that would need the full tensors is refused."""
     from substation_amd import Encoder, causal_mask, layouts as L
     from substation_amd._lib import SubstationError
     lay = L.mi355x_layouts()
@@ -352,11 +368,16 @@ def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback()
     for a, b in zip(*outs):
         assert torch.isfinite(a.float()).all()
         assert torch.equal(a, b)
-    enc.set_attention_mask(causal_mask(Ls, 'cuda', torch.float16))
+    # a mask that is not 8-byte aligned cannot take this path
+    storage = torch.zeros(Ls * Ls + 1, dtype=torch.float16, device='cuda')
+    enc.set_attention_mask(storage[1:].view(Ls, Ls))
     with pytest.raises(SubstationError, match='required'):
         enc(X)
-    enc.set_attention_mask(None)
+    enc.set_attention_mask(causal_mask(Ls, 'cuda', torch.float16))
     enc(X)
+    enc._handle.set_option(4, 0)             # switching the path off is noticed before anything is launched
+    with pytest.raises(RuntimeError, match='compact_attention'):
+        enc(X)
 
 
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
