@@ -4,7 +4,7 @@ from .layouts import load_layouts, mi355x_layouts, reference_layouts, save_layou
 
 
 def __getattr__(name):
-    if name in ('Encoder', 'causal_mask'):       # torch is imported only when the module is used
+    if name in ('Encoder', 'EncoderStack', 'causal_mask'):       # torch is imported only when the module is used
         from . import encoder
         return getattr(encoder, name)
     raise AttributeError(name)

@@ -5,9 +5,11 @@ naming/shapes (one ``nn.Parameter`` per ``layouts['params']`` entry, shaped in
 layout order), ``forward(X)`` and autograd backward returning ``(DX, *grads)``,
 ``debug`` capture.  Differences: nothing is compiled at construction (the
 library is prebuilt, ``compilation_dir`` is accepted and unused), kernels run on
-the caller's current stream, and three keyword-only extras exist: ``activation``
-('relu' as in the CUDA module, or 'gelu'), ``seed`` for the dropout masks and
-``intermediate_size`` (default ``4 * embedding_size``, encoder.py:33).
+the caller's current stream, and keyword-only extras exist: ``activation``
+('relu' as in the CUDA module, or 'gelu'), ``seed`` for the dropout masks,
+``intermediate_size`` (default ``4 * embedding_size``, encoder.py:33),
+``compact_attention``, ``persistent_workspace`` and ``canonical_state_dict``
+(see the constructor).  ``EncoderStack`` chains several layers.
 """
 import ctypes
 import math
@@ -33,7 +35,16 @@ class Encoder(torch.nn.Module):
                  softmax_dropout_probability, residual1_dropout_probability,
                  activation_dropout_probability, residual2_dropout_probability,
                  enable_debug=False, profiling=False, *, activation='relu', seed=0,
-                 intermediate_size=None, compact_attention=False):
+                 intermediate_size=None, compact_attention=False, persistent_workspace=False,
+                 canonical_state_dict=False):
+        """``persistent_workspace``: the intermediates are allocated once and reused
+        by every call instead of 37 ``torch.empty`` per iteration
+        (pytorch_module/encoder.py:78-85,113-119); a forward call then overwrites
+        what an earlier forward call saved for its backward pass, which backward()
+        detects and refuses.  ``canonical_state_dict``: ``state_dict()`` holds every
+        parameter in its canonical dimension order (``layouts.CANONICAL``) rather than
+        in this module's layout, so a checkpoint loads into a module built with any
+        other layouts."""
         super().__init__()
         if torch_dtype not in _SUPPORTED_DTYPES:
             raise NotImplementedError(
@@ -85,8 +96,8 @@ class Encoder(torch.nn.Module):
         # four of the six score-sized tensors ([H,B,J,K]) are never touched and the
         # other two only hold 8 resp. K/8 bytes per score row; allocate just that
         # (at B=8 L=512 H=16: 5 MiB instead of 384 MiB per layer call).  The path is
-        # then required: a later change that rules it out (an attention mask, option
-        # 4 = 0) makes forward() raise instead of writing through the small buffers.
+        # then required: a later change that rules it out (option 4 = 0, a misaligned
+        # tensor) makes forward() raise instead of writing through the small buffers.
         self.compact_attention = bool(compact_attention and not enable_debug
                                       and self._handle.attention_in_registers())
         if self.compact_attention:
@@ -96,6 +107,11 @@ class Encoder(torch.nn.Module):
         if self.compact_attention:
             compact = {'BETA': 8, 'ATTN_DROP': 8, 'DATTN_DROP': 8, 'DBETA': 8,
                        'ALPHA': rows * 4, 'ATTN_DROP_MASK': rows * max(max_seq_len // 16, 1)}
+        self.persistent_workspace = bool(persistent_workspace)
+        self.canonical_state_dict = bool(canonical_state_dict)
+        self._workspace = {}           # 'forward_interm' / 'backward_interm' -> tensors, when persistent
+        self._shared_backward = None   # set by EncoderStack: one backward workspace for all layers
+        self._generation = 0
         handle = self._handle
         lib = handle.lib
         module = self
@@ -113,6 +129,17 @@ class Encoder(torch.nn.Module):
                                 device=device, dtype=module.torch_dtype, requires_grad=False)
                     for name, layout in layouts[key]]
 
+        def _workspace(key, device):
+            if not module.persistent_workspace:
+                return _alloc(key, device)
+            if key == 'backward_interm' and module._shared_backward is not None:
+                store = module._shared_backward
+            else:
+                store = module._workspace
+            if key not in store or store[key][0].device != device:
+                store[key] = _alloc(key, device)
+            return store[key]
+
         class EncoderFunction(torch.autograd.Function):
             @staticmethod
             def forward(ctx, X, *weights):
@@ -128,7 +155,9 @@ class Encoder(torch.nn.Module):
                 X = X.contiguous()
                 # same element count as X, shaped in the output's own dimension order
                 Y = torch.empty(out_shape, device=dev, dtype=X.dtype)
-                forward_intermediate = _alloc('forward_interm', dev)
+                forward_intermediate = _workspace('forward_interm', dev)
+                module._generation += 1
+                ctx.generation = module._generation
                 weights_c = [t.contiguous() for t in weights]
                 handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)
                 ptrs = fwd_array(X.data_ptr(), *(t.data_ptr() for t in weights_c),
@@ -146,10 +175,13 @@ class Encoder(torch.nn.Module):
 
             @staticmethod
             def backward(ctx, DY):
+                if module.persistent_workspace and ctx.generation != module._generation:
+                    raise RuntimeError('persistent_workspace: forward() ran again before this backward pass; '
+                                       'what it had saved has been overwritten')
                 dev = DY.device
                 DY = DY.contiguous()
                 DX = torch.empty(in_shape, device=dev, dtype=DY.dtype)
-                backward_intermediate = _alloc('backward_interm', dev)
+                backward_intermediate = _workspace('backward_interm', dev)
                 param_gradients = _alloc('params', dev)
                 handle.set_stream(torch.cuda.current_stream(dev).cuda_stream)
                 ptrs = bwd_array(DY.data_ptr(), *(t.data_ptr() for t in param_gradients),
@@ -166,6 +198,31 @@ class Encoder(torch.nn.Module):
                 return (DX, *param_gradients)
 
         self.encoder_func = EncoderFunction
+
+    def _canonical_perm(self, name, layout):
+        canon = _lay.CANONICAL[name]
+        return [layout.index(d) for d in canon]
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if not self.canonical_state_dict:
+            return
+        for name, layout in self.layouts['params']:
+            t = destination[prefix + name]
+            destination[prefix + name] = t.detach().permute(self._canonical_perm(name, layout)).contiguous()
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys,
+                              unexpected_keys, error_msgs):
+        if self.canonical_state_dict:
+            for name, layout in self.layouts['params']:
+                key = prefix + name
+                if key in state_dict:
+                    canon = _lay.CANONICAL[name]
+                    t = state_dict[key]
+                    if t.dim() == len(canon):
+                        state_dict[key] = t.permute([canon.index(d) for d in layout]).contiguous()
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys,
+                                      unexpected_keys, error_msgs)
 
     def reset_parameters(self):
         """U(-1/sqrt(2), 1/sqrt(2)) for every parameter, pytorch_module/encoder.py:144-158."""
@@ -227,3 +284,64 @@ class Encoder(torch.nn.Module):
         """Run the encoder.  X is in ``layouts['input'][1]`` order; the result is
         in ``layouts['output'][1]`` order."""
         return self.encoder_func.apply(X, *self.params)
+
+
+class EncoderStack(torch.nn.Module):
+    """``num_layers`` encoder layers applied one after the other.
+
+    What chaining needs beyond the single layer of pytorch_module/encoder.py: the
+    output layout must equal the input layout (config_selection/ops.py:265-270
+    ties them for this reason; checked here), every layer draws its dropout masks
+    from its own stream (seed + layer index), the forward intermediates of each
+    layer are allocated once and reused by every iteration, all layers share one
+    set of backward intermediates (only one layer's backward pass is running at a
+    time), and ``state_dict()`` is in canonical dimension order so that a
+    checkpoint does not depend on the layouts the stack was built with."""
+
+    def __init__(self, num_layers, batch_size, max_seq_len, num_heads, embedding_size, layouts, torch_dtype,
+                 softmax_dropout_probability, residual1_dropout_probability,
+                 activation_dropout_probability, residual2_dropout_probability, *, activation='relu', seed=0,
+                 intermediate_size=None, compact_attention=True, persistent_workspace=True,
+                 canonical_state_dict=True, profiling=False):
+        super().__init__()
+        if layouts['input'][1] != layouts['output'][1]:
+            raise ValueError(f"layers stack only when the output layout ({layouts['output'][1]}) equals the "
+                             f"input layout ({layouts['input'][1]})")
+        self.num_layers = num_layers
+        self.layers = torch.nn.ModuleList([
+            Encoder('unused', batch_size, max_seq_len, num_heads, embedding_size, layouts, torch_dtype,
+                    softmax_dropout_probability, residual1_dropout_probability,
+                    activation_dropout_probability, residual2_dropout_probability, profiling=profiling,
+                    activation=activation, seed=seed + i, intermediate_size=intermediate_size,
+                    compact_attention=compact_attention, persistent_workspace=persistent_workspace,
+                    canonical_state_dict=canonical_state_dict)
+            for i in range(num_layers)])
+        shared = {}
+        for layer in self.layers:
+            layer._shared_backward = shared
+
+    def forward(self, X):
+        for layer in self.layers:
+            X = layer(X)
+        return X
+
+    def set_rng(self, seed, step=0):
+        """Layer i draws from the stream of ``seed + i``."""
+        for i, layer in enumerate(self.layers):
+            layer.set_rng(seed + i, step)
+
+    def set_attention_mask(self, mask, layout='JK'):
+        for layer in self.layers:
+            layer.set_attention_mask(mask, layout)
+
+    def workspace_bytes(self):
+        """Device bytes held by the persistent workspaces (0 before the first call)."""
+        seen, total = set(), 0
+        stores = [layer._workspace for layer in self.layers]
+        stores += [layer._shared_backward for layer in self.layers if layer._shared_backward is not None]
+        for store in stores:
+            if id(store) in seen:
+                continue
+            seen.add(id(store))
+            total += sum(t.numel() * t.element_size() for ts in store.values() for t in ts)
+        return total
