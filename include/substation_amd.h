@@ -195,6 +195,28 @@ int sub_profile_read(void* handle, int cap, const char** names, float* ms);
 /* Sizes come from the handle's configuration; every tensor takes its own layout
  * string.  Vectors of parameters ([I], [U]) are dense. */
 
+/* Scaled-dot-product attention with the scores kept in registers, forward and
+ * backward (the chain encoder.cu:104-131 and :222-262 as one operator; with
+ * n_keys != n_queries the encoder-decoder attention of
+ * substation/transformer.py:288-441, attention.py:31-179).  q, out, d_out, dq:
+ * layouts over B, J, H, P; k, v, dk, dv: over B, K, H, P (P innermost; B, H, P from
+ * the handle; n_queries, n_keys multiples of 128; head size 64 or 128).
+ * out = dropout(softmax(scale * (q.k^T + attn_mask))) . v, keep mask drawn for
+ * (site, the handle's seed and step) over the canonical [H,B,J,K] element index.
+ * stats: 2*H*B*n_queries floats, keep: H*B*n_queries*n_keys/8 bytes (both 16-byte
+ * aligned), written by the forward call and read by the backward call, which
+ * also needs the forward call's out.  attn_mask may be null.  These calls fail
+ * (nothing is launched) when the sizes, layouts or alignment are not supported. */
+int sub_op_attention_forward(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                             const void* k, const void* v, const char* l_kv, void* out, const char* l_out,
+                             void* stats, void* keep, const void* attn_mask, const char* l_attn_mask,
+                             float scale, float p, uint32_t site);
+int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                              const void* k, const void* v, const char* l_kv, const void* out,
+                              const char* l_out, const void* d_out, const char* l_dout, void* stats,
+                              const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
+                              const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale);
+
 /* block_softmax.cuh:127-188; `scale` multiplies the input (1 in the layer, where
  * the factor is the GEMM's alpha, encoder.cu:116). */
 int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alpha,

@@ -64,6 +64,10 @@ SIGNATURES = {
     'sub_op_softmax': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _U32]),
     'sub_op_softmax_masked': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _F, _U32]),
     'sub_set_attention_mask': (_I, [_VP, _VP, _CP]),
+    'sub_op_attention_forward': (_I, [_VP, _I, _I, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _CP,
+                                      _F, _F, _U32]),
+    'sub_op_attention_backward': (_I, [_VP, _I, _I, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP,
+                                       _VP, _CP, _VP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_bs': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_bdrln': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP, _CP, _VP, _CP, _VP, _CP,
                           _VP, _CP, _VP, _CP, _VP, _CP, _F, _U32]),

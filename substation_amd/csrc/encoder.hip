@@ -1101,6 +1101,66 @@ int sub_op_softmax_masked(void* handle, const void* beta, const char* l_beta, vo
     });
 }
 
+namespace {
+// Operands of the attention operators: layouts over (B, J or K, H, P) with the
+// numbers of query and key positions given per call (they differ in
+// encoder-decoder attention, substation/transformer.py:288-441).
+void op_attention_args(Handle& h, int n_queries, int n_keys, const void* q, const char* l_q, const void* k,
+                       const void* v, const char* l_kv, const void* out, const char* l_out, void* stats,
+                       void* keep, const void* attn_mask, const char* l_attn_mask, float scale, AttnArgs& a) {
+    if (n_queries <= 0 || n_keys <= 0) fail("attention: numbers of query and key positions must be positive");
+    Sizes z = h.sz;
+    z.n[dJ] = n_queries; z.n[dK] = n_keys;
+    const Layout lq = make_layout(l_q, z), lkv = make_layout(l_kv, z), lo = make_layout(l_out, z);
+    if (!attn_side(q, lq, dJ, a.q) || !attn_side(k, lkv, dK, a.k) || !attn_side(v, lkv, dK, a.v) ||
+        !attn_side(out, lo, dJ, a.o))
+        fail("attention: q and out take a layout over B, J, H, P and k, v one over B, K, H, P, P innermost");
+    a.H = (int)z.n[dH]; a.B = (int)z.n[dB]; a.J = n_queries; a.K = n_keys;
+    a.alpha = scale;
+    a.lse = (float*)stats; a.dsum = a.lse + (size_t)a.H * a.B * a.J;
+    a.keep = (uint32_t*)keep;
+    if (attn_mask) {
+        const Layout lm = make_layout(l_attn_mask, z);
+        if (lm.rank != 2 || !lm.has[dJ] || !lm.has[dK]) fail("attention: the mask layout must be JK or KJ");
+        a.amask = (const half_t*)attn_mask; a.am_sj = lm.stride[dJ]; a.am_sk = lm.stride[dK];
+    }
+}
+}  // namespace
+
+int sub_op_attention_forward(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                             const void* k, const void* v, const char* l_kv, void* out, const char* l_out,
+                             void* stats, void* keep, const void* attn_mask, const char* l_attn_mask,
+                             float scale, float p, uint32_t site) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        AttnArgs a;
+        op_attention_args(h, n_queries, n_keys, q, l_q, k, v, l_kv, out, l_out, stats, keep, attn_mask,
+                          l_attn_mask, scale, a);
+        launch_mha_forward(a, (int)h.sz.n[dP], make_key(h, site, p), h.stream);
+    });
+}
+
+int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                              const void* k, const void* v, const char* l_kv, const void* out,
+                              const char* l_out, const void* d_out, const char* l_dout, void* stats,
+                              const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
+                              const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        AttnArgs a;
+        op_attention_args(h, n_queries, n_keys, q, l_q, k, v, l_kv, out, l_out, stats, const_cast<void*>(keep),
+                          attn_mask, l_attn_mask, scale, a);
+        Sizes z = h.sz;
+        z.n[dJ] = n_queries; z.n[dK] = n_keys;
+        if (!attn_side(d_out, make_layout(l_dout, z), dJ, a.d_o) || !attn_side(dq, make_layout(l_dq, z), dJ, a.dq) ||
+            !attn_side(dk, make_layout(l_dkv, z), dK, a.dk) || !attn_side(dv, make_layout(l_dkv, z), dK, a.dv))
+            fail("attention backward: d_out and dq take a layout over B, J, H, P and dk, dv one over B, K, H, P, "
+                 "P innermost");
+        launch_mha_backward_dq(a, (int)h.sz.n[dP], h.stream);
+        launch_mha_backward_dkv(a, (int)h.sz.n[dP], h.stream);
+    });
+}
+
 int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layout) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);

@@ -59,6 +59,30 @@ class Ops:
                                            _p(mask), _s(l_mask), _p(drop), _s(l_drop), scale, p, site),
                    'softmax')
 
+    def attention_workspace(self, n_queries, n_keys, device='cuda'):
+        """(stats, keep): what attention_forward hands to attention_backward."""
+        rows = self.sizes['H'] * self.sizes['B'] * n_queries
+        return (torch.empty(2 * rows, dtype=torch.float32, device=device),
+                torch.empty(rows * (n_keys // 32), dtype=torch.int32, device=device))
+
+    def attention_forward(self, q, l_q, k, v, l_kv, out, l_out, stats, keep, scale, p=0.0, site=0,
+                          attn_mask=None, l_attn_mask='JK'):
+        """out = dropout(softmax(scale * (q.k^T + attn_mask))) . v with the scores in
+        registers; the numbers of query and key positions are read off the tensors."""
+        nq, nk = q.shape[l_q.index('J')], k.shape[l_kv.index('K')]
+        _lib.check(self.lib.sub_op_attention_forward(
+            self._pre(), nq, nk, _p(q), _s(l_q), _p(k), _p(v), _s(l_kv), _p(out), _s(l_out),
+            ctypes.c_void_p(stats.data_ptr()), ctypes.c_void_p(keep.data_ptr()), _p(attn_mask), _s(l_attn_mask),
+            scale, p, site), 'attention_forward')
+
+    def attention_backward(self, q, l_q, k, v, l_kv, out, l_out, d_out, l_dout, stats, keep, dq, l_dq, dk, dv,
+                           l_dkv, scale, attn_mask=None, l_attn_mask='JK'):
+        nq, nk = q.shape[l_q.index('J')], k.shape[l_kv.index('K')]
+        _lib.check(self.lib.sub_op_attention_backward(
+            self._pre(), nq, nk, _p(q), _s(l_q), _p(k), _p(v), _s(l_kv), _p(out), _s(l_out), _p(d_out),
+            _s(l_dout), ctypes.c_void_p(stats.data_ptr()), ctypes.c_void_p(keep.data_ptr()), _p(dq), _s(l_dq),
+            _p(dk), _p(dv), _s(l_dkv), _p(attn_mask), _s(l_attn_mask), scale), 'attention_backward')
+
     def bs(self, alpha, l_alpha, mask, l_mask, ddrop, l_ddrop, dbeta, l_dbeta, scale=1.0):
         _lib.check(self.lib.sub_op_bs(self._pre(), _p(alpha), _s(l_alpha), _p(mask), _s(l_mask),
                                       _p(ddrop), _s(l_ddrop), _p(dbeta), _s(l_dbeta), scale), 'bs')

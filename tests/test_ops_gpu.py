@@ -237,3 +237,68 @@ def test_aib_baib(B, L, H, E):
         torch.cuda.synchronize()
         assert_close(from_layout(out, 'QPHBJ', lout), ref.op_aib(w, bias), name='KKQQVV ' + lin)
         assert_close(from_layout(db, 'QPH', lb), ref.op_baib(w), name='DBKQV ' + lin, tol=2e-2)
+
+
+@pytest.mark.parametrize('B,H,P,J,K,p,masked,l_q,l_kv', [
+    (2, 2, 64, 128, 128, 0.1, False, 'BJHP', 'BKHP'),
+    (2, 2, 64, 128, 384, 0.1, False, 'BJHP', 'BKHP'),      # more keys than queries (encoder-decoder attention)
+    (1, 3, 64, 256, 128, 0.0, False, 'BHJP', 'BHKP'),      # fewer keys than queries, head-major rows
+    (2, 2, 128, 128, 256, 0.25, True, 'JBHP', 'KBHP'),     # head size 128, additive mask, position-major rows
+    (8, 16, 64, 512, 512, 0.1, False, 'BJHP', 'BKHP'),     # the bench workload's attention
+])
+def test_attention_operator_forward_and_backward(B, H, P, J, K, p, masked, l_q, l_kv):
+    """The attention kernels as one operator against the closed form
+    (substation/attention.py:31-179 restated for one head: softmax over the keys of
+    scale*(q.k^T + mask), {0,1} dropout mask without rescale, weighted sum of v,
+    and its gradients), in float64 on the fp16-rounded inputs.  The keep bits are
+    compared exactly with the oracle's Philox stream over the [H,B,J,K] index."""
+    o = _ops(B, 128, H, H * P)
+    o.set_rng(SEED, 2)
+    rng = np.random.default_rng(J * 7 + K)
+    q = h16(rng.standard_normal((B, J, H, P)))
+    k = h16(rng.standard_normal((B, K, H, P)))
+    v = h16(rng.standard_normal((B, K, H, P)))
+    d_out = h16(rng.standard_normal((B, J, H, P)))
+    scale = 1.0 / np.sqrt(P)
+    am = None
+    if masked:
+        am = h16(rng.standard_normal((J, K)))
+        am[np.triu_indices(J, 1, K)] = -np.inf
+        am[:, 0] = 0.0                                       # no row is masked out entirely
+    tq, tk, tv = to_layout(q, 'BJHP', l_q), to_layout(k, 'BKHP', l_kv), to_layout(v, 'BKHP', l_kv)
+    tdo = to_layout(d_out, 'BJHP', l_q)
+    out, dq = torch.empty_like(tq), torch.empty_like(tq)
+    dk, dv = torch.empty_like(tk), torch.empty_like(tk)
+    stats, keep = o.attention_workspace(J, K)
+    tam = None if am is None else torch.from_numpy(am).half().cuda()
+    o.attention_forward(tq, l_q, tk, tv, l_kv, out, l_q, stats, keep, scale, p=p, site=ph.SITE_SOFTMAX, attn_mask=tam)
+    o.attention_backward(tq, l_q, tk, tv, l_kv, out, l_q, tdo, l_q, stats, keep, dq, l_q, dk, dv, l_kv, scale,
+                         attn_mask=tam)
+    torch.cuda.synchronize()
+
+    mask = ph.dropout_mask((H, B, J, K), p, SEED, ph.SITE_SOFTMAX, step=2, dtype=np.float64)
+    words = keep.cpu().numpy().view(np.uint32).reshape(H, B, J, K // 32)
+    bits = ((words[..., None] >> np.arange(32, dtype=np.uint32)) & 1).reshape(H, B, J, K)
+    assert np.array_equal(bits, mask.astype(np.uint32))
+
+    s = np.einsum('bjhp,bkhp->hbjk', q, k)
+    if am is not None:
+        s = s + am
+    s = s * scale
+    e = np.exp(s - s.max(-1, keepdims=True))
+    alpha = e / e.sum(-1, keepdims=True)
+    drop = alpha * mask
+    want_out = np.einsum('hbjk,bkhp->bjhp', drop, v)
+    d_drop = np.einsum('bjhp,bkhp->hbjk', d_out, v)
+    d_alpha = d_drop * mask
+    d_s = alpha * (d_alpha - (alpha * d_alpha).sum(-1, keepdims=True))
+    want_dq = scale * np.einsum('hbjk,bkhp->bjhp', d_s, k)
+    want_dk = scale * np.einsum('hbjk,bjhp->bkhp', d_s, q)
+    want_dv = np.einsum('hbjk,bjhp->bkhp', drop, d_out)
+    lse = stats.cpu().numpy()[:H * B * J].reshape(H, B, J)
+    want_lse = (s.max(-1) + np.log(e.sum(-1))) / np.log(2.0)
+    assert_close(lse, want_lse, tol=1e-3, name='log-sum-exp')
+    assert_close(from_layout(out, 'BJHP', l_q), want_out, name='out')
+    assert_close(from_layout(dq, 'BJHP', l_q), want_dq, name='dq')
+    assert_close(from_layout(dk, 'BKHP', l_kv), want_dk, name='dk')
+    assert_close(from_layout(dv, 'BKHP', l_kv), want_dv, name='dv')
