@@ -245,6 +245,7 @@ def test_aib_baib(B, L, H, E):
     (1, 3, 64, 256, 128, 0.0, False, 'BHJP', 'BHKP'),      # fewer keys than queries, head-major rows
     (2, 2, 128, 128, 256, 0.25, True, 'JBHP', 'KBHP'),     # head size 128, additive mask, position-major rows
     (8, 16, 64, 512, 512, 0.1, False, 'BJHP', 'BKHP'),     # the bench workload's attention
+    (1, 2, 128, 2048, 2048, 0.1, True, 'BJHP', 'BKHP'),    # 64 key tiles, head size 128 (the wide workload's shape per head)
 ])
 def test_attention_operator_forward_and_backward(B, H, P, J, K, p, masked, l_q, l_kv):
     """The attention kernels as one operator against the closed form
