@@ -377,12 +377,15 @@ void configure(Handle& h, const sub_config* c) {
         size_t baib = colreduce_ws_floats(sq.rs, 1), baib2 = colreduce_ws_floats(merged, 1);
         h.ws_need_bwd = colreduce_ws_floats(si.rs, 2) + colreduce_ws_floats(si.rs, 3) +
                         colreduce_ws_floats(su.rs, 1) + colreduce_ws_floats(si.rs, 1) +
-                        (baib > baib2 ? baib : baib2) + 6 * 64;
+                        (baib > baib2 ? baib : baib2) + 8 * 64;
         // the fused LayerNorm-backward launches replace four of those reductions;
         // size for whichever set is larger
         size_t fused = lnbwd_ws_floats(si.rs, false) + lnbwd_ws_floats(si.rs, true) +
-                       colreduce_ws_floats(su.rs, 1) + (baib > baib2 ? baib : baib2) + 6 * 64;
+                       colreduce_ws_floats(su.rs, 1) + (baib > baib2 ? baib : baib2) + 8 * 64;
         if (fused > h.ws_need_bwd) h.ws_need_bwd = fused;
+        // the attention kernels' partial sums for the projection-bias gradient stand in for baib's
+        const size_t attn_bias = (size_t)(3 * sz.n[dH] * sz.n[dB] * ((sz.n[dJ] + 127) / 128) * sz.n[dP]);
+        if (attn_bias > (baib > baib2 ? baib : baib2)) h.ws_need_bwd += attn_bias;
     }
     h.gws_need = 0;
     for (int i = 0; i < G_COUNT; ++i) {
@@ -840,16 +843,39 @@ void backward(Handle& h, const BwdPtrs& t) {
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
     AttnArgs at;
+    bool attn_bias = false;
     if (attention_fused(h, F, at)) {
         if (!attn_side(D[DGAMMA], h.lb[DGAMMA], dJ, at.d_o) || !attn_side(DQQ, h.lDQQ, dJ, at.dq) ||
             !attn_side(DKK, h.lDKK, dK, at.dk) || !attn_side(DVV, h.lDKK, dK, at.dv))
             fail("encoder_backward: attention layouts changed since the forward pass");
+        // the sums over (sample, position) of dQ, dK, dV -- the gradient of the projection
+        // biases (BackwardAttentionInputBiases, encoder.cu:288-290) -- start in these launches
+        const Layout& lbias = h.lp[BKQV];
+        attn_bias = lbias.has[dQ] && lbias.has[dH] && lbias.has[dP];
+        const int P = (int)h.sz.n[dP], H = (int)h.sz.n[dH];
+        const int ntq = at.B * (at.J / 128), ntk = at.B * (at.K / 128);
+        half_t* dbias = (half_t*)DW[BKQV];
+        auto finish = [&](float* ws, int ns, int ntc, half_t* o0, half_t* o1) {
+            FinishJob job{ws, FinishArgs{{o0, o1, nullptr, nullptr}, 0, lbias.stride[dH], lbias.stride[dP], H}, ns, H,
+                          ntc, P};
+            if (h.deferring) {
+                if (h.deferred.n >= kMaxFinishJobs) fail("encoder_backward: too many deferred reductions");
+                h.deferred.j[h.deferred.n++] = job;
+            } else {
+                FinishJobs one; one.n = 1; one.j[0] = job;
+                launch_colfinish(one, h.stream);
+            }
+        };
         {
             ProfScope ps(h, "attention-bwd-dQ");
-            launch_mha_backward_dq(at, (int)h.sz.n[dP], h.stream);
+            if (attn_bias) at.bias_q = take_ws(h, (size_t)H * ntq * P);
+            launch_mha_backward_dq(at, P, h.stream);
+            if (attn_bias) finish(at.bias_q, 1, ntq, dbias + 1 * lbias.stride[dQ], nullptr);
         }
         ProfScope ps(h, "attention-bwd-dKdV");
-        launch_mha_backward_dkv(at, (int)h.sz.n[dP], h.stream);
+        if (attn_bias) at.bias_kv = take_ws(h, (size_t)2 * H * ntk * P);
+        launch_mha_backward_dkv(at, P, h.stream);
+        if (attn_bias) finish(at.bias_kv, 2, ntk, dbias, dbias + 2 * lbias.stride[dQ]);
     } else {
         run_gemm(h, G_DX2GAMMA, D[DGAMMA], F[ATTN_DROP], DVV, "dX2gamma");
         bool fused_scores = false;
@@ -877,7 +903,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         run_gemm(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused");
     }
     run_gemm(h, G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused");
-    {
+    if (!attn_bias) {
         ProfScope ps(h, "baib");
         op_baib(h, D[DKKQQVV], h.lb[DKKQQVV], DW[BKQV], h.lp[BKQV]);
     }

@@ -170,6 +170,24 @@ __device__ __forceinline__ float keep_if(float x, uint32_t bits, int pos) {
     return __int_as_float(__float_as_int(x) & __builtin_amdgcn_sbfe((int)bits, pos, 1));
 }
 
+// Sums over the 128 positions of a workgroup of the rows store_rows() writes
+// (same rounding), one value per feature: 32 lanes hold the positions of a
+// wave, the four waves meet in LDS (`red`: 4 * P floats, free to use).
+template <int P>
+__device__ __forceinline__ void column_sums(const f16v (&acc)[P / 32], float scale, float* red, float* out,
+                                            int tid) {
+    const int lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
+#pragma unroll
+    for (int pt = 0; pt < P / 32; ++pt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const float x = group_sum<32>((float)(half_t)(acc[pt][v] * scale));
+            if (l32 == 0) red[wave * P + pt * 32 + reg_pos(v, hi)] = x;
+        }
+    __syncthreads();
+    if (tid < P) out[tid] = (red[tid] + red[P + tid]) + (red[2 * P + tid] + red[3 * P + tid]);
+}
+
 __device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
     uint32_t b = 0;
 #pragma unroll
@@ -450,6 +468,9 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         const int x = cur; cur = nxt; nxt = nn; nn = x;
     }
     store_rows<P>(a.dq, h, b, j, hi, dq, a.alpha);
+    if (a.bias_q)
+        column_sums<P>(dq, a.alpha, reinterpret_cast<float*>(&kt[0][0]),
+                       a.bias_q + ((size_t)h * (a.B * qblocks) + b * qblocks + qb) * P, tid);
 }
 
 // ---------------------------------------------------------------------------
@@ -581,6 +602,12 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
     }
     store_rows<P>(a.dk, h, b, kpos, hi, dk, a.alpha);
     store_rows<P>(a.dv, h, b, kpos, hi, dv, 1.0f);
+    if (a.bias_kv) {
+        const size_t ntc = (size_t)a.B * kblocks, part = (size_t)h * ntc + b * kblocks + kb;
+        float* red = reinterpret_cast<float*>(&stage[0]);
+        column_sums<P>(dk, a.alpha, red, a.bias_kv + part * P, tid);
+        column_sums<P>(dv, 1.0f, red + 4 * P, a.bias_kv + ((size_t)a.H * ntc + part) * P, tid);
+    }
 }
 
 // 8-byte loads of four mask values along whichever dim is contiguous

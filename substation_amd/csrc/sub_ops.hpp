@@ -122,6 +122,11 @@ struct AttnArgs {
     uint32_t* keep = nullptr;  // [H*B*J][K/32]  keep bits of the softmax dropout, bit k%32 of word k/32
     int H = 0, B = 0, J = 0, K = 0;
     float alpha = 1.f;         // score scale
+    // optional (backward): per-workgroup sums over positions of the rounded dq resp.
+    // dk, dv rows, for the gradient of the projection biases.  bias_q: [H][B*J/128][P]
+    // floats, bias_kv: [2][H][B*K/128][P] (dk, then dv).
+    float* bias_q = nullptr;
+    float* bias_kv = nullptr;
     const half_t* amask = nullptr;   // optional additive mask over (query, key), added before the scaling
     long am_sj = 0, am_sk = 0;
 };
