@@ -68,7 +68,8 @@ ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused', 'bei'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
-    ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT'),
+    ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT',
+     'baib'),
     ('bsb+blnrd1', 'bsb', 'blnrd1'),
     ('ebsb+blnrd2+baob', 'ebsb', 'blnrd2', 'baob'),
 ]
