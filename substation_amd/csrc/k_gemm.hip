@@ -769,6 +769,7 @@ void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, bool dma, hi
 }
 
 constexpr size_t kSplitMaxOut = 2u << 20;     // largest output (elements) whose contraction is split
+constexpr long kSplitTarget = 256;            // workgroups a split product aims for (the CUs of the device)
 
 // How many ways to split k so that a small output still fills the chip: the
 // weight-gradient products have few output tiles and a long contraction.
@@ -776,7 +777,8 @@ int pick_splits(const GemmArgs& a, long batch, size_t ws_floats) {
     static const int force = [] { const char* e = getenv("SUB_GEMM_SPLITK"); return e ? atoi(e) : 0; }();
     const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
     const int nkt = a.K0 * ((a.K1 + BK - 1) / BK);
-    int splits = force > 0 ? force : (int)((384 + tiles - 1) / tiles);
+    // one workgroup per CU: a second, partly filled round costs more than it gains
+    int splits = force > 0 ? force : (int)(kSplitTarget / tiles);
     if (force < 0) splits = 1;
     if (splits > 8) splits = 8;
     while (splits > 1 && nkt / splits < 8) --splits;
@@ -800,8 +802,8 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
     // traffic costs more than the extra workgroups gain)
     size_t per = (size_t)s.batch() * s.M * s.N;
     long tiles = ((s.M + 127) / 128) * ((s.N + 127) / 128) * s.batch();
-    if (tiles >= 384 || per > kSplitMaxOut) return 0;
-    size_t splits = (384 + tiles - 1) / tiles;
+    if (tiles > kSplitTarget / 2 || per > kSplitMaxOut) return 0;
+    size_t splits = kSplitTarget / tiles;
     if (splits > 8) splits = 8;
     return per * splits;
 }
