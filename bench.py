@@ -38,12 +38,12 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 88458689, 'attention': 38113369, 'out': 33775290, 'bdrln1': 59014038,
-    'lin1': 84251664, 'bad': 134454950, 'lin2': 109264818, 'bdrln2': 59011094,
-    'bsb+blnrd1': 61022393, 'dXlin2': 84238426, 'dWlin2': 109275276, 'bdrlb': 135394527,
-    'dXlin1': 109260448, 'dWlin1': 109274947, 'ebsb+blnrd2+baob': 79939868, 'dWout': 101803120,
-    'dXout': 33771067, 'attention-bwd-dQ': 55131503, 'attention-bwd-dKdV': 55150951,
-    'dXQKV-fused': 92484993, 'dWQKV-fused': 115565358, 'baib': 25997151,
+    'QKV-fused': 88458973, 'attention': 38113622, 'out': 33775361, 'bdrln1': 59015091,
+    'lin1': 84251804, 'bad': 134460163, 'lin2': 109265042, 'bdrln2': 59013701,
+    'bsb+blnrd1': 61022706, 'dXlin2': 84238493, 'dWlin2': 109275573, 'bdrlb': 135394861,
+    'dXlin1': 109260727, 'dWlin1': 109275061, 'ebsb+blnrd2+baob': 79940136, 'dWout': 92477161,
+    'dXout': 33771119, 'attention-bwd-dQ': 55316257, 'attention-bwd-dKdV': 55519010,
+    'dXQKV-fused': 92485226, 'dWQKV-fused': 115565660,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
