@@ -96,6 +96,78 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
     return want, got
 
 
+def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=None, compact=False):
+    """The module as a user gets it (no debug capture: every fusion on, attention
+    with the scores in registers where the sizes allow) against the oracle, which
+    draws the four dropout masks itself from the same seeded Philox streams.
+    GELU, so that no gradient hinges on the sign of a rounded pre-activation.
+    Returns (oracle dict, device dict) with the output, DX and the 12 gradients."""
+    from substation_amd import Encoder, layouts as Lm
+    lay = Lm.mi355x_layouts()
+    enc = Encoder('unused', B, L, H, E, lay, torch.float16, p, p, p, p, activation='gelu', seed=SEED,
+                  compact_attention=compact).cuda()
+    enc.set_rng(SEED, step)
+    if attn_mask is not None:
+        enc.set_attention_mask(torch.from_numpy(attn_mask).half().cuda())
+    sz = enc.sizes
+    rng = np.random.default_rng(seed_data)
+    params_np = {}
+    for name, _ in lay['params']:
+        canon = ref.CANONICAL[name]
+        shape = tuple(sz[d] for d in canon)
+        if name in ('S1', 'S2'):
+            v = 1 + 0.1 * rng.normal(size=shape)
+        elif len(canon) == 1 or name == 'BKQV':
+            v = 0.1 * rng.normal(size=shape)
+        else:
+            v = w_std * rng.normal(size=shape)
+        params_np[name] = h16(v)
+    X_np = h16(rng.normal(size=(B, L, E)))
+    DY_np = h16(rng.normal(size=(B, L, E)))
+    with torch.no_grad():
+        for name, layout in lay['params']:
+            canon = ref.CANONICAL[name]
+            getattr(enc, name).copy_(torch.from_numpy(
+                np.transpose(params_np[name], [canon.index(d) for d in layout]).copy()).half())
+    X = torch.from_numpy(X_np).half().cuda().requires_grad_(True)
+    Y = enc(X)
+    Y.backward(torch.from_numpy(DY_np).half().cuda())
+    torch.cuda.synchronize()
+    got = {'SB2': Y.detach().float().cpu().numpy().astype(np.float64),
+           'DX': X.grad.float().cpu().numpy().astype(np.float64)}
+    for name, layout in lay['params']:
+        canon = ref.CANONICAL[name]
+        got['D' + name] = from_layout(getattr(enc, name).grad, canon, layout)
+    U = sz['U']
+    masks = {name: ph.dropout_mask(shape, p, SEED, site, step=step, dtype=np.float64)
+             for name, shape, site in (('ATTN_DROP_MASK', (H, B, L, L), 0), ('DROP1MASK', (B, L, E), 1),
+                                       ('DROP2MASK', (B, L, U), 2), ('DROP3MASK', (B, L, E), 3))}
+    want = ref.run_named(params_np, X_np, DY_np, masks, 'gelu', attn_mask=attn_mask)
+    return want, got
+
+
+OUTPUTS = ['SB2', 'DX', 'DWKQV', 'DBKQV', 'DWO', 'DBO', 'DS1', 'DB1', 'DLINB1', 'DLINW1', 'DS2', 'DB2',
+           'DLINB2', 'DLINW2']
+
+
+@pytest.mark.parametrize('dims,p,masked,compact', [
+    ((2, 128, 2, 128), 0.1, False, False),
+    ((2, 256, 4, 256), 0.1, False, True),
+    ((1, 256, 2, 256), 0.2, True, False),         # head size 128, causal mask
+    ((4, 512, 4, 256), 0.1, False, False),
+])
+def test_default_path_matches_the_oracle(dims, p, masked, compact):
+    """Output, DX and the 12 gradients of the layer as shipped -- attention with the
+    scores in registers, the keep bits never materialised as a mask tensor --
+    against the NumPy oracle fed the masks of oracle/philox_ref.py."""
+    B, L, H, E = dims
+    am = None
+    if masked:
+        am = np.triu(np.full((L, L), -np.inf), 1)
+    want, got = run_layer_default(B, L, H, E, p, seed_data=L + H, attn_mask=am, compact=compact)
+    _compare(want, got, names=OUTPUTS)
+
+
 CHECK = ['KKQQVV', 'WKKWQQWVV', 'BETA', 'ALPHA', 'ATTN_DROP', 'GAMMA', 'ATT', 'SB1', 'SB1_LINW1',
          'LIN1', 'DROP2', 'DROP2_LINW2', 'LIN2', 'LN1', 'LN1STD', 'LN1DIFF', 'LN2', 'LN2STD', 'LN2DIFF',
          'SB2', 'DLN2', 'DRESID2', 'DLIN2', 'DDROP2', 'DLIN1', 'DLIN1_LINW1', 'DLN1', 'DRESID1', 'DATT',
