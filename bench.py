@@ -85,6 +85,9 @@ def algorithmic_work(B, L, H, E):
     w['attention'] = ('mfma', 2 * attn[0], 2 * 4 * bji + hbjk // 8)
     w['attention-bwd-dQ'] = ('mfma', 3 * attn[0], 2 * 6 * bji + hbjk // 8)
     w['attention-bwd-dKdV'] = ('mfma', 4 * attn[0], 2 * 6 * bji + hbjk // 8)
+    # two products in one launch
+    w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
+    w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

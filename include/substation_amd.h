@@ -173,6 +173,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * row behind ATTN_DROP_MASK (both 16-byte aligned). */
 #define SUB_OPT_FUSE_ATTENTION 4
 #define SUB_FUSE_REQUIRED 2
+/* SUB_OPT_PAIR_PRODUCTS (default 1): in encoder_backward a data-gradient product
+ * and the weight-gradient product next to it (encoder.cu:205-216 DLIN1_LINW1 and
+ * DLINW1; :262-276 DXATT and DWKQV), which do not depend on one another, run as
+ * one launch with their workgroups interleaved when both have about one 128x128
+ * tile per CU: every CU then holds one workgroup of each and one runs while the
+ * other waits.  Results are unchanged.  Profiling names: `dXlin1+dWlin1`,
+ * `dXQKV-fused+dWQKV-fused`. */
+#define SUB_OPT_PAIR_PRODUCTS 5
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

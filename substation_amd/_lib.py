@@ -18,6 +18,7 @@ OPT_FUSE_EPILOGUES = 1
 OPT_FUSE_LN_BACKWARD = 2
 OPT_FUSE_SCORES = 3
 OPT_FUSE_ATTENTION = 4
+OPT_PAIR_PRODUCTS = 5
 FUSE_REQUIRED = 2
 
 

@@ -184,6 +184,7 @@ struct Handle {
     bool fuse_ln_backward = true;
     bool fuse_scores = true;
     int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
+    bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -418,6 +419,29 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
     }
     launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream, h.gws,
                 h.gws_floats);
+}
+
+// Two products that do not depend on one another (a data gradient and the weight
+// gradient next to it) in one launch where they qualify, else one after the other.
+void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1, const char* name1,
+                   const void* addend1, int id2, const void* A2, const void* B2, void* C2, const char* name2,
+                   const char* pair_name) {
+    if (h.pair_products) {
+        ProfScope ps(h, pair_name);
+        const GemmPlan& p1 = h.gemm[id1];
+        const GemmPlan& p2 = h.gemm[id2];
+        GemmEpilogue e1, e2;
+        if (addend1) {
+            e1.bias = (const half_t*)addend1; e1.sbM = p1.sM; e1.sbN = p1.sN;
+            for (int i = 0; i < 3; ++i) e1.sbb[i] = p1.sb[i];
+        }
+        if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha, e1, p2.shape,
+                             (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream))
+            return;
+        ps.cancel();
+    }
+    run_gemm(h, id1, A1, B1, C1, name1, addend1);
+    run_gemm(h, id2, A2, B2, C2, name2);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -811,8 +835,8 @@ void backward(Handle& h, const BwdPtrs& t) {
         op_bdrlb(h, D[DDROP2], h.lb[DDROP2], F[DROP2MASK], h.lf[DROP2MASK], F[LIN1], h.lf[LIN1],
                  D[DLIN1], h.lb[DLIN1], DW[LINB1]);
     }
-    run_gemm(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1");
-    run_gemm(h, G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1");
+    run_gemm_pair(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1", nullptr,
+                  G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1", "dXlin1+dWlin1");
     fused = false;
     if (h.fuse_ln_backward) {
         ProfScope ps(h, "ebsb+blnrd2+baob");
@@ -898,11 +922,12 @@ void backward(Handle& h, const BwdPtrs& t) {
                          aligned16(t.DX);
     if (fuse_dx) {
         // DX = WKQV.DKKQQVV + DRESID1 in one pass; DXATT is not written
-        run_gemm(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1]);
+        run_gemm_pair(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1],
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused");
     } else {
-        run_gemm(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused");
+        run_gemm_pair(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused", nullptr,
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused");
     }
-    run_gemm(h, G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused");
     if (!attn_bias) {
         ProfScope ps(h, "baib");
         op_baib(h, D[DKKQQVV], h.lb[DKKQQVV], DW[BKQV], h.lp[BKQV]);
@@ -1068,6 +1093,7 @@ int sub_set_option(void* handle, int option, int value) {
         if (option == SUB_OPT_FUSE_EPILOGUES) h.fuse_epilogues = value != 0;
         else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
         else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
+        else if (option == SUB_OPT_PAIR_PRODUCTS) h.pair_products = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;

@@ -175,16 +175,24 @@ struct Tile {
     }
 };
 
+// LDS (in halves) of one workgroup of the register-staged kernel: two pipeline
+// stages, reused by the epilogue's per-wave staging slabs.
+template <int TM, int TN, bool AKC, bool BKC>
+constexpr int mfma_lds_halves() {
+    constexpr int stage = Tile<64 * TM, AKC>::HALVES + Tile<64 * TN, BKC>::HALVES;
+    constexpr int slabs = 4 * 32 * (32 * TN + 8);
+    return 2 * stage > slabs ? 2 * stage : slabs;
+}
+
+// One workgroup's share of a product: block `block_id` of `nblocks`.
 template <int TM, int TN, bool AKC, bool BKC, bool FULL>
-__global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
+__device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id, long nblocks, half_t* lds) {
     constexpr int BM = 64 * TM, BN = 64 * TN;
     using TA = Tile<BM, AKC>;
     using TB = Tile<BN, BKC>;
     constexpr int STAGE = TA::HALVES + TB::HALVES;                   // one pipeline stage
     constexpr int STAGE_PITCH = 32 * TN + 8;                          // halves
     constexpr int STAGE_WAVE = 32 * STAGE_PITCH;                      // one 32-row slab per wave
-    constexpr int LDS_HALVES = 2 * STAGE > 4 * STAGE_WAVE ? 2 * STAGE : 4 * STAGE_WAVE;
-    __shared__ __attribute__((aligned(16))) half_t lds[LDS_HALVES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -195,11 +203,8 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
     // within a batch tiles are walked in groups of 8 tile-rows so that the
     // workgroups resident together share A and B tiles in that L2.
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    long lid = blockIdx.x;
-    {
-        const long nblocks = gridDim.x;
-        if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
-    }
+    long lid = block_id;
+    if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
     const int per_batch = tiles_m * tiles_n;
     const int split = (int)(lid % g.splits);        // k-splits of one tile sit next to each other
     lid /= g.splits;
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 
     if (g.splits > 1) {
         // split k: raw fp32 partial tile, [split][batch][M][N]; a second kernel adds them up
-        const long nb_total = (long)gridDim.x / g.splits / per_batch;
+        const long nb_total = nblocks / g.splits / per_batch;
         float* P = g.partial + ((long)split * nb_total + bz) * (long)g.M * g.N;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
@@ -374,6 +379,36 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
                 *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
             }
         }
+    }
+}
+
+template <int TM, int TN, bool AKC, bool BKC, bool FULL>
+__global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) half_t lds[mfma_lds_halves<TM, TN, AKC, BKC>()];
+    gemm_mfma_body<TM, TN, AKC, BKC, FULL>(g, blockIdx.x, gridDim.x, lds);
+}
+
+// Two independent products with the same number of 128x128 tiles in one launch,
+// eight workgroups of the one, then eight of the other: every XCD and (with about
+// one tile per CU each) every CU gets workgroups of both, two per CU, and while
+// one of them waits -- for its operands, at its barrier, in its first fetch or
+// its output write -- the other one runs.  Alone, each product would leave a
+// single wave on every SIMD.
+template <bool A1, bool B1, bool A2, bool B2>
+__global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2) {
+    constexpr int L1 = mfma_lds_halves<2, 2, A1, B1>(), L2 = mfma_lds_halves<2, 2, A2, B2>();
+    __shared__ __attribute__((aligned(16))) half_t lds[L1 > L2 ? L1 : L2];
+    // n1, n2: workgroups of the two products (multiples of 8).  While both have
+    // some left they alternate in groups of 8; the rest belongs to the larger one.
+    const unsigned b = blockIdx.x, both = 2 * (n1 < n2 ? n1 : n2);
+    if (b < both) {
+        const unsigned id = ((b >> 4) << 3) | (b & 7);
+        if ((b >> 3) & 1) gemm_mfma_body<2, 2, A2, B2, true>(g2, id, n2, lds);
+        else gemm_mfma_body<2, 2, A1, B1, true>(g1, id, n1, lds);
+    } else {
+        const unsigned id = b - both / 2;
+        if (n2 > n1) gemm_mfma_body<2, 2, A2, B2, true>(g2, id, n2, lds);
+        else gemm_mfma_body<2, 2, A1, B1, true>(g1, id, n1, lds);
     }
 }
 
@@ -806,6 +841,43 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
     size_t splits = kSplitTarget / tiles;
     if (splits > 8) splits = 8;
     return per * splits;
+}
+
+// Two independent products in one launch (see k_gemm_pair).  Returns false, having
+// launched nothing, unless both are products the register-staged kernel would take
+// as whole 128x128 tiles with about one tile per CU, in an operand orientation
+// that is instantiated; the caller then launches them one after the other.
+bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
+                      const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
+                      half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st) {
+    static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
+    if (off) return false;
+    const GemmShape* sh[2] = {&s1, &s2};
+    Canon c[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
+    bool akc[2], bkc[2];
+    long n[2];
+    for (int i = 0; i < 2; ++i) {
+        const long batch = sh[i]->batch();
+        if (batch == 0 || pick_kind(c[i], akc[i], bkc[i]) != 1) return false;
+        const GemmArgs& a = c[i].a;
+        if (a.M % 128 || a.N % 128 || a.K1 % BK) return false;
+        n[i] = (long)(a.M / 128) * (a.N / 128) * batch;
+        if (n[i] % 8 || n[i] < 128 || n[i] > 384) return false;
+        if (pick_tile(a, batch, akc[i], bkc[i]) != 22) return false;
+        if (akc[i] && bkc[i]) return false;                  // the asynchronous kernel's products stay on their own
+    }
+    dim3 grid((unsigned)(n[0] + n[1]));
+    const unsigned n1 = (unsigned)n[0], n2 = (unsigned)n[1];
+    if (akc[0] && !bkc[0] && !akc[1] && !bkc[1])
+        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+    else if (!akc[0] && !bkc[0] && !akc[1] && !bkc[1])
+        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+    else if (akc[0] && !bkc[0] && akc[1] && !bkc[1])
+        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+    else
+        return false;
+    check_launch("gemm pair");
+    return true;
 }
 
 void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C, float alpha,

@@ -34,6 +34,7 @@ OPERATORS = [
     ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
     ('dWlin2', 'bwd', ('DLIN2', 'DROP2', 'LINW2')),
     ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DLIN1')),
+    ('dXlin1+dWlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1', 'SB1')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
     ('dWlin1', 'bwd', ('DLIN1', 'SB1', 'LINW1')),
     ('ebsb+blnrd2+baob', 'bwd', ('LN1', 'DRESID2', 'DLIN1_LINW1', 'DLIN2', 'DLN1', 'LN1STD', 'LN1DIFF',
@@ -53,6 +54,7 @@ OPERATORS = [
     ('bs', 'bwd', ('ALPHA', 'ATTN_DROP_MASK', 'DATTN_DROP', 'DBETA')),
     ('dX1QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
     ('dX2QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
+    ('dXQKV-fused+dWQKV-fused', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X')),
     ('dXQKV-fused', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X')),
     ('dWQKV-fused', 'bwd', ('X', 'DKKQQVV', 'WKQV')),
     ('baib', 'bwd', ('DKKQQVV', 'BKQV')),
@@ -66,7 +68,8 @@ OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 #: which of them run depends on the layouts of the whole group's tensors.
 ALTERNATIVES = [
     ('QKV-fused', 'aib'),
-    ('dXQKV-fused', 'bei'),
+    ('dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei'),
+    ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
     ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT',
      'baib'),
