@@ -38,12 +38,12 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 88458973, 'attention': 38113622, 'out': 33775361, 'bdrln1': 59015091,
-    'lin1': 84251804, 'bad': 134460163, 'lin2': 109265042, 'bdrln2': 59013701,
-    'bsb+blnrd1': 61022706, 'dXlin2': 84238493, 'dWlin2': 109275573, 'bdrlb': 135394861,
-    'dXlin1': 109260727, 'dWlin1': 109275061, 'ebsb+blnrd2+baob': 79940136, 'dWout': 92477161,
-    'dXout': 33771119, 'attention-bwd-dQ': 55316257, 'attention-bwd-dKdV': 55519010,
-    'dXQKV-fused': 92485226, 'dWQKV-fused': 115565660,
+    'QKV-fused': 88468913, 'attention': 38113652, 'out': 33767950, 'bdrln1': 59012996,
+    'lin1': 84263091, 'bad': 134456888, 'lin2': 109257904, 'bdrln2': 59009138,
+    'bsb+blnrd1': 61023472, 'dXlin2': 84250804, 'dWlin2': 109268217, 'bdrlb': 135394945,
+    'dXlin1+dWlin1': 299754811, 'ebsb+blnrd2+baob': 79940105, 'dWout': 92476695, 'dXout': 33770162,
+    'attention-bwd-dQ': 55315932, 'attention-bwd-dKdV': 55519064,
+    'dXQKV-fused+dWQKV-fused': 287512461,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
