@@ -123,7 +123,11 @@ const char* sub_last_error(void);
  * "KJ"; -inf above the diagonal for a causal layer).  As in
  * substation/attention.py:65-68 the mask is added to the raw scores, before the
  * 1/sqrt(P) scaling.  encoder_forward uses it until it is cleared with NULL;
- * encoder_backward needs nothing (masked positions have zero probability). */
+ * encoder_backward needs nothing (masked positions have zero probability).
+ * The mask's contents are read by every encoder_forward call (also to find the
+ * tiles that are -inf throughout, which the attention kernels pass over) and
+ * must stay unchanged until the matching encoder_backward has been issued.
+ * Allocates a small table: not to be called during a graph capture. */
 int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layout);
 
 /* Options.  SUB_OPT_FUSE_EPILOGUES (default 1): add BKQV in the epilogue of the

@@ -180,6 +180,9 @@ struct Handle {
     uint32_t* step_dev = nullptr;     // optional device-side dropout step (HIP-graph replays)
     const void* attn_mask = nullptr;  // optional additive [J,K] attention mask (caller-owned)
     Layout l_attn_mask;
+    void* mask_plan = nullptr;        // what the mask leaves to do (see mask_plan())
+    size_t mask_plan_bytes = 0;
+    bool mask_plan_built = false;     // a forward pass has filled it for the present mask pointer
     bool fuse_epilogues = true;
     bool fuse_ln_backward = true;
     bool fuse_scores = true;
@@ -196,6 +199,7 @@ struct Handle {
         const bool swapped = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
         if (ws) (void)hipFree(ws);
         if (gws) (void)hipFree(gws);
+        if (mask_plan) (void)hipFree(mask_plan);
         for (auto& e : prof) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
         if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
     }
@@ -636,6 +640,17 @@ bool attention_fused(const Handle& h, void* const* F, AttnArgs& a) {
     return ok;
 }
 
+// The plan of the mask (which tiles it leaves to do, which blocks need the
+// addition) is rebuilt from the mask's present contents by every forward pass: the
+// caller owns the mask and may have rewritten it.  The backward pass reuses the plan
+// of its forward pass, whose mask it has to share anyway (and builds it when this
+// handle has run no forward pass since the mask was set).
+void mask_plan(Handle& h, AttnArgs& a, bool forward) {
+    if (!a.amask || !h.mask_plan) return;
+    launch_mha_mask_plan(a, h.mask_plan, forward || !h.mask_plan_built, h.stream);
+    h.mask_plan_built = true;
+}
+
 // bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
 // false, having done nothing, when the shape or the layouts rule the fused
 // kernel out; the caller then runs the separate operators.
@@ -750,6 +765,7 @@ void forward(Handle& h, const FwdPtrs& t) {
     const bool fused_attention = attention_fused(h, F, at);
     if (fused_attention) {
         ProfScope ps(h, "attention");
+        mask_plan(h, at, true);
         launch_mha_forward(at, (int)h.sz.n[dP], make_key(h, SUB_SITE_SOFTMAX, h.p_softmax), h.stream);
     }
     bool fused_scores = fused_attention;
@@ -892,6 +908,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         };
         {
             ProfScope ps(h, "attention-bwd-dQ");
+            mask_plan(h, at, false);
             if (attn_bias) at.bias_q = take_ws(h, (size_t)H * ntq * P);
             launch_mha_backward_dq(at, P, h.stream);
             if (attn_bias) finish(at.bias_q, 1, ntq, dbias + 1 * lbias.stride[dQ], nullptr);
@@ -1216,10 +1233,20 @@ int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const voi
 int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layout) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
+        h.mask_plan_built = false;
         if (!attn_mask) { h.attn_mask = nullptr; return; }
         Layout l = L(h, layout);
         if (l.rank != 2 || !l.has[dJ] || !l.has[dK]) fail("sub_set_attention_mask: layout must be JK or KJ");
         h.attn_mask = attn_mask; h.l_attn_mask = l;
+        const Sizes& z = h.sz;
+        if (z.n[dJ] % 128 == 0 && z.n[dK] % 128 == 0 && !h.mask_plan) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(h.stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+                fail("sub_set_attention_mask: allocates a small table, call it outside the graph capture");
+            const size_t bytes = mha_mask_plan_bytes(z.n[dJ], z.n[dK]);
+            hip_check(hipMalloc(&h.mask_plan, bytes), "hipMalloc(mask plan)");
+            h.mask_plan_bytes = bytes;
+        }
     });
 }
 

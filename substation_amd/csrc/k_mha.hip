@@ -198,22 +198,121 @@ __device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
 // Additive attention mask (substation/attention.py:65-68: added to the raw scores,
 // before the scaling) for the 16 scores of a lane.  QUERY_LANES: the lane holds
 // one query and registers run over keys (forward, dQ); otherwise the lane holds
-// one key and registers run over queries (dK/dV).
+// one key and registers run over queries (dK/dV).  The values of a tile are loaded
+// while the tile before it is worked on, ahead of that pass's K/V (Q/dO) loads:
+// loads complete in order, so a wait for mask values issued after those would
+// also wait for them.
+struct MaskRegs { h4 q[4]; };
+
 template <bool QUERY_LANES>
-__device__ __forceinline__ void add_mask(const AttnArgs& a, unsigned lane_pos, unsigned tile0, int hi, f16v& s) {
+__device__ __forceinline__ void load_mask(const AttnArgs& a, unsigned lane_pos, unsigned tile0, int hi, MaskRegs& mk) {
     const long lane_stride = QUERY_LANES ? a.am_sj : a.am_sk, reg_stride = QUERY_LANES ? a.am_sk : a.am_sj;
     const half_t* m = a.amask + (long)lane_pos * lane_stride + (long)tile0 * reg_stride;
     if (reg_stride == 1) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const h4 w = *reinterpret_cast<const h4*>(m + q * 8 + hi * 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) s[q * 4 + e] += (float)w[e];
-        }
+        for (int q = 0; q < 4; ++q) mk.q[q] = *reinterpret_cast<const h4*>(m + q * 8 + hi * 4);
     } else {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] += (float)m[(long)reg_pos(v, hi) * reg_stride];
+        for (int v = 0; v < 16; ++v) mk.q[v >> 2][v & 3] = m[(long)reg_pos(v, hi) * reg_stride];
     }
+}
+
+// The scores of a tile start from the mask's values instead of zero: the product
+// accumulates on top of them.
+__device__ __forceinline__ void start_from_mask(const MaskRegs& mk, f16v& s) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] = (float)mk.q[v >> 2][v & 3];
+}
+
+// ---------------------------------------------------------------------------
+// What a mask leaves to do.  Each 32x32 block of the mask is classed as mixed,
+// dead (all -inf: the scores vanish) or clear (all zero: nothing to add).  Per
+// workgroup of the attention kernels (128 queries, or 128 keys in the dK/dV
+// kernel) a list names the tiles of the other side that are not dead for all
+// four waves; the kernels walk that list instead of all tiles.
+//   row of a list: [0] = number of entries, then the entries, then padding that
+//   reads as "tile 0, dead for all waves" (the kernels read up to 3 past the end).
+//   entry: bits 0..15 tile index, bits 16+2w.. the class of the block for wave w.
+// ---------------------------------------------------------------------------
+enum : uint32_t { BLOCK_MIXED = 0, BLOCK_DEAD = 1, BLOCK_CLEAR = 2 };
+constexpr uint32_t kAllDead = BLOCK_DEAD * 0x55u << 16;
+constexpr int kListPad = 4;       // the count and three entries of padding
+
+// One wave per 32x32 block of the mask.
+__global__ __launch_bounds__(64) void k_mha_mask_classes(const half_t* mask, long sj, long sk, int K, uint8_t* cls) {
+    const int lane = threadIdx.x, nkb = K / 32;
+    const int qb = blockIdx.x / nkb, kb = blockIdx.x % nkb;
+    const half_t* p = mask + (long)(qb * 32 + (lane & 31)) * sj + (long)(kb * 32 + (lane >> 5) * 16) * sk;
+    bool dead = true, clear = true;
+    for (int i = 0; i < 16; ++i) {
+        const float x = (float)p[(long)i * sk];
+        dead = dead && (x == -INFINITY);
+        clear = clear && (x == 0.f);
+    }
+    const bool all_dead = __builtin_amdgcn_ballot_w64(dead) == ~0ull;
+    const bool all_clear = __builtin_amdgcn_ballot_w64(clear) == ~0ull;
+    if (lane == 0) cls[blockIdx.x] = all_dead ? BLOCK_DEAD : all_clear ? BLOCK_CLEAR : BLOCK_MIXED;
+}
+
+// One wave per list row: blocks 0 .. J/128-1 build the key-tile lists of the query
+// blocks, the others the query-tile lists of the key blocks.
+__global__ __launch_bounds__(64) void k_mha_mask_lists(const uint8_t* cls, int J, int K, uint32_t* qlist, uint32_t* klist) {
+    const int lane = threadIdx.x, nqb = J / 32, nkb = K / 32;
+    const bool by_query = (int)blockIdx.x < J / QB;
+    const int blk = by_query ? blockIdx.x : blockIdx.x - J / QB;
+    const int ntiles = by_query ? nkb : nqb;
+    uint32_t* row = (by_query ? qlist : klist) + (size_t)blk * (ntiles + kListPad);
+    unsigned count = 0;
+    for (int t0 = 0; t0 < ntiles; t0 += 64) {
+        const int t = t0 + lane;
+        uint32_t e = kAllDead;
+        if (t < ntiles) {
+            e = (uint32_t)t;
+            for (int w = 0; w < 4; ++w) {
+                const uint32_t c = by_query ? cls[(size_t)(blk * 4 + w) * nkb + t] : cls[(size_t)t * nkb + blk * 4 + w];
+                e |= c << (16 + 2 * w);
+            }
+        }
+        const bool live = (e & (0xffu << 16)) != kAllDead;
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(live);
+        if (live) row[1 + count + __builtin_popcountll(m & ((1ull << lane) - 1))] = e;
+        count += (unsigned)__builtin_popcountll(m);
+    }
+    if (lane == 0) row[0] = count;
+    for (int i = count + lane; i < ntiles + kListPad - 1; i += 64) row[1 + i] = kAllDead;
+}
+
+// Which block of 128 (and which head and sample) a workgroup takes when a mask has
+// left the blocks unequal amounts to do.  Workgroups start in the order of their
+// index.  The blocks of a head and sample are ranked long to short (the reverse of
+// their positions when the last has more to do than the first: a causal mask seen
+// from the queries) and dealt in four passes over the heads and samples of an XCD,
+// a quarter of the ranks per pass, so that the launch does not end on a few long
+// blocks running alone.
+__device__ __forceinline__ void masked_order(const uint32_t* list, unsigned nblocks, unsigned ntiles, unsigned ngroups,
+                                             unsigned lb, unsigned& blk, unsigned& hb) {
+    blk = lb % nblocks; hb = lb / nblocks;
+    if (!list) return;
+    const bool rev = list[(size_t)(nblocks - 1) * (ntiles + kListPad)] > list[0];
+    unsigned rank = blk;
+    if (nblocks % 4 == 0 && ngroups % 8 == 0) {
+        const unsigned gx = ngroups / 8, per = nblocks / 4;          // groups per XCD; blocks per pass and group
+        const unsigned x = lb / (gx * nblocks), i = lb % (gx * nblocks);
+        const unsigned pass = i / (gx * per), rem = i % (gx * per);
+        hb = x * gx + rem / per;
+        rank = pass * per + rem % per;
+    }
+    blk = rev ? nblocks - 1 - rank : rank;
+}
+
+// Entry i of a list row; without a list every tile is walked and treated as mixed.
+template <bool MASKED>
+__device__ __forceinline__ uint32_t live_entry(const uint32_t* row, unsigned i) {
+    return (MASKED && row) ? row[1 + i] : i;
+}
+__device__ __forceinline__ unsigned entry_tile(uint32_t e) { return e & 0xffffu; }
+__device__ __forceinline__ uint32_t entry_class(uint32_t e, int wave) {
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)((e >> (16 + 2 * wave)) & 3u));
 }
 
 // ---------------------------------------------------------------------------
@@ -241,20 +340,25 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned qblocks = a.J / QB;
     const unsigned lb = logical_block();
-    const unsigned qb = lb % qblocks, hb = lb / qblocks;
+    const unsigned nt = a.K / 32;
+    unsigned qb = lb % qblocks, hb = lb / qblocks;
+    if (MASKED) masked_order(a.qlist, qblocks, nt, a.H * a.B, lb, qb, hb);
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned j = qb * QB + wave * 32 + l32;                    // this lane's query
     const unsigned row = (h * a.B + b) * a.J + j;                    // its score row
-    const unsigned nt = a.K / 32;
     const float c = a.alpha * LOG2E;
+    // the key tiles to walk: all of them, or those a mask leaves for these 128 queries
+    const uint32_t* live = (MASKED && a.qlist) ? a.qlist + (size_t)qb * (nt + kListPad) : nullptr;
+    const unsigned n = live ? live[0] : nt;
+    uint32_t e0 = live_entry<MASKED>(live, 0), e1 = live_entry<MASKED>(live, 1), e2 = live_entry<MASKED>(live, 2);
 
     h8 fq[G::NKS], fk[G::NKS], kr[G::VL], vr[G::VL];
     {   // the first two tiles and the query rows: all loads in flight together
         h8 kr1[G::VL], vr1[G::VL];
-        tile_fetch<P>(a.k, h, b, 0, tid, kr);
-        tile_fetch<P>(a.v, h, b, 0, tid, vr);
-        tile_fetch<P>(a.k, h, b, 32, tid, kr1);
-        tile_fetch<P>(a.v, h, b, 32, tid, vr1);
+        tile_fetch<P>(a.k, h, b, entry_tile(e0) * 32, tid, kr);
+        tile_fetch<P>(a.v, h, b, entry_tile(e0) * 32, tid, vr);
+        tile_fetch<P>(a.k, h, b, entry_tile(e1) * 32, tid, kr1);
+        tile_fetch<P>(a.v, h, b, entry_tile(e1) * 32, tid, vr1);
         row_frags<P>(a.q, h, b, j, hi, fq);
         tile_put<P>(kt[0], tid, kr);
         tile_put<P>(vt[0], tid, vr);
@@ -272,20 +376,26 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
     float m_ref = -INFINITY, l_run = 0.f;                            // l_run: this lane's keys only
     const float slack = RESCALE_SLACK / c;
     int cur = 0, nxt = 1, nn = 2;
+    MaskRegs mk = {};
+    if (MASKED && n > 0 && entry_class(e0, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e0) * 32, hi, mk);
     wait_loads();
 
-    for (unsigned t = 0; t < nt; ++t) {
-        const bool fetch = t + 2 < nt;
+    for (unsigned i = 0; i < n; ++i) {
+        const uint32_t e3 = live_entry<MASKED>(live, i + 3);
+        const unsigned t = entry_tile(e0);
+        const bool from_mask = MASKED && entry_class(e0, wave) != BLOCK_CLEAR;
+        const bool fetch = i + 2 < n;
         if (fetch) {
-            tile_fetch<P>(a.k, h, b, (t + 2) * 32, tid, kr);
-            tile_fetch<P>(a.v, h, b, (t + 2) * 32, tid, vr);
+            tile_fetch<P>(a.k, h, b, entry_tile(e2) * 32, tid, kr);
+            tile_fetch<P>(a.v, h, b, entry_tile(e2) * 32, tid, vr);
         }
         f16v s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
+        if (from_mask) start_from_mask(mk, s);
+        if (MASKED && i + 1 < n && entry_class(e1, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e1) * 32, hi, mk);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
-        if (MASKED) add_mask<true>(a, j, t * 32, hi, s);
         // fragments for the second product of this tile and the first of the next
         h8 va[2][G::NPT];
 #pragma unroll
@@ -317,7 +427,9 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         mt = fmaxf(mt, __shfl_xor(mt, 32));
         if (__builtin_amdgcn_ballot_w64(mt > m_ref + slack) != 0) {
             const float m_new = fmaxf(m_ref, mt);
-            const float corr = __builtin_amdgcn_exp2f((m_ref - m_new) * c);
+            // (masked: a query that has seen no key yet has nothing to rescale; the
+            // difference of its two infinities is not a number)
+            const float corr = (MASKED && m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f((m_ref - m_new) * c);
             m_ref = m_new;
             l_run *= corr;
 #pragma unroll
@@ -353,6 +465,7 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         }
         __syncthreads();
         const int x = cur; cur = nxt; nxt = nn; nn = x;
+        e0 = e1; e1 = e2; e2 = e3;
     }
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     store_rows<P>(a.o, h, b, j, hi, o, 1.0f / l_tot);
@@ -370,12 +483,16 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned qblocks = a.J / QB;
     const unsigned lb = logical_block();
-    const unsigned qb = lb % qblocks, hb = lb / qblocks;
+    const unsigned nt = a.K / 32;
+    unsigned qb = lb % qblocks, hb = lb / qblocks;
+    if (MASKED) masked_order(a.qlist, qblocks, nt, a.H * a.B, lb, qb, hb);
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned j = qb * QB + wave * 32 + l32;
     const unsigned row = (h * a.B + b) * a.J + j;
-    const unsigned nt = a.K / 32;
     const float c = a.alpha * LOG2E;
+    const uint32_t* live = (MASKED && a.qlist) ? a.qlist + (size_t)qb * (nt + kListPad) : nullptr;
+    const unsigned n = live ? live[0] : nt;
+    uint32_t e0 = live_entry<MASKED>(live, 0), e1 = live_entry<MASKED>(live, 1), e2 = live_entry<MASKED>(live, 2);
 
     h8 fq[G::NKS], fdo[G::NKS], fk[G::NKS], fv[G::NKS], kr[G::VL], vr[G::VL];
     float dsum, lse;
@@ -383,15 +500,15 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
     {   // the first two tiles, the rows of this lane's query and its statistics: all
         // loads in flight together
         h8 kr1[G::VL], vr1[G::VL], fo[G::NKS];
-        tile_fetch<P>(a.k, h, b, 0, tid, kr);
-        tile_fetch<P>(a.v, h, b, 0, tid, vr);
-        tile_fetch<P>(a.k, h, b, 32, tid, kr1);
-        tile_fetch<P>(a.v, h, b, 32, tid, vr1);
+        tile_fetch<P>(a.k, h, b, entry_tile(e0) * 32, tid, kr);
+        tile_fetch<P>(a.v, h, b, entry_tile(e0) * 32, tid, vr);
+        tile_fetch<P>(a.k, h, b, entry_tile(e1) * 32, tid, kr1);
+        tile_fetch<P>(a.v, h, b, entry_tile(e1) * 32, tid, vr1);
         row_frags<P>(a.q, h, b, j, hi, fq);
         row_frags<P>(a.d_o, h, b, j, hi, fdo);
         row_frags<P>(a.o, h, b, j, hi, fo);
         lse = a.lse[row];
-        word = a.keep[(size_t)row * nt];
+        word = a.keep[(size_t)row * nt + entry_tile(e0)];
         tile_put<P>(kt[0], tid, kr);
         tile_put<P>(vt[0], tid, vr);
         tile_put<P>(kt[1], tid, kr1);
@@ -414,23 +531,28 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) dq[pt][v] = 0.f;
     int cur = 0, nxt = 1, nn = 2;
+    MaskRegs mk = {};
+    if (MASKED && n > 0 && entry_class(e0, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e0) * 32, hi, mk);
     wait_loads();
 
-    for (unsigned t = 0; t < nt; ++t) {
-        const bool fetch = t + 2 < nt;
+    for (unsigned i = 0; i < n; ++i) {
+        const uint32_t e3 = live_entry<MASKED>(live, i + 3);
+        const bool from_mask = MASKED && entry_class(e0, wave) != BLOCK_CLEAR;
+        const bool fetch = i + 2 < n;
         if (fetch) {
-            tile_fetch<P>(a.k, h, b, (t + 2) * 32, tid, kr);
-            tile_fetch<P>(a.v, h, b, (t + 2) * 32, tid, vr);
+            tile_fetch<P>(a.k, h, b, entry_tile(e2) * 32, tid, kr);
+            tile_fetch<P>(a.v, h, b, entry_tile(e2) * 32, tid, vr);
         }
-        const uint32_t wordn = t + 1 < nt ? a.keep[(size_t)row * nt + t + 1] : 0u;
+        const uint32_t wordn = i + 1 < n ? a.keep[(size_t)row * nt + entry_tile(e1)] : 0u;
         f16v s, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
+        if (from_mask) start_from_mask(mk, s);
+        if (MASKED && i + 1 < n && entry_class(e1, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e1) * 32, hi, mk);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fv[ks], fdo[ks], dp, 0, 0, 0);
-        if (MASKED) add_mask<true>(a, j, t * 32, hi, s);
         h8 ka[2][G::NPT];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
@@ -466,6 +588,7 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         word = wordn;
         __syncthreads();
         const int x = cur; cur = nxt; nxt = nn; nn = x;
+        e0 = e1; e1 = e2; e2 = e3;
     }
     store_rows<P>(a.dq, h, b, j, hi, dq, a.alpha);
     if (a.bias_q)
@@ -488,18 +611,23 @@ struct KvStage {
 };
 
 template <int P, bool MASKED>
-__global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
+__global__ __launch_bounds__(256, (P == 64 && MASKED) ? 2 : 1) void k_mha_bwd_dkv(AttnArgs a) {
     using G = Geo<P>;
     __shared__ __attribute__((aligned(16))) KvStage<P> stage[RING];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
     const unsigned kblocks = a.K / QB;
     const unsigned lb = logical_block();
-    const unsigned kb = lb % kblocks, hb = lb / kblocks;
+    const unsigned nq = a.J / 32, nkt = a.K / 32;
+    unsigned kb = lb % kblocks, hb = lb / kblocks;
+    if (MASKED) masked_order(a.klist, kblocks, nq, a.H * a.B, lb, kb, hb);
     const unsigned b = hb % a.B, h = hb / a.B;
     const unsigned kpos = kb * QB + wave * 32 + l32;                 // this lane's key
     const unsigned row0 = (h * a.B + b) * a.J;                       // score row of query 0
-    const unsigned nq = a.J / 32, nkt = a.K / 32;
     const float c = a.alpha * LOG2E;
+    // the query tiles to walk: all of them, or those a mask leaves for these 128 keys
+    const uint32_t* live = (MASKED && a.klist) ? a.klist + (size_t)kb * (nq + kListPad) : nullptr;
+    const unsigned n = live ? live[0] : nq;
+    uint32_t e0 = live_entry<MASKED>(live, 0), e1 = live_entry<MASKED>(live, 1), e2 = live_entry<MASKED>(live, 2);
 
     h8 fk[G::NKS], fv[G::NKS], fq[G::NKS], fdo[G::NKS];
     struct InFlight {             // one tile of queries on its way from memory
@@ -530,8 +658,8 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
     {
         InFlight f1;
         f1.stat = 0.f; f1.kw = make_uint4(0, 0, 0, 0);
-        fetch(0, fl);
-        fetch(1, f1);
+        fetch(entry_tile(e0), fl);
+        fetch(entry_tile(e1), f1);
         row_frags<P>(a.k, h, b, kpos, hi, fk);
         row_frags<P>(a.v, h, b, kpos, hi, fv);
         put(stage[0], fl);
@@ -547,20 +675,25 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) { dk[pt][v] = 0.f; dv[pt][v] = 0.f; }
     int cur = 0, nxt = 1, nn = 2;
+    MaskRegs mk = {};
+    if (MASKED && n > 0 && entry_class(e0, wave) != BLOCK_CLEAR) load_mask<false>(a, kpos, entry_tile(e0) * 32, hi, mk);
     wait_loads();
 
-    for (unsigned qt = 0; qt < nq; ++qt) {
-        const bool more = qt + 2 < nq;
-        if (more) fetch(qt + 2, fl);
+    for (unsigned i = 0; i < n; ++i) {
+        const uint32_t e3 = live_entry<MASKED>(live, i + 3);
+        const bool from_mask = MASKED && entry_class(e0, wave) != BLOCK_CLEAR;
+        const bool more = i + 2 < n;
+        if (more) fetch(entry_tile(e2), fl);
         const KvStage<P>& sg = stage[cur];
         f16v s, dp;
 #pragma unroll
         for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
+        if (from_mask) start_from_mask(mk, s);
+        if (MASKED && i + 1 < n && entry_class(e1, wave) != BLOCK_CLEAR) load_mask<false>(a, kpos, entry_tile(e1) * 32, hi, mk);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fq[ks], fk[ks], s, 0, 0, 0);
 #pragma unroll
         for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fdo[ks], fv[ks], dp, 0, 0, 0);
-        if (MASKED) add_mask<false>(a, kpos, qt * 32, hi, s);
         h8 qa[2][G::NPT], da[2][G::NPT];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
@@ -599,6 +732,7 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dkv(AttnArgs a) {
         if (more) put(stage[nn], fl);
         __syncthreads();
         const int x = cur; cur = nxt; nxt = nn; nn = x;
+        e0 = e1; e1 = e2; e2 = e3;
     }
     store_rows<P>(a.dk, h, b, kpos, hi, dk, a.alpha);
     store_rows<P>(a.dv, h, b, kpos, hi, dv, 1.0f);
@@ -639,6 +773,29 @@ bool mha_forward_ok(const AttnArgs& a, int P) {
     return mha_shape_ok(a.H, a.B, a.J, a.K, P) && a.alpha > 0.f && side_ok(a.q) && side_ok(a.k) && side_ok(a.v) && side_ok(a.o) &&
            a.lse && a.keep && (reinterpret_cast<uintptr_t>(a.lse) & 15) == 0 &&
            (reinterpret_cast<uintptr_t>(a.keep) & 15) == 0 && mask_ok(a);
+}
+
+namespace {
+size_t up16(size_t x) { return (x + 15) & ~(size_t)15; }
+size_t qlist_bytes(long J, long K) { return up16((size_t)(J / QB) * (size_t)(K / 32 + kListPad) * 4); }
+size_t klist_bytes(long J, long K) { return up16((size_t)(K / QB) * (size_t)(J / 32 + kListPad) * 4); }
+}  // namespace
+
+size_t mha_mask_plan_bytes(long J, long K) {
+    return qlist_bytes(J, K) + klist_bytes(J, K) + up16((size_t)(J / 32) * (size_t)(K / 32));
+}
+
+void launch_mha_mask_plan(AttnArgs& a, void* plan, bool rebuild, hipStream_t st) {
+    uint32_t* qlist = (uint32_t*)plan;
+    uint32_t* klist = (uint32_t*)((char*)plan + qlist_bytes(a.J, a.K));
+    uint8_t* cls = (uint8_t*)plan + qlist_bytes(a.J, a.K) + klist_bytes(a.J, a.K);
+    if (rebuild) {
+        hipLaunchKernelGGL(k_mha_mask_classes, dim3((unsigned)((a.J / 32) * (a.K / 32))), dim3(64), 0, st, a.amask,
+                           a.am_sj, a.am_sk, a.K, cls);
+        hipLaunchKernelGGL(k_mha_mask_lists, dim3((unsigned)(a.J / QB + a.K / QB)), dim3(64), 0, st, cls, a.J, a.K, qlist,
+                           klist);
+    }
+    a.qlist = qlist; a.klist = klist;
 }
 
 void launch_mha_forward(const AttnArgs& a, int P, PhiloxKey key, hipStream_t st) {

@@ -129,6 +129,12 @@ struct AttnArgs {
     float* bias_kv = nullptr;
     const half_t* amask = nullptr;   // optional additive mask over (query, key), added before the scaling
     long am_sj = 0, am_sk = 0;
+    // optional, with amask: [J/32][K/32] bytes, non-zero where the mask is -inf over the
+    // whole 32x32 block (mha_mask_blocks); such tiles are not computed at all
+    // optional, built from the mask by launch_mha_mask_plan: per block of 128 queries the
+    // key tiles the mask leaves to do, per block of 128 keys the query tiles
+    const uint32_t* qlist = nullptr;
+    const uint32_t* klist = nullptr;
 };
 // head_size 64 or 128, J and K multiples of 128
 bool mha_shape_ok(long H, long B, long J, long K, long head_size);
@@ -137,6 +143,11 @@ size_t mha_keep_bytes(long H, long B, long J, long K);
 bool mha_forward_ok(const AttnArgs& a, int head_size);
 bool mha_backward_ok(const AttnArgs& a, int head_size);
 void launch_mha_forward(const AttnArgs& a, int head_size, PhiloxKey key, hipStream_t st);
+// skip[J/32][K/32] = 1 where mask[j][k] is -inf for every (j, k) of the block
+// Device bytes of the plan of a [J, K] mask, and the launches that fill it (rebuild)
+// and point the arguments at it.  J and K multiples of 128.
+size_t mha_mask_plan_bytes(long J, long K);
+void launch_mha_mask_plan(AttnArgs& a, void* plan, bool rebuild, hipStream_t st);
 void launch_mha_backward_dq(const AttnArgs& a, int head_size, hipStream_t st);
 void launch_mha_backward_dkv(const AttnArgs& a, int head_size, hipStream_t st);
 

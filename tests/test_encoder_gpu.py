@@ -362,6 +362,10 @@ def test_fused_epilogues_match_unfused(which, dims, act):
     ('mi355x', (2, 256, 2, 128), 'gelu', 0.1, 'JK'),           # causal mask plus finite entries
     ('mi355x', (2, 256, 2, 256), 'gelu', 0.1, 'KJ'),           # the same, stored key-major
     ('mi355x', (2, 128, 2, 128), 'gelu', 0.1, 'late'),         # first keys masked out for every query
+    ('mi355x', (2, 512, 2, 128), 'gelu', 0.1, 'JK'),           # whole 32x32 blocks masked out: the kernels pass over them
+    ('mi355x', (2, 512, 2, 128), 'gelu', 0.1, 'band'),         # blocks masked out before, between and after the visible keys
+    ('mi355x', (4, 512, 2, 128), 'gelu', 0.1, 'JK'),           # eight (head, sample) pairs: blocks dealt long ones first
+    ('mi355x', (2, 512, 4, 256), 'gelu', 0.1, 'band'),
 ])
 def test_attention_in_registers_matches_separate_operators(which, dims, act, p, mask):
     """The attention kernels that keep the scores in registers (default) against
@@ -383,6 +387,10 @@ def test_attention_in_registers_matches_separate_operators(which, dims, act, p, 
         if mask == 'late':      # no query sees the first 40 keys: the running softmax starts without a reference
             am = 2.0 * torch.randn(L, L, generator=g)
             am[:, :40] = float('-inf')
+        elif mask == 'band':    # each query sees keys within 70 positions and a stripe of far ones
+            jj, kk = torch.meshgrid(torch.arange(L), torch.arange(L), indexing='ij')
+            am = 2.0 * torch.randn(L, L, generator=g)
+            am[((jj - kk).abs() > 70) & ~((kk >= 300) & (kk < 330))] = float('-inf')
         elif mask == 'KJ':
             am, am_layout = am.t().contiguous(), 'KJ'
         am = am.half().cuda()
