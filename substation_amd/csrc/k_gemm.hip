@@ -428,10 +428,10 @@ typedef __attribute__((address_space(1))) const void* global_void_ptr;
 
 constexpr int waitcnt_vm(int vm) { return (vm & 0xF) | ((vm >> 4) << 14) | 0x0F70; }
 
-template <int ROWS, bool KC>
+template <int ROWS, bool KC, int NW>
 struct DTile {
     static constexpr int HALVES = ROWS * BK;
-    static constexpr int NV = ROWS / 32;            // loads per thread (16 per tile per wave group)
+    static constexpr int NV = ROWS / (8 * NW);      // loads per thread: the tile is ROWS / 8 slabs of 1024 bytes
     static constexpr int VPR = ROWS / 8;            // 16-byte units per k-row (!KC)
 
     static __device__ __forceinline__ int kc_off(int row, int slot) {
@@ -490,23 +490,33 @@ struct DTile {
     }
 };
 
-template <int TM, int TN, bool AKC, bool BKC, int S>
-__global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
+// NW waves as 2 x (NW / 2); each wave owns TM x TN accumulator tiles of 32 x 32.
+// Eight waves (two per SIMD) on a 256 x 256 tile: a wave cannot issue past an
+// asynchronous load that the memory path has not accepted yet, and with all 256 CUs
+// drawing on L2 that takes long (measured: the loads of a step alone cost about as
+// much time as its multiplications, and with one wave per SIMD the two add up);
+// while one wave of a SIMD sits in the issue of its loads the other multiplies.
+template <int TM, int TN, bool AKC, bool BKC, int S, int NW>
+__global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     static_assert(S == 2 || S == 3, "two or three LDS stages");
-    constexpr int BM = 64 * TM, BN = 64 * TN;
-    using TA = DTile<BM, AKC>;
-    using TB = DTile<BN, BKC>;
+    static_assert(NW == 4 || NW == 8, "four or eight waves");
+    constexpr int WN = NW / 2;
+    constexpr int BM = 64 * TM, BN = 32 * TN * WN;
+    using TA = DTile<BM, AKC, NW>;
+    using TB = DTile<BN, BKC, NW>;
     constexpr int STAGE = TA::HALVES + TB::HALVES;
     constexpr int STAGE_PITCH = 32 * TN + 8;
     constexpr int STAGE_WAVE = 32 * STAGE_PITCH;
-    static_assert(4 * STAGE_WAVE <= STAGE, "epilogue staging must fit one stage");
+    static_assert(NW * STAGE_WAVE <= STAGE, "epilogue staging must fit one stage");
+    // one array per stage: the compiler then sees that an asynchronous load into one
+    // stage does not alias the fragment reads from another, and adds no waits of its own
     __shared__ __attribute__((aligned(16))) half_t st0[STAGE];
     __shared__ __attribute__((aligned(16))) half_t st1[STAGE];
-    __shared__ __attribute__((aligned(16))) half_t st2[S == 3 ? STAGE : 8];
+    __shared__ __attribute__((aligned(16))) half_t st2[S > 2 ? STAGE : 8];
     constexpr int L = TA::NV + TB::NV;               // loads per thread per tile
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, hi = lane >> 5;
 
     const int tiles_m = g.M / BM, tiles_n = g.N / BN;
@@ -563,7 +573,7 @@ __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
         fetched += more_ ? 1 : 0;                                                                 \
     } while (0)
 
-#define SUB_DMA_COMPUTE(stage_)                                                                   \
+#define SUB_DMA_COMPUTE(stage_, nx_)                                                              \
     do {                                                                                          \
         const half_t* sA = stage_;                                                                \
         const half_t* sB = stage_ + TA::HALVES;                                                   \
@@ -573,6 +583,10 @@ __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
             fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
+            if (NW == 8 && ks == BK / 32) {                                                       \
+                if (late) SUB_DMA_ISSUE(nx_);                                                     \
+                __builtin_amdgcn_sched_barrier(0);                                                \
+            }                                                                                     \
             if (ks + 1 < BK / 16) {                                                               \
                 _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
                     fa[(ks + 1) & 1][i] = TA::frag(sA, (wm * TM + i) * 32, ks + 1, lane);         \
@@ -591,35 +605,42 @@ __global__ __launch_bounds__(256) void k_gemm_dma(GemmArgs g) {
     // that the fetch below overwrites (it was computed on one step earlier).
 #define SUB_DMA_STEP(cur_, nxt2_)                                                                 \
     do {                                                                                          \
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(S == 3 ? L : 0));                                   \
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((S - 2) * L));                                      \
         __builtin_amdgcn_s_barrier();                                                             \
-        SUB_DMA_ISSUE(nxt2_);                                                                     \
+        if (!late) SUB_DMA_ISSUE(nxt2_);                                                          \
         /* keep the fetches ahead of the multiply phase: the scheduler must not sink them */      \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        SUB_DMA_COMPUTE(cur_);                                                                    \
+        SUB_DMA_COMPUTE(cur_, nxt2_);                                                            \
     } while (0)
 
-    if (S == 3) {
-        SUB_DMA_ISSUE(st0);                // tile 0
-        SUB_DMA_ISSUE(st1);                // tile 1 (or a surplus copy of the last tile)
-        const int ntriples = nkt / 3;
-        for (int p = 0; p < ntriples; ++p) {
-            SUB_DMA_STEP(st0, st2);
-            SUB_DMA_STEP(st1, st0);
-            SUB_DMA_STEP(st2, st1);
-        }
-        const int rem = nkt - 3 * ntriples;
-        if (rem >= 1) SUB_DMA_STEP(st0, st2);
-        if (rem >= 2) SUB_DMA_STEP(st1, st0);
-    } else {
-        // two stages: the next tile is in flight while the current one is multiplied
+    // Eight waves: the second wave of each SIMD issues its loads half a step after
+    // the first, so that the two are not held up in the issue at the same time.
+    const bool late = NW == 8 && __builtin_amdgcn_readfirstlane(wave) >= 4;
+    // S stages: while tile kt is multiplied, tiles kt+1 .. kt+S-2 are landed or on
+    // their way and the fetch of tile kt+S-1 goes into the stage of tile kt-1.
+    // (One array per stage and each round of S steps as straight-line code: with one
+    // array for the ring, or the steps behind conditions of their own, the compiler
+    // no longer sees which stage a fragment read touches and waits for every load
+    // in flight before it.  More than three stages of 128 x 128 tiles gained nothing.)
+    if (S == 2) {
         SUB_DMA_ISSUE(st0);
-        const int npairs = nkt / 2;
-        for (int p = 0; p < npairs; ++p) {
+        const int nr = nkt / 2;
+        for (int p = 0; p < nr; ++p) {
             SUB_DMA_STEP(st0, st1);
             SUB_DMA_STEP(st1, st0);
         }
         if (nkt & 1) SUB_DMA_STEP(st0, st1);
+    } else if (S == 3) {
+        SUB_DMA_ISSUE(st0);
+        SUB_DMA_ISSUE(st1);
+        const int nr = nkt / 3, rem = nkt - 3 * nr;
+        for (int p = 0; p < nr; ++p) {
+            SUB_DMA_STEP(st0, st2);
+            SUB_DMA_STEP(st1, st0);
+            SUB_DMA_STEP(st2, st1);
+        }
+        if (rem >= 1) SUB_DMA_STEP(st0, st2);
+        if (rem >= 2) SUB_DMA_STEP(st1, st0);
     }
 #undef SUB_DMA_STEP
 #undef SUB_DMA_COMPUTE
@@ -778,13 +799,23 @@ void launch_mfma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t 
     else hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, false, FULL>), grid, dim3(256), 0, st, a);
 }
 
+template <int TM, int TN, int S, int NW>
+void launch_dma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
+    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true, S, NW>), grid, dim3(NW * 64), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false, S, NW>), grid, dim3(NW * 64), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true, S, NW>), grid, dim3(NW * 64), 0, st, a);
+    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false, S, NW>), grid, dim3(NW * 64), 0, st, a);
+}
+
 template <int TM, int TN>
 void launch_dma(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
-    constexpr int S = (TM * TN >= 16) ? 2 : 3;      // 256x256 tiles: two 64 KiB stages
-    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true, S>), grid, dim3(256), 0, st, a);
-    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false, S>), grid, dim3(256), 0, st, a);
-    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true, S>), grid, dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false, S>), grid, dim3(256), 0, st, a);
+    static const bool eight = [] { const char* e = getenv("SUB_GEMM_W8"); return !e || atoi(e) != 0; }();
+    if constexpr (TM * TN >= 16) {                    // 256x256 tiles: two 64 KiB stages
+        if (eight) launch_dma2<TM, TN / 2, 2, 8>(a, akc, bkc, grid, st);
+        else launch_dma2<TM, TN, 2, 4>(a, akc, bkc, grid, st);
+    } else {
+        launch_dma2<TM, TN, 3, 4>(a, akc, bkc, grid, st);
+    }
 }
 
 template <int TM, int TN, bool DMA_OK>
