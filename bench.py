@@ -38,12 +38,12 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 88468913, 'attention': 38113652, 'out': 33767950, 'bdrln1': 59012996,
-    'lin1': 84263091, 'bad': 134456888, 'lin2': 109257904, 'bdrln2': 59009138,
-    'bsb+blnrd1': 61023472, 'dXlin2': 84250804, 'dWlin2': 109268217, 'bdrlb': 135394945,
-    'dXlin1+dWlin1': 299754811, 'ebsb+blnrd2+baob': 79940105, 'dWout': 92476695, 'dXout': 33770162,
-    'attention-bwd-dQ': 55315932, 'attention-bwd-dKdV': 55519064,
-    'dXQKV-fused+dWQKV-fused': 287512461,
+    'QKV-fused': 91468969, 'attention': 38114624, 'out': 33767823, 'bdrln1': 59013649,
+    'lin1': 88312974, 'bad': 134588115, 'lin2': 109257530, 'bdrln2': 59013979,
+    'bsb+blnrd1': 61022329, 'dXlin2': 84115472, 'dWlin2': 109267824, 'bdrlb': 135394553,
+    'dXlin1+dWlin1': 300850548, 'ebsb+blnrd2+baob': 79940110, 'dWout': 92474380, 'dWout split-k sum': 18967823,
+    'dXout': 33770072, 'attention-bwd-dQ': 55315548, 'attention-bwd-dKdV': 55518545, 'dXQKV-fused+dWQKV-fused': 279625554,
+    'column-sum finish': 7819467,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
