@@ -287,6 +287,14 @@ int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void*
  * dimension roles derived from the three layout strings (einsumparser.h:9-55). */
 int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
                   void* C, const char* l_C, float alpha);
+/* The same with an addend in the epilogue: C = alpha * einsum(A, B) + T, where the
+ * dims of T are free or batch dims of C (the others broadcast): a projection and
+ * its bias (gemm.cuh:134-147 followed by block_aib.cuh:17-155, or the `linear` of
+ * substation/transformer.py:41-52 with its bias), or a product added to a residual
+ * (block_bei.cuh:12-106).  T may be C (accumulate in place).  Fails when the layouts
+ * lead to a kernel that has no epilogue. */
+int sub_op_einsum_add(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
+                      const void* T, const char* l_T, void* C, const char* l_C, float alpha);
 
 /* ---- host-only helpers (no GPU needed) ------------------------------------- */
 

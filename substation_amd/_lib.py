@@ -82,6 +82,7 @@ SIGNATURES = {
     'sub_op_baib': (_I, [_VP, _VP, _CP, _VP, _CP]),
     'sub_op_bei': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
     'sub_op_einsum': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
+    'sub_op_einsum_add': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_layout_strides': (_I, [_VP, _CP, ctypes.POINTER(ctypes.c_int64)]),
     'sub_einsum_classify': (_I, [_VP, _CP, _CP, _CP, ctypes.POINTER(ctypes.c_int64)]),
     'sub_philox_fields_host': (_I, [_U64, _U32, _U32, _U64, _U64, ctypes.POINTER(ctypes.c_uint16)]),

@@ -1360,6 +1360,25 @@ int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, c
     });
 }
 
+int sub_op_einsum_add(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
+                      const void* T, const char* l_T, void* C, const char* l_C, float alpha) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        const Layout lc = L(h, l_C), lt = L(h, l_T);
+        GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), lc);
+        GemmEpilogue ep;
+        if (!T) fail("sub_op_einsum_add: null addend");
+        if (!addend_strides(g, lt, lc, ep.sbM, ep.sbN, ep.sbb))
+            fail(std::string("sub_op_einsum_add: the dims of ") + l_T + " are not free or batch dims of " + l_C +
+                 " in one dense run each");
+        ep.bias = (const half_t*)T;
+        if (gemm_kernel_kind(g, A, B, C, ep) != 1)
+            fail("sub_op_einsum_add: these layouts go to the kernel without an epilogue (addend and output "
+                 "must be contiguous along the same free dims)");
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream);
+    });
+}
+
 int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);

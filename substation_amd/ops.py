@@ -134,6 +134,11 @@ class Ops:
         _lib.check(self.lib.sub_op_bei(self._pre(), _p(dxatt), _s(l_dxatt), _p(dresid1),
                                        _s(l_dresid1), _p(dx), _s(l_dx)), 'bei')
 
-    def einsum(self, a, l_a, b, l_b, c, l_c, alpha=1.0):
+    def einsum(self, a, l_a, b, l_b, c, l_c, alpha=1.0, addend=None, l_addend=None):
+        """c = alpha * einsum(a, b) [+ addend, broadcast over the dims it lacks]."""
+        if addend is not None:
+            _lib.check(self.lib.sub_op_einsum_add(self._pre(), _p(a), _s(l_a), _p(b), _s(l_b), _p(addend),
+                                                  _s(l_addend), _p(c), _s(l_c), alpha), 'einsum_add')
+            return
         _lib.check(self.lib.sub_op_einsum(self._pre(), _p(a), _s(l_a), _p(b), _s(l_b), _p(c), _s(l_c),
                                           alpha), 'einsum')
