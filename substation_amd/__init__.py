@@ -7,4 +7,7 @@ def __getattr__(name):
     if name in ('Encoder', 'EncoderStack', 'causal_mask'):       # torch is imported only when the module is used
         from . import encoder
         return getattr(encoder, name)
+    if name == 'DecoderLayer':
+        from . import decoder
+        return decoder.DecoderLayer
     raise AttributeError(name)
