@@ -405,6 +405,16 @@ void configure(Handle& h, const sub_config* c) {
 // ---------------------------------------------------------------------------
 // Operators on a handle
 // ---------------------------------------------------------------------------
+// fp32 scratch for the split contractions of small outputs, grown on demand
+void ensure_gws(Handle& h, size_t floats) {
+    if (floats <= h.gws_floats) return;
+    refuse_capture(h, "split-k workspace");
+    if (h.gws) hip_check(hipFree(h.gws), "hipFree");
+    h.gws = nullptr; h.gws_floats = 0;
+    hip_check(hipMalloc((void**)&h.gws, floats * sizeof(float)), "hipMalloc(split-k workspace)");
+    h.gws_floats = floats;
+}
+
 void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const char* name,
               const void* addend = nullptr) {
     ProfScope ps(h, name);
@@ -414,13 +424,7 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
         ep.bias = (const half_t*)addend; ep.sbM = p.sM; ep.sbN = p.sN;
         for (int i = 0; i < 3; ++i) ep.sbb[i] = p.sb[i];
     }
-    if (h.gws_need > h.gws_floats) {
-        refuse_capture(h, "split-k workspace");
-        if (h.gws) hip_check(hipFree(h.gws), "hipFree");
-        h.gws = nullptr; h.gws_floats = 0;
-        hip_check(hipMalloc((void**)&h.gws, h.gws_need * sizeof(float)), "hipMalloc(split-k workspace)");
-        h.gws_floats = h.gws_need;
-    }
+    ensure_gws(h, h.gws_need);
     launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream, h.gws,
                 h.gws_floats);
 }
@@ -1356,7 +1360,8 @@ int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, c
         Handle& h = as_handle(handle); need_cfg(h);
         GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), L(h, l_C));
         GemmEpilogue ep;
-        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream);
+        ensure_gws(h, gemm_splitk_ws_floats(g));
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream, h.gws, h.gws_floats);
     });
 }
 
@@ -1375,7 +1380,8 @@ int sub_op_einsum_add(void* handle, const void* A, const char* l_A, const void* 
         if (gemm_kernel_kind(g, A, B, C, ep) != 1)
             fail("sub_op_einsum_add: these layouts go to the kernel without an epilogue (addend and output "
                  "must be contiguous along the same free dims)");
-        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream);
+        ensure_gws(h, gemm_splitk_ws_floats(g));
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream, h.gws, h.gws_floats);
     });
 }
 
