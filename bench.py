@@ -88,6 +88,7 @@ def algorithmic_work(B, L, H, E):
     # two products in one launch
     w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
     w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
+    w['dXout+dWout'] = ('mfma', 2 * outp[0], 2 * outp[1])
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

@@ -443,8 +443,10 @@ void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1,
             e1.bias = (const half_t*)addend1; e1.sbM = p1.sM; e1.sbN = p1.sN;
             for (int i = 0; i < 3; ++i) e1.sbb[i] = p1.sb[i];
         }
+        ensure_gws(h, h.gws_need);
         if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha, e1, p2.shape,
-                             (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream))
+                             (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream, h.gws,
+                             h.gws_floats))
             return;
         ps.cancel();
     }
@@ -882,8 +884,8 @@ void backward(Handle& h, const BwdPtrs& t) {
             op_baob(h, D[DATT], h.lb[DATT], DW[BO]);
         }
     }
-    run_gemm(h, G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout");
-    run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
+    run_gemm_pair(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout", nullptr,
+                  G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout", "dXout+dWout");
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
     AttnArgs at;

@@ -880,12 +880,13 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
 // that is instantiated; the caller then launches them one after the other.
 bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
-                      half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st) {
+                      half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws,
+                      size_t ws_floats) {
     static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
     if (off) return false;
     const GemmShape* sh[2] = {&s1, &s2};
     Canon c[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
-    bool akc[2], bkc[2];
+    bool akc[2], bkc[2], split_used = false;
     long n[2];
     for (int i = 0; i < 2; ++i) {
         const long batch = sh[i]->batch();
@@ -893,6 +894,11 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
         const GemmArgs& a = c[i].a;
         if (a.M % 128 || a.N % 128 || a.K1 % BK) return false;
         n[i] = (long)(a.M / 128) * (a.N / 128) * batch;
+        // a small output has its contraction split, as on its own (the scratch serves one product)
+        if (ws && !split_used && n[i] < 128 && (size_t)batch * a.M * a.N <= kSplitMaxOut) {
+            c[i].a.splits = pick_splits(a, batch, ws_floats);
+            if (c[i].a.splits > 1) { c[i].a.partial = ws; split_used = true; n[i] *= c[i].a.splits; }
+        }
         if (n[i] % 8 || n[i] < 128 || n[i] > 384) return false;
         if (pick_tile(a, batch, akc[i], bkc[i]) != 22) return false;
         if (akc[i] && bkc[i]) return false;                  // the asynchronous kernel's products stay on their own
@@ -907,6 +913,11 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
         hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
     else
         return false;
+    for (int i = 0; i < 2; ++i)
+        if (c[i].a.splits > 1) {
+            const long batch = sh[i]->batch(), nq = batch * (long)c[i].a.M * (c[i].a.N / 4);
+            hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, c[i].a, batch);
+        }
     check_launch("gemm pair");
     return true;
 }

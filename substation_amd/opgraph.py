@@ -43,6 +43,7 @@ OPERATORS = [
     ('blnrd2', 'bwd', ('DLN1', 'LN1STD', 'LN1DIFF', 'DROP1MASK', 'DRESID1', 'DATT')),
     ('baob', 'bwd', ('DATT',)),
     ('dWout', 'bwd', ('GAMMA', 'DATT', 'WO')),
+    ('dXout+dWout', 'bwd', ('WO', 'DATT', 'DGAMMA', 'GAMMA')),
     ('dXout', 'bwd', ('WO', 'DATT', 'DGAMMA')),
     ('attention-bwd-dQ', 'bwd', ('KKQQVV', 'GAMMA', 'DGAMMA', 'DATTN_DROP', 'ALPHA', 'ATTN_DROP_MASK', 'DBETA',
                                  'DKKQQVV')),
@@ -70,6 +71,7 @@ ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei'),
     ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
+    ('dXout+dWout', 'dXout', 'dWout'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
     ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT',
      'baib'),
