@@ -38,12 +38,11 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91468969, 'attention': 38114624, 'out': 33767823, 'bdrln1': 59013649,
-    'lin1': 88312974, 'bad': 134588115, 'lin2': 109257530, 'bdrln2': 59013979,
-    'bsb+blnrd1': 61022329, 'dXlin2': 84115472, 'dWlin2': 109267824, 'bdrlb': 135394553,
-    'dXlin1+dWlin1': 300850548, 'ebsb+blnrd2+baob': 79940110, 'dWout': 92474380, 'dWout split-k sum': 18967823,
-    'dXout': 33770072, 'attention-bwd-dQ': 55315548, 'attention-bwd-dKdV': 55518545, 'dXQKV-fused+dWQKV-fused': 279625554,
-    'column-sum finish': 7819467,
+    'QKV-fused': 91469396, 'attention': 38114651, 'out': 33767833, 'bdrln1': 59008298,
+    'lin1': 88318589, 'bad': 134560333, 'lin2': 109257624, 'bdrln2': 59011407,
+    'bsb+blnrd1': 61023201, 'dXlin2': 84115546, 'dWlin2': 109267917, 'bdrlb': 135394500,
+    'dXlin1+dWlin1': 301487462, 'ebsb+blnrd2+baob': 79940001, 'dXout+dWout': 121571707, 'dWout split-k sum': 18967830,
+    'attention-bwd-dQ': 55315255, 'attention-bwd-dKdV': 55518559, 'dXQKV-fused+dWQKV-fused': 287646007, 'column-sum finish': 7819470,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
