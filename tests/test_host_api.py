@@ -203,3 +203,22 @@ def test_reference_layout_literals_equal_the_shipped_pickles(name):
         assert [tuple(x) for x in got[key]] == [tuple(x) for x in want[key]] or tuple(got[key]) == tuple(want[key]), key
     assert got['special_dims'] == want['special_dims']
     assert got['algorithms'] == want['algorithms']
+
+
+def test_einsum_with_addend_rejects_an_addend_that_is_no_sub_block_of_the_output():
+    """sub_op_einsum_add checks the addend's layout on the host, before any launch:
+    its dims must be free or batch dims of the output, each merged group in one
+    dense run (the argument check of an epilogue addend; no GPU needed to fail)."""
+    h = _handle(2, 128, 2, 128)
+    lib = _lib.load()
+    one = ctypes.c_void_p(16)
+    s = lambda t: t.encode()
+    # U is not a dim of the output
+    rc = lib.sub_op_einsum_add(h.ptr, one, s('BJI'), one, s('HPI'), one, s('U'), one, s('BJHP'), 1.0)
+    assert rc < 0 and b'sub_op_einsum_add' in lib.sub_last_error()
+    # (H, P) merged in the output but transposed in the addend: not one stride
+    rc = lib.sub_op_einsum_add(h.ptr, one, s('BJI'), one, s('HPI'), one, s('PH'), one, s('BJHP'), 1.0)
+    assert rc < 0 and b'sub_op_einsum_add' in lib.sub_last_error()
+    # a null addend
+    rc = lib.sub_op_einsum_add(h.ptr, one, s('BJI'), one, s('HPI'), None, s('HP'), one, s('BJHP'), 1.0)
+    assert rc < 0 and b'null addend' in lib.sub_last_error()
