@@ -58,3 +58,25 @@ def test_k_remainder_and_tile_edges():
         o.einsum(to_layout(A, la, la), la, to_layout(Bm, lb, lb), lb, C, lc)
         torch.cuda.synchronize()
         assert_close(from_layout(C, lc, lc), want, name=f'{la},{lb}->{lc}')
+
+
+@pytest.mark.parametrize('E,H', [(192, 3), (64, 1), (128, 2)])
+def test_wide_tiles_every_operand_orientation(E, H):
+    """4096 x 4096 outputs take the 256 x 256 tiles of the asynchronous kernel with
+    eight waves: each operand k-contiguous or not, with an odd number of 64-deep
+    k-tiles (three, one) and an even one."""
+    from substation_amd.ops import Ops
+    o = Ops(8, 512, H, E, intermediate_size=4096)
+    sz = o.sizes
+    rng = np.random.default_rng(E)
+    for la in ('BJI', 'IBJ'):
+        for lb in ('UI', 'IU'):
+            lc = 'BJU'
+            A = h16(rng.normal(size=tuple(sz[d] for d in la)))
+            Bm = h16(rng.normal(size=tuple(sz[d] for d in lb)))
+            want = np.einsum(f'{la},{lb}->{lc}'.lower(), A, Bm)
+            C = torch.full(tuple(sz[d] for d in lc), float('nan'), dtype=torch.float16, device='cuda')
+            assert o.handle.classify(la, lb, lc)['kernel'] == 1
+            o.einsum(to_layout(A, la, la), la, to_layout(Bm, lb, lb), lb, C, lc)
+            torch.cuda.synchronize()
+            assert_close(from_layout(C, lc, lc), want, name=f'{la},{lb}->{lc} K={E}')
