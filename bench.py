@@ -186,6 +186,41 @@ def cpu_baseline(cfg, budget_s=20.0):
     }
 
 
+def bench_decoder(cfg, args):
+    """Forward + backward of substation_amd.DecoderLayer (substation/transformer.py:288-441), not the headline
+    metric: one JSON line of its own."""
+    import torch
+    from substation_amd import DecoderLayer
+    B, L, H, E = cfg['B'], cfg['L'], cfg['H'], cfg['E']
+    layer = DecoderLayer(B, L, L, H, E, 0.1, 0.1, 0.1, 0.1, activation=cfg.get('act', 'relu'), seed=0x5EED,
+                         intermediate_size=cfg.get('U')).cuda()
+    g = torch.Generator().manual_seed(1000 + args.config)
+    x = torch.randn(B, L, E, generator=g).half().cuda().requires_grad_(True)
+    enc_out = torch.randn(B, L, E, generator=g).half().cuda().requires_grad_(True)
+    dy = torch.randn(B, L, E, generator=g).half().cuda()
+    params = list(layer.parameters())
+
+    def step():
+        x.grad = None; enc_out.grad = None
+        for q in params:
+            q.grad = None
+        layer(x, enc_out).backward(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    print(json.dumps({'metric': 'fwd+bwd ms/decoder layer with encoder-decoder attention', 'value': round(ms, 4),
+                      'unit': 'ms', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                      'ms_per_step': round(ms, 4), 'higher_is_better': False, 'dtype': 'fp16', 'data': 'synthetic',
+                      'vs_baseline': None,
+                      'config': {'workload': f'decoder layer B={B} target=source={L} H={H} E={E} causal, 4 dropouts p=0.1'}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -202,6 +237,9 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE readings')
+    ap.add_argument('--decoder', action='store_true',
+                    help='time the decoder layer with encoder-decoder attention (both lengths = the '
+                         "configuration's L, causal self-attention) instead of the encoder layer; prints its own line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py: this build runs the encoder layer on ONE GPU only (no collectives exist on '
@@ -214,6 +252,9 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     cfg = CONFIGS[args.config]
+    if args.decoder:
+        bench_decoder(cfg, args)
+        return
     enc, X, DY = make_encoder(cfg, args.layouts)
     for item in args.option:
         k, v = item.split('=')
