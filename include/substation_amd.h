@@ -280,6 +280,20 @@ int sub_op_aib(void* handle, const void* in, const char* l_in, const void* bias,
                void* out, const char* l_out);
 /* block_baib.cuh:161-211, on the Q-stacked tensors */
 int sub_op_baib(void* handle, const void* d, const char* l_d, void* dbias, const char* l_dbias);
+/* The backward pass around one LayerNorm in one launch where the sizes and layouts
+ * allow (rows of up to 1024 contiguous features), else as the separate operators,
+ * with the same results.  extended = 0: block_bsb_ebsb.cuh:12-204 (bsb) followed
+ * by block_blnrd.cuh:14-259: g = dout1 * scale, dscale, dbias, then d_ln_in and
+ * d_drop_in from g.  extended = 1: block_bsb_ebsb.cuh:206-420 (ebsb: g =
+ * (dout1 + dout2) * scale, dlinear_bias = column sums of dlinear), blnrd, and
+ * block_baob.cuh:10-97 on d_drop_in (dout_bias).  Pass NULL for the tensors the
+ * plain form does not use. */
+int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l_in, const void* scale,
+                       const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                       const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
+                       const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
+                       const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                       const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias);
 /* block_bei.cuh:58-106 */
 int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void* dresid1,
                const char* l_dresid1, void* dx, const char* l_dx);

@@ -1317,6 +1317,31 @@ int sub_op_ebsb(void* handle, const void* in, const char* l_in, const void* scal
     });
 }
 
+int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l_in, const void* scale,
+                       const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                       const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
+                       const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
+                       const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                       const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        const bool ext = extended != 0;
+        if (ext && (!dout2 || !dlinear || !dlinear_bias || !dout_bias))
+            fail("sub_op_ln_backward: the extended form needs dout2, dlinear, dlinear_bias and dout_bias");
+        const Layout li = L(h, l_in), l1 = L(h, l_dout1), lis = L(h, l_istd), ldf = L(h, l_diff), lm = L(h, l_mask),
+                     lg = L(h, l_g), lo1 = L(h, l_d_ln_in), lo2 = L(h, l_d_drop_in);
+        const Layout l2 = ext ? L(h, l_dout2) : l1, ldl = ext ? L(h, l_dlinear) : l1;
+        if (op_lnbwd(h, ext, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, istd, lis, diff, ldf, mask, lm, g, lg,
+                     d_ln_in, lo1, d_drop_in, lo2, dscale, dbias, dlinear_bias, dout_bias))
+            return;
+        // shapes or layouts the one-launch form does not take: the separate operators, same results
+        if (ext) op_ebsb(h, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, g, lg, dscale, dbias, dlinear_bias);
+        else op_bsb(h, in, li, scale, dout1, l1, g, lg, dscale, dbias);
+        op_blnrd(h, g, lg, istd, lis, diff, ldf, mask, lm, d_ln_in, lo1, d_drop_in, lo2);
+        if (ext) op_baob(h, d_drop_in, lo2, dout_bias);
+    });
+}
+
 int sub_op_bdrlb(void* handle, const void* ddrop, const char* l_ddrop, const void* mask,
                  const char* l_mask, const void* lin, const char* l_lin, void* dlinear,
                  const char* l_dlinear, void* dbias) {

@@ -6,8 +6,8 @@ the encoder layer alone).  Here it runs on the device as a sequence of the
 library's operators -- the contraction kernel with bias and residual addends in
 its epilogue, the attention kernels that keep the scores in registers (with an
 additive mask for the self-attention and with a key length of their own for the
-attention over the encoder output), bdrln / bad and the LayerNorm- and
-dropout-backward operators -- in the order of the reference's statements.
+attention over the encoder output), bdrln / bad and the LayerNorm-backward
+operator -- in the order of the reference's statements.
 
 Argument and parameter names follow the reference's (``sattn_*``, ``edattn_*``,
 ``norm{1,2,3}_*``, ``linear{1,2}_*``).  The three self-attention projections are
@@ -166,8 +166,8 @@ def _make_function(m):
             g = {n: torch.empty_like(w[n]) for n in names}
             # norm3, residual, feed-forward                           transformer.py:371-395
             dln3, dres3, dff = e('BJI'), e('BJI'), e('BJI')
-            o.bsb(s['ln3'], 'BJI', w['norm3_scale'], dy, 'BJI', dln3, 'BJI', g['norm3_scale'], g['norm3_bias'])
-            o.blnrd(dln3, 'BJI', s['istd3'], 'BJ', s['diff3'], 'BJI', s['mask4'], 'BJI', dres3, 'BJI', dff, 'BJI')
+            o.ln_backward(s['ln3'], 'BJI', w['norm3_scale'], dy, 'BJI', s['istd3'], 'BJ', s['diff3'], 'BJI',
+                          s['mask4'], 'BJI', dln3, 'BJI', dres3, 'BJI', dff, 'BJI', g['norm3_scale'], g['norm3_bias'])
             dff1, dlin1 = e('BJU'), e('BJU')
             o.einsum(dff, 'BJI', w['linear2_w'], 'IU', dff1, 'BJU')
             o.einsum(dff, 'BJI', s['ff1'], 'BJU', g['linear2_w'], 'IU')
@@ -177,9 +177,10 @@ def _make_function(m):
             o.einsum(dlin1, 'BJU', s['normed2'], 'BJI', g['linear1_w'], 'UI')
             # norm2, residual, encoder-decoder attention              transformer.py:396-413
             dln2, dres2, datt2 = e('BJI'), e('BJI'), e('BJI')
-            o.ebsb(s['ln2'], 'BJI', w['norm2_scale'], dres3, 'BJI', dnormed2_linear, 'BJI', dff, 'BJI', dln2, 'BJI',
-                   g['norm2_scale'], g['norm2_bias'], g['linear2_b'])
-            o.blnrd(dln2, 'BJI', s['istd2'], 'BJ', s['diff2'], 'BJI', s['mask2'], 'BJI', dres2, 'BJI', datt2, 'BJI')
+            o.ln_backward(s['ln2'], 'BJI', w['norm2_scale'], dres3, 'BJI', s['istd2'], 'BJ', s['diff2'], 'BJI',
+                          s['mask2'], 'BJI', dln2, 'BJI', dres2, 'BJI', datt2, 'BJI', g['norm2_scale'], g['norm2_bias'],
+                          dout2=dnormed2_linear, l_dout2='BJI', dlinear=dff, l_dlinear='BJI',
+                          dlinear_bias=g['linear2_b'], dout_bias=g['edattn_out_b'])
             dgamma2 = e('BJHP')
             o.einsum(datt2, 'BJI', s['gamma2'], 'BJHP', g['edattn_wo'], 'IHP')
             o.einsum(w['edattn_wo'], 'IHP', datt2, 'BJI', dgamma2, 'BJHP')
@@ -199,10 +200,11 @@ def _make_function(m):
             os_.baob(dv2, 'BJI', g['edattn_in_b'][2])
             # norm1, residual, self-attention                         transformer.py:414-434
             dln1, dres1, datt1 = e('BJI'), e('BJI'), e('BJI')
-            o.ebsb(s['ln1'], 'BJI', w['norm1_scale'], dres2, 'BJI', dnormed1_attn, 'BJI', datt2, 'BJI', dln1, 'BJI',
-                   g['norm1_scale'], g['norm1_bias'], g['edattn_out_b'])
-            o.blnrd(dln1, 'BJI', s['istd1'], 'BJ', s['diff1'], 'BJI', s['mask1'], 'BJI', dres1, 'BJI', datt1, 'BJI')
-            o.baob(datt1, 'BJI', g['sattn_out_b'])
+            unused = torch.empty_like(g['sattn_out_b'])          # the column sums of the third input are not needed here
+            o.ln_backward(s['ln1'], 'BJI', w['norm1_scale'], dres2, 'BJI', s['istd1'], 'BJ', s['diff1'], 'BJI',
+                          s['mask1'], 'BJI', dln1, 'BJI', dres1, 'BJI', datt1, 'BJI', g['norm1_scale'], g['norm1_bias'],
+                          dout2=dnormed1_attn, l_dout2='BJI', dlinear=datt2, l_dlinear='BJI',
+                          dlinear_bias=unused, dout_bias=g['sattn_out_b'])
             dgamma1 = e('BJHP')
             o.einsum(datt1, 'BJI', s['gamma1'], 'BJHP', g['sattn_wo'], 'IHP')
             o.einsum(w['sattn_wo'], 'IHP', datt1, 'BJI', dgamma1, 'BJHP')

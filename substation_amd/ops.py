@@ -115,6 +115,18 @@ class Ops:
             _p(dlinear), _s(l_dlinear), _p(din), _s(l_din), _p(dscale), _p(dbias), _p(dlinear_bias)),
             'ebsb')
 
+    def ln_backward(self, inp, l_in, scale, dout1, l_dout1, istd, l_istd, diff, l_diff, mask, l_mask, g, l_g,
+                    d_ln_in, l_d_ln_in, d_drop_in, l_d_drop_in, dscale, dbias, dout2=None, l_dout2=None,
+                    dlinear=None, l_dlinear=None, dlinear_bias=None, dout_bias=None):
+        """bsb + blnrd, or with dout2 / dlinear / dlinear_bias / dout_bias given ebsb + blnrd + baob, in one
+        launch where the sizes and layouts allow."""
+        ext = dout2 is not None
+        _lib.check(self.lib.sub_op_ln_backward(
+            self._pre(), int(ext), _p(inp), _s(l_in), _p(scale), _p(dout1), _s(l_dout1), _p(dout2),
+            _s(l_dout2 or l_dout1), _p(dlinear), _s(l_dlinear or l_dout1), _p(istd), _s(l_istd), _p(diff), _s(l_diff),
+            _p(mask), _s(l_mask), _p(g), _s(l_g), _p(d_ln_in), _s(l_d_ln_in), _p(d_drop_in), _s(l_d_drop_in),
+            _p(dscale), _p(dbias), _p(dlinear_bias), _p(dout_bias)), 'ln_backward')
+
     def bdrlb(self, ddrop, l_ddrop, mask, l_mask, lin, l_lin, dlinear, l_dlinear, dbias):
         _lib.check(self.lib.sub_op_bdrlb(self._pre(), _p(ddrop), _s(l_ddrop), _p(mask), _s(l_mask),
                                          _p(lin), _s(l_lin), _p(dlinear), _s(l_dlinear), _p(dbias)),

@@ -303,3 +303,44 @@ def test_attention_operator_forward_and_backward(B, H, P, J, K, p, masked, l_q, 
     assert_close(from_layout(dq, 'BJHP', l_q), want_dq, name='dq')
     assert_close(from_layout(dk, 'BKHP', l_kv), want_dk, name='dk')
     assert_close(from_layout(dv, 'BKHP', l_kv), want_dv, name='dv')
+
+
+@pytest.mark.parametrize('B,L,H,E', [(2, 128, 4, 512), (4, 64, 1, 1024), (3, 24, 2, 48), (1, 4, 1, 4096)])
+@pytest.mark.parametrize('extended', [False, True])
+def test_ln_backward_one_launch_or_separate(B, L, H, E, extended):
+    """sub_op_ln_backward (bsb + blnrd, or ebsb + blnrd + baob) against the oracle's
+    operators, for sizes and layouts the one-launch kernel takes (rows of up to 1024
+    contiguous features) and for ones it hands to the separate operators."""
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(12)
+    g = lambda: h16(rng.normal(size=(B, L, E)))
+    normed, d1, d2, dl, diff = g(), g(), g(), g(), g()
+    istd = h16(1.0 + 0.2 * rng.random(size=(B, L)))
+    s = h16(1 + 0.1 * rng.normal(size=E))
+    mask = ph.dropout_mask((B, L, E), 0.3, SEED, ph.SITE_RESID1, step=0)
+    dev = lambda v: torch.from_numpy(np.asarray(v)).to(torch.float16).cuda()
+    vec = lambda: torch.empty(E, dtype=torch.float16, device='cuda')
+    for lay, lay2, lstd in (('BJI', 'BJI', 'BJ'), ('JBI', 'BJI', 'JB'), ('IBJ', 'JBI', 'BJ')):
+        gt, o1, o2 = o.empty(lay), o.empty(lay2), o.empty(lay)
+        ds, db, dlb, dob = vec(), vec(), vec(), vec()
+        kw = {}
+        if extended:
+            kw = dict(dout2=to_layout(d2, 'BJI', lay2), l_dout2=lay2, dlinear=to_layout(dl, 'BJI', lay), l_dlinear=lay,
+                      dlinear_bias=dlb, dout_bias=dob)
+        o.ln_backward(to_layout(normed, 'BJI', lay), lay, dev(s), to_layout(d1, 'BJI', lay2), lay2,
+                      to_layout(istd, 'BJ', lstd), lstd, to_layout(diff, 'BJI', lay2), lay2,
+                      to_layout(mask, 'BJI', lay), lay, gt, lay, o1, lay2, o2, lay, ds, db, **kw)
+        torch.cuda.synchronize()
+        if extended:
+            w = ref.op_ebsb(normed, s, d1, d2, dl)
+        else:
+            w = ref.op_bsb(normed, s, d1)
+        assert_close(from_layout(gt, 'BJI', lay), w[0], name='G')
+        assert_close(ds.float().cpu().numpy(), w[1], name='DSCALE', tol=2e-2)
+        assert_close(db.float().cpu().numpy(), w[2], name='DBIAS', tol=2e-2)
+        w1, w2 = ref.op_blnrd(from_layout(gt, 'BJI', lay), istd, diff, mask)      # from the device's rounded G
+        assert_close(from_layout(o1, 'BJI', lay2), w1, name='D_LN_IN')
+        assert_close(from_layout(o2, 'BJI', lay), w2, name='D_DROP_IN')
+        if extended:
+            assert_close(dlb.float().cpu().numpy(), w[3], name='DLINEAR_BIAS', tol=2e-2)
+            assert_close(dob.float().cpu().numpy(), ref.op_baob(from_layout(o2, 'BJI', lay)), name='DOUT_BIAS', tol=2e-2)
