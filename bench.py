@@ -49,9 +49,12 @@ GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin
             'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
 
 
-def algorithmic_work(B, L, H, E):
+def algorithmic_work(B, L, H, E, relu_from_output=True):
     """Per operator: ('hbm', bytes) or ('mfma', flops, bytes).  Bytes = each big
-    tensor read once + written once in fp16; flops = 2*batch*M*N*K."""
+    tensor read once + written once in fp16; flops = 2*batch*M*N*K.
+    relu_from_output: the ReLU layer as it runs by default -- bad writes only its
+    output (one [B,J,U] tensor in, one out) and bdrlb reads the gate off that output
+    (two in, one out); otherwise both move four."""
     U, P = 4 * E, E // H
     bji, bju, hbjk, q = B * L * E, B * L * U, H * B * L * L, 3 * B * L * E
     w = {
@@ -59,7 +62,8 @@ def algorithmic_work(B, L, H, E):
         'bdrln1': ('hbm', 7 * bji * 2), 'bdrln2': ('hbm', 7 * bji * 2),
         'blnrd1': ('hbm', 5 * bji * 2), 'blnrd2': ('hbm', 5 * bji * 2),
         'bsb': ('hbm', 3 * bji * 2), 'ebsb': ('hbm', 5 * bji * 2), 'baob': ('hbm', bji * 2),
-        'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', 4 * bju * 2), 'bdrlb': ('hbm', 4 * bju * 2),
+        'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', (2 if relu_from_output else 4) * bju * 2),
+        'bdrlb': ('hbm', (3 if relu_from_output else 4) * bju * 2),
         'baib': ('hbm', q * 2),
         # single-launch forms: the scaled gradient is written but not read back
         # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
@@ -301,7 +305,8 @@ def main():
         for n, ms in enc.profile():
             per_op.setdefault(n, []).append(ms)
     enc._handle.profile_enable(False)
-    work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'])
+    work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
+                            relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option)
     ops = []
     for n, ts in per_op.items():
         t = statistics.mean(ts) * 1e-3

@@ -185,6 +185,15 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * other waits.  Results are unchanged.  Profiling names: `dXlin1+dWlin1`,
  * `dXQKV-fused+dWQKV-fused`. */
 #define SUB_OPT_PAIR_PRODUCTS 5
+/* SUB_OPT_RELU_FROM_OUTPUT (default 1; ReLU layers only): the backward pass reads
+ * the gate of dropout and ReLU off the forward output DROP2 = relu(LIN1) * mask,
+ * which is positive exactly where the mask kept a positive LIN1
+ * (block_bdrlb.cuh:72 reads DROP2MASK and LIN1 for it).  encoder_forward then
+ * writes neither LIN1 nor DROP2MASK and encoder_backward reads neither: 64 MiB less
+ * traffic in each of the two launches at B=8, L=512, E=1024.  Outputs and gradients
+ * are bit-identical to those with the option off.  Set it to 0 before the forward
+ * call when LIN1 or DROP2MASK are wanted (debug capture). */
+#define SUB_OPT_RELU_FROM_OUTPUT 6
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

@@ -19,6 +19,7 @@ OPT_FUSE_LN_BACKWARD = 2
 OPT_FUSE_SCORES = 3
 OPT_FUSE_ATTENTION = 4
 OPT_PAIR_PRODUCTS = 5
+OPT_RELU_FROM_OUTPUT = 6
 FUSE_REQUIRED = 2
 
 

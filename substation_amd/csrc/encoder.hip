@@ -188,6 +188,7 @@ struct Handle {
     bool fuse_scores = true;
     int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
+    bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
 
@@ -511,12 +512,12 @@ void op_blnrd(Handle& h, const void* dout, const Layout& ldout, const void* istd
 
 void op_bad(Handle& h, const void* in, const Layout& lin_, const void* bias, void* lin,
             const Layout& llin, void* mask, const Layout& lmask, void* out, const Layout& lout,
-            float p, uint32_t site) {
+            float p, uint32_t site, bool out_only = false) {
     Space sp = make_space(h.sz, {dB, dJ}, dU);
     View vi = make_view(in, lin_, sp), vl = make_view(lin, llin, sp), vm = make_view(mask, lmask, sp),
          vo = make_view(out, lout, sp);
     flatten(sp.rs, {&vi, &vl, &vm, &vo});
-    launch_bad(sp.rs, vi, vector_view(bias, sp.rs.R), vl, vm, vo, h.act, make_key(h, site, p), h.stream);
+    launch_bad(sp.rs, vi, vector_view(bias, sp.rs.R), vl, vm, vo, h.act, make_key(h, site, p), h.stream, out_only);
 }
 
 void op_bsb(Handle& h, const void* in, const Layout& lin_, const void* scale, const void* dout,
@@ -547,6 +548,19 @@ void op_bdrlb(Handle& h, const void* ddrop, const Layout& ld, const void* mask, 
     launch_bdrlb(sp.rs, make_view(ddrop, ld, sp), make_view(mask, lm, sp), make_view(lin, ll, sp),
                  make_view(dlinear, lo, sp), ColOut{(half_t*)dbias}, h.act, ws, h.stream, defer_of(h));
 }
+
+// The ReLU layer's bdrlb with the gate taken from the forward output DROP2 = relu(LIN1) * mask, which is
+// positive exactly where the mask kept a positive LIN1 (block_bdrlb.cuh:72 reads the two separately).
+void op_bdrlb_from_output(Handle& h, const void* ddrop, const Layout& ld, const void* out, const Layout& lo_,
+                          void* dlinear, const Layout& lo, void* dbias) {
+    Space sp = make_space(h.sz, {dB, dJ}, dU);
+    float* ws = take_ws(h, colreduce_ws_floats(sp.rs, 1));
+    launch_bdrlb_from_output(sp.rs, make_view(ddrop, ld, sp), make_view(out, lo_, sp), make_view(dlinear, lo, sp),
+                             ColOut{(half_t*)dbias}, ws, h.stream, defer_of(h));
+}
+
+// Both passes decide this from the handle alone, so they agree.
+bool relu_from_output(const Handle& h) { return h.relu_from_output && h.act == ACT_RELU; }
 
 void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
@@ -800,7 +814,7 @@ void forward(Handle& h, const FwdPtrs& t) {
     {
         ProfScope ps(h, "bad");
         op_bad(h, F[SB1_LINW1], h.lf[SB1_LINW1], W[LINB1], F[LIN1], h.lf[LIN1], F[DROP2MASK],
-               h.lf[DROP2MASK], F[DROP2], h.lf[DROP2], h.p_act, SUB_SITE_ACT);
+               h.lf[DROP2MASK], F[DROP2], h.lf[DROP2], h.p_act, SUB_SITE_ACT, relu_from_output(h));
     }
     run_gemm(h, G_LIN2, F[DROP2], W[LINW2], F[DROP2_LINW2], "lin2");
     {
@@ -854,8 +868,11 @@ void backward(Handle& h, const BwdPtrs& t) {
     run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
     {
         ProfScope ps(h, "bdrlb");
-        op_bdrlb(h, D[DDROP2], h.lb[DDROP2], F[DROP2MASK], h.lf[DROP2MASK], F[LIN1], h.lf[LIN1],
-                 D[DLIN1], h.lb[DLIN1], DW[LINB1]);
+        if (relu_from_output(h))
+            op_bdrlb_from_output(h, D[DDROP2], h.lb[DDROP2], F[DROP2], h.lf[DROP2], D[DLIN1], h.lb[DLIN1], DW[LINB1]);
+        else
+            op_bdrlb(h, D[DDROP2], h.lb[DDROP2], F[DROP2MASK], h.lf[DROP2MASK], F[LIN1], h.lf[LIN1],
+                     D[DLIN1], h.lb[DLIN1], DW[LINB1]);
     }
     run_gemm_pair(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1", nullptr,
                   G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1", "dXlin1+dWlin1");
@@ -1117,6 +1134,7 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_FUSE_LN_BACKWARD) h.fuse_ln_backward = value != 0;
         else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
         else if (option == SUB_OPT_PAIR_PRODUCTS) h.pair_products = value != 0;
+        else if (option == SUB_OPT_RELU_FROM_OUTPUT) h.relu_from_output = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;

@@ -16,7 +16,7 @@ namespace {
 constexpr int BLOCK = 256;
 constexpr int WPB = BLOCK / WAVE;
 
-enum ColKind { COL_BSB, COL_EBSB, COL_BDRLB, COL_BAOB };
+enum ColKind { COL_BSB, COL_EBSB, COL_BDRLB, COL_BAOB, COL_BDRLB_OUT };
 
 struct ColArgs {
     View v[7];
@@ -28,6 +28,7 @@ template <> struct ColTraits<COL_BSB> { static constexpr int NS = 2; };
 template <> struct ColTraits<COL_EBSB> { static constexpr int NS = 3; };
 template <> struct ColTraits<COL_BDRLB> { static constexpr int NS = 1; };
 template <> struct ColTraits<COL_BAOB> { static constexpr int NS = 1; };
+template <> struct ColTraits<COL_BDRLB_OUT> { static constexpr int NS = 1; };
 
 __device__ __forceinline__ float gelu_grad(float x) {
     const float c = 0.7978845608028654f;
@@ -44,6 +45,8 @@ template <int KIND> struct ColIn;      // which views are read: count and indice
 template <> struct ColIn<COL_BSB> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; static constexpr bool nt[4] = {true, false, false, false}; };
 template <> struct ColIn<COL_EBSB> { static constexpr int N = 4; static constexpr int idx[4] = {0, 1, 2, 4}; static constexpr bool nt[4] = {true, true, false, true}; };
 template <> struct ColIn<COL_BDRLB> { static constexpr int N = 3; static constexpr int idx[4] = {0, 1, 2, 0}; static constexpr bool nt[4] = {true, true, true, false}; };
+// the ReLU gate read off the forward pass's output: DROP2 > 0 exactly where the mask kept a positive LIN1
+template <> struct ColIn<COL_BDRLB_OUT> { static constexpr int N = 2; static constexpr int idx[4] = {0, 1, 0, 0}; static constexpr bool nt[4] = {true, false, false, false}; };
 template <> struct ColIn<COL_BAOB> { static constexpr int N = 1; static constexpr int idx[4] = {0, 0, 0, 0}; static constexpr bool nt[4] = {false, false, false, false}; };
 
 // Raw 128-bit loads of the inputs of one row chunk (inputs T, T+1, ...).
@@ -94,6 +97,15 @@ __device__ __forceinline__ void col_compute(const ColArgs& a, const RowIdx& ix, 
             float g = a.act == ACT_GELU ? gelu_grad(in[2].v[i]) * d : (in[2].v[i] > 0.f ? d : 0.f);
             oh[i] = (half_t)g;
         }
+        oh = pin(oh);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[0][i] += i < nv ? (float)oh[i] : 0.f;
+        store8h(a.v[3], view_offset(a.v[3], ix), e0, nv, oh);
+    } else if (KIND == COL_BDRLB_OUT) {
+        // in0 DDROP, in1 DROP2 (= relu(LIN1) * mask) -> DLINEAR
+        h8 oh;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) oh[i] = (half_t)(in[1].v[i] > 0.f ? in[0].v[i] : 0.f);
         oh = pin(oh);
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[0][i] += i < nv ? (float)oh[i] : 0.f;
@@ -343,6 +355,13 @@ void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlin
     ColArgs a{}; a.v[0] = ddrop; a.v[1] = mask; a.v[2] = lin; a.v[3] = dlinear; a.act = act;
     FinishArgs fo{{dbias.p, nullptr, nullptr}, 0, 0, 1, 1};
     run_col<COL_BDRLB>(rs, a, fo, ws, st, "backward dropout-activation-bias", defer);
+}
+
+void launch_bdrlb_from_output(const RowSpace& rs, View ddrop, View out, View dlinear, ColOut dbias, float* ws,
+                              hipStream_t st, FinishJobs* defer) {
+    ColArgs a{}; a.v[0] = ddrop; a.v[1] = out; a.v[3] = dlinear; a.act = 0;
+    FinishArgs fo{{dbias.p, nullptr, nullptr}, 0, 0, 1, 1};
+    run_col<COL_BDRLB_OUT>(rs, a, fo, ws, st, "backward dropout-relu-bias", defer);
 }
 
 void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st, FinishJobs* defer) {

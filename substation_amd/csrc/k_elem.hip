@@ -39,7 +39,7 @@ __device__ __forceinline__ Chunk chunk_of(const RowSpace& rs, unsigned idx, unsi
 template <bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, View lin, View mask,
                                                View out, int act, PhiloxKey key_, unsigned nchunks,
-                                               unsigned cpr) {
+                                               unsigned cpr, int out_only) {
     const PhiloxKey key = resolved(key_);
     const unsigned stride = gridDim.x * BLOCK;
     for (unsigned base = blockIdx.x * BLOCK + threadIdx.x; base < nchunks; base += stride * UNROLL) {
@@ -65,8 +65,10 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
                 float a = act == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
                 oh[i] = ((bits >> i) & 1u) ? (half_t)a : (half_t)0.0f;
             }
-            st8h<FAST, true>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
-            st8h<FAST, true>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
+            if (!out_only) {
+                st8h<FAST, true>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
+                st8h<FAST, true>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
+            }
             st8h<FAST>(out, view_offset(out, c[u].ix), c[u].e0, c[u].nv, oh);
         }
     }
@@ -112,17 +114,17 @@ inline unsigned check_chunks(long nchunks, const char* what) {
 }  // namespace
 
 void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, View out, int act,
-                PhiloxKey key, hipStream_t st) {
+                PhiloxKey key, hipStream_t st, bool out_only) {
     unsigned cpr = (unsigned)((rs.R + 7) / 8);
     unsigned nchunks = check_chunks(rs.rows() * cpr, "bias-activation-dropout");
     if (nchunks == 0) return;
     const bool fast = in.vec && bias.vec && lin.vec && mask.vec && out.vec;
     if (fast)
         hipLaunchKernelGGL(k_bad<true>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
-                           mask, out, act, key, nchunks, cpr);
+                           mask, out, act, key, nchunks, cpr, out_only ? 1 : 0);
     else
         hipLaunchKernelGGL(k_bad<false>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
-                           mask, out, act, key, nchunks, cpr);
+                           mask, out, act, key, nchunks, cpr, out_only ? 1 : 0);
     check_launch("bias-activation-dropout");
 }
 

@@ -28,8 +28,9 @@ void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask
                   View d_drop_in, hipStream_t st);
 
 // --- elementwise operators ---------------------------------------------------
+// out_only: neither LIN (input + bias) nor the mask is written, only the output
 void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, View out, int act,
-                PhiloxKey key, hipStream_t st);
+                PhiloxKey key, hipStream_t st, bool out_only = false);
 // out = a + b (b may be a broadcast view): bei, aib
 void launch_add(const RowSpace& rs, View a, View b, View out, hipStream_t st);
 
@@ -67,6 +68,10 @@ void launch_ebsb(const RowSpace& rs, View in, View dout1, View dout2, View dline
                  hipStream_t st, FinishJobs* defer = nullptr);
 void launch_bdrlb(const RowSpace& rs, View ddrop, View mask, View lin, View dlinear, ColOut dbias,
                   int act, float* ws, hipStream_t st, FinishJobs* defer = nullptr);
+// bdrlb for ReLU with the gate read off the forward pass's output (out > 0 exactly where the
+// mask kept a positive pre-activation): neither the mask nor LIN is read
+void launch_bdrlb_from_output(const RowSpace& rs, View ddrop, View out, View dlinear, ColOut dbias, float* ws,
+                              hipStream_t st, FinishJobs* defer = nullptr);
 void launch_baob(const RowSpace& rs, View datt, ColOut dbo, float* ws, hipStream_t st,
                  FinishJobs* defer = nullptr);
 // out[i0,i1,e] = sum over (i2,i3) of d; out strides ob0, ob1 (kept dims) and of.

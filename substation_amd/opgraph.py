@@ -33,7 +33,7 @@ OPERATORS = [
     ('blnrd1', 'bwd', ('DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
     ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
     ('dWlin2', 'bwd', ('DLIN2', 'DROP2', 'LINW2')),
-    ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DLIN1')),
+    ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DROP2', 'DLIN1')),      # ReLU: the gate is read off DROP2
     ('dXlin1+dWlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1', 'SB1')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
     ('dWlin1', 'bwd', ('DLIN1', 'SB1', 'LINW1')),

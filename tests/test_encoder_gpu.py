@@ -460,6 +460,39 @@ def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback()
         enc(X)
 
 
+@pytest.mark.parametrize('dims', [(2, 256, 4, 256), (8, 512, 16, 1024)])
+def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
+    """ReLU layers (the default of the module, as in the reference) read the gate
+    of dropout and ReLU in the backward pass off DROP2 = relu(LIN1) * mask, which
+    is positive exactly where the mask kept a positive LIN1; LIN1 and DROP2MASK are
+    then neither written nor read.  Output and every gradient must equal, bit for
+    bit, those with the option off (block_bdrlb.cuh:72: gate from DROP2MASK and
+    LIN1), and the two tensors must really be left alone."""
+    from substation_amd import Encoder, layouts as L
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = dims
+    outs = []
+    for from_output in (0, 1):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED).cuda()
+        enc._handle.set_option(6, from_output)
+        enc.set_rng(SEED, 0)
+        g = torch.Generator().manual_seed(5)
+        X = (0.5 * torch.randn(B, Ls, E, generator=g)).half().cuda().requires_grad_(True)
+        DY = torch.randn(B, Ls, E, generator=g).half().cuda()
+        with torch.no_grad():
+            for q in enc.parameters():
+                q.mul_(0.1)
+        Y = enc(X)
+        Y.backward(DY)
+        torch.cuda.synchronize()
+        outs.append([Y.detach().clone(), X.grad.clone()] + [q.grad.clone() for q in enc.parameters()])
+    for a, b in zip(*outs):
+        assert torch.isfinite(a.float()).all()
+        assert torch.equal(a, b)
+    assert float(outs[0][1].abs().max()) > 0
+
+
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
     """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
     the library's one-time allocations) and replayed with eager work in between:
