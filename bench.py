@@ -38,11 +38,11 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91469396, 'attention': 38114651, 'out': 33767833, 'bdrln1': 59008298,
-    'lin1': 88318589, 'bad': 134560333, 'lin2': 109257624, 'bdrln2': 59011407,
-    'bsb+blnrd1': 61023201, 'dXlin2': 84115546, 'dWlin2': 109267917, 'bdrlb': 135394500,
-    'dXlin1+dWlin1': 301487462, 'ebsb+blnrd2+baob': 79940001, 'dXout+dWout': 121571707, 'dWout split-k sum': 18967830,
-    'attention-bwd-dQ': 55315255, 'attention-bwd-dKdV': 55518559, 'dXQKV-fused+dWQKV-fused': 287646007, 'column-sum finish': 7819470,
+    'QKV-fused': 91469343, 'attention': 38114651, 'out': 33767869, 'bdrln1': 59008853,
+    'lin1': 88315355, 'bad': 67316332, 'lin2': 109257713, 'bdrln2': 59011779,
+    'bsb+blnrd1': 61022518, 'dXlin2': 84115563, 'dWlin2': 109268080, 'bdrlb': 101781592,
+    'dXlin1+dWlin1': 300874502, 'ebsb+blnrd2+baob': 79940530, 'dXout+dWout': 120659452, 'dWout split-k sum': 18967854,
+    'attention-bwd-dQ': 55315797, 'attention-bwd-dKdV': 55518614, 'dXQKV-fused+dWQKV-fused': 288128157, 'column-sum finish': 7831768,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
