@@ -92,6 +92,8 @@ def algorithmic_work(B, L, H, E, relu_from_output=True):
     w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
     w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
     w['dXout+dWout'] = ('mfma', 2 * outp[0], 2 * outp[1])
+    # lin1 with bias, ReLU and dropout in its epilogue: the product's flops, SB1 and LINW1 in, DROP2 out
+    w['lin1+bad'] = ('mfma',) + ffn
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

@@ -191,8 +191,11 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * (block_bdrlb.cuh:72 reads DROP2MASK and LIN1 for it).  encoder_forward then
  * writes neither LIN1 nor DROP2MASK and encoder_backward reads neither: 64 MiB less
  * traffic in each of the two launches at B=8, L=512, E=1024.  Outputs and gradients
- * are bit-identical to those with the option off.  Set it to 0 before the forward
- * call when LIN1 or DROP2MASK are wanted (debug capture). */
+ * are bit-identical to those with the option off.  With SUB_OPT_FUSE_EPILOGUES on
+ * and DROP2 in BJU order, bias, ReLU and dropout then run in the epilogue of the
+ * lin1 product (profiling name `lin1+bad`) and SB1_LINW1 is not written either.
+ * Set it to 0 before the forward call when LIN1, DROP2MASK or SB1_LINW1 are
+ * wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers

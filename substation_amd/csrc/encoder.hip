@@ -150,7 +150,7 @@ struct GemmPlan {
 // G_QKV_BIAS: QKV projection writing KKQQVV directly with BKQV added in the
 // epilogue (replaces QKV-fused + aib).  G_DXQKV_RESID: input-gradient projection
 // writing DX directly with DRESID1 added (replaces dXQKV-fused + bei).
-enum G { G_QKV_BIAS, G_DXQKV_RESID, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
+enum G { G_QKV_BIAS, G_DXQKV_RESID, G_LIN1_BAD, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
          G_DWOUT, G_DXOUT, G_DX1GAMMA, G_DX2GAMMA, G_DX1QKT, G_DX2QKT, G_DXQKV, G_DWQKV, G_COUNT };
 
 struct ProfEntry { const char* name; hipEvent_t a, b; };
@@ -375,6 +375,15 @@ void configure(Handle& h, const sub_config* c) {
     };
     plan_fused(G_QKV_BIAS, h.lX, h.lp[WKQV], h.lf[KKQQVV], h.lp[BKQV]);
     plan_fused(G_DXQKV_RESID, h.lp[WKQV], h.lb[DKKQQVV], h.lX, h.lb[DRESID1]);
+    // lin1 with LINB1, ReLU and dropout in its epilogue (writes DROP2; SB1_LINW1 is not produced): DROP2 must be
+    // dense in canonical order, since the keep bits are indexed by the canonical element index
+    plan_fused(G_LIN1_BAD, h.lf[SB1], h.lp[LINW1], h.lf[DROP2], h.lp[LINB1]);
+    if (h.gemm[G_LIN1_BAD].ok) {
+        GemmPlan& p = h.gemm[G_LIN1_BAD];
+        GemmEpilogue ep; ep.bias = (const half_t*)16; ep.sbM = p.sM; ep.sbN = p.sN; ep.relu_dropout = true;
+        p.ok = h.lf[DROP2].str() == "BJU" &&
+               gemm_relu_dropout_ok(p.shape, (const void*)16, (const void*)16, (const void*)16, ep);
+    }
 
     {   // scratch of the five column reductions of one backward pass, side by side
         Space si = make_space(sz, {dB, dJ}, dI), su = make_space(sz, {dB, dJ}, dU);
@@ -810,11 +819,22 @@ void forward(Handle& h, const FwdPtrs& t) {
                  F[DROP1MASK], h.lf[DROP1MASK], F[LN1DIFF], h.lf[LN1DIFF], F[LN1], h.lf[LN1],
                  F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1);
     }
+    if (relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok && aligned16(W[LINB1]) && aligned16(F[DROP2]) &&
+        aligned16(F[SB1]) && aligned16(W[LINW1])) {
+        // product, bias, ReLU and dropout in one launch: SB1_LINW1 (and LIN1, DROP2MASK) are not produced
+        ProfScope ps(h, "lin1+bad");
+        const GemmPlan& p = h.gemm[G_LIN1_BAD];
+        GemmEpilogue ep;
+        ep.bias = (const half_t*)W[LINB1]; ep.sbM = p.sM; ep.sbN = p.sN;
+        ep.relu_dropout = true; ep.key = make_key(h, SUB_SITE_ACT, h.p_act);
+        launch_gemm(p.shape, (const half_t*)F[SB1], (const half_t*)W[LINW1], (half_t*)F[DROP2], p.alpha, ep, h.stream);
+    } else {
     run_gemm(h, G_LIN1, F[SB1], W[LINW1], F[SB1_LINW1], "lin1");
     {
         ProfScope ps(h, "bad");
         op_bad(h, F[SB1_LINW1], h.lf[SB1_LINW1], W[LINB1], F[LIN1], h.lf[LIN1], F[DROP2MASK],
                h.lf[DROP2MASK], F[DROP2], h.lf[DROP2], h.p_act, SUB_SITE_ACT, relu_from_output(h));
+    }
     }
     run_gemm(h, G_LIN2, F[DROP2], W[LINW2], F[DROP2_LINW2], "lin2");
     {

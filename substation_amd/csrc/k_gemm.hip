@@ -33,6 +33,8 @@ struct GemmArgs {
     const half_t* bias; long sbM, sbN, sbb[3];
     int splits;                   // > 1: the k range is split, fp32 partial tiles go to `partial`
     float* partial;               // [split][batch][M][N]
+    int relu_dropout = 0;         // epilogue of the asynchronous kernel: ReLU and dropout after the addend
+    PhiloxKey key;
 };
 
 // ---------------------------------------------------------------------------
@@ -650,6 +652,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     __syncthreads();
 
     half_t* stage = st0 + wave * STAGE_WAVE;
+    PhiloxKey rd_key = g.key;
+    if (g.relu_dropout) rd_key = resolved(g.key);
     half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
     const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
     constexpr int LPR = 4 * TN;
@@ -676,6 +680,14 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                 h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
+            }
+            if (g.relu_dropout) {
+                // what the bias-activation-dropout operator does to the rounded sum, with the
+                // same keep bits (the element index is the offset into the dense output)
+                const uint32_t bits = keep_bits8(rd_key, (uint64_t)mm * (uint64_t)g.sCM + (uint64_t)nn);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    val[e] = ((bits >> e) & 1u) ? (half_t)fmaxf((float)val[e], 0.f) : (half_t)0.0f;
             }
             *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
         }
@@ -745,6 +757,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     a.nb1 = (int)s.nb[1]; a.nb2 = (int)s.nb[2];
     for (int i = 0; i < 3; ++i) { a.sCb[i] = s.sCb[i]; a.sbb[i] = ep.sbb[i]; }
     a.alpha = alpha; a.bias = ep.bias;
+    a.relu_dropout = ep.relu_dropout ? 1 : 0; a.key = ep.key;
     a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;
@@ -863,6 +876,14 @@ int gemm_kernel_kind(const GemmShape& s, const void* A, const void* B, const voi
     return pick_kind(c, akc, bkc);
 }
 
+bool gemm_relu_dropout_ok(const GemmShape& s, const void* A, const void* B, const void* C,
+                          const GemmEpilogue& ep) {
+    if (s.batch() != 1 || s.sCN != 1 || s.sCM != s.N) return false;       // one dense row-major output
+    Canon c = canonicalise(s, (const half_t*)A, (const half_t*)B, (half_t*)C, 1.f, ep);
+    bool akc, bkc;
+    return pick_kind(c, akc, bkc) == 1 && pick_tile(c.a, 1, akc, bkc) == 44;
+}
+
 size_t gemm_splitk_ws_floats(const GemmShape& s) {
     // only small outputs are split (measured: beyond ~2M elements the fp32 partial
     // traffic costs more than the extra workgroups gain)
@@ -941,12 +962,15 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             c.a.partial = ws;
         }
         const int tile = force ? force : pick_tile(c.a, batch, akc, bkc);
+        if (ep.relu_dropout && (tile != 44 || batch != 1 || s.sCN != 1 || s.sCM != s.N))
+            fail("gemm: the ReLU-dropout epilogue needs the 256x256 asynchronous kernel (see gemm_relu_dropout_ok)");
         const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
         if (tile == 44) launch_mfma<4, 4, true>(c.a, akc, bkc, batch, true, st);
         else if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
         else if (tile == 21) launch_mfma<2, 1, false>(c.a, akc, bkc, batch, false, st);
         else launch_mfma<2, 2, true>(c.a, akc, bkc, batch, dma, st);
     } else {
+        if (ep.relu_dropout) fail("gemm: the ReLU-dropout epilogue needs the MFMA kernel");
         long total = batch * (long)c.a.M * c.a.N;
         long blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffL) fail("gemm: problem too large for the scalar kernel");

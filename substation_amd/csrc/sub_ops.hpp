@@ -163,11 +163,18 @@ struct GemmEpilogue {
     const half_t* bias = nullptr;
     int64_t sbM = 0, sbN = 0;       // addend strides along M and N
     int64_t sbb[3] = {0, 0, 0};     // and along the batch dims
+    // after the addend: out = keep ? max(x, 0) : 0 with the keep bits of `key`, the element
+    // index being the offset into C (C dense in canonical order).  See gemm_relu_dropout_ok.
+    bool relu_dropout = false;
+    PhiloxKey key;
 };
 // `ws` (optional): fp32 scratch of ws_floats elements for splitting the
 // contraction of small-output products across workgroups.
 void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C, float alpha,
                  const GemmEpilogue& ep, hipStream_t st, float* ws = nullptr, size_t ws_floats = 0);
+// Can launch_gemm apply ep.relu_dropout to this product?  Only the asynchronous kernel with
+// 256x256 tiles does, on a single dense row-major output.
+bool gemm_relu_dropout_ok(const GemmShape& g, const void* A, const void* B, const void* C, const GemmEpilogue& ep);
 // Two independent contractions in one launch, their workgroups interleaved so that
 // every CU works on both at once.  Returns false, having launched nothing, when
 // the pair does not qualify (then call launch_gemm for each).

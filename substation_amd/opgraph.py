@@ -25,6 +25,7 @@ OPERATORS = [
     ('out', 'fwd', ('WO', 'GAMMA', 'ATT')),
     ('bdrln1', 'fwd', ('ATT', 'X', 'DROP1MASK', 'LN1DIFF', 'LN1', 'SB1', 'LN1STD')),
     ('lin1', 'fwd', ('SB1', 'LINW1', 'SB1_LINW1')),
+    ('lin1+bad', 'fwd', ('SB1', 'LINW1', 'DROP2')),
     ('bad', 'fwd', ('SB1_LINW1', 'LIN1', 'DROP2MASK', 'DROP2')),
     ('lin2', 'fwd', ('DROP2', 'LINW2', 'DROP2_LINW2')),
     ('bdrln2', 'fwd', ('DROP2_LINW2', 'SB1', 'LIN2', 'DROP3MASK', 'LN2DIFF', 'LN2', 'SB2', 'LN2STD')),
@@ -70,6 +71,7 @@ OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei'),
+    ('lin1+bad', 'lin1', 'bad'),
     ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
     ('dXout+dWout', 'dXout', 'dWout'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
