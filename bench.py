@@ -94,6 +94,7 @@ def algorithmic_work(B, L, H, E, relu_from_output=True):
     w['dXout+dWout'] = ('mfma', 2 * outp[0], 2 * outp[1])
     # lin1 with bias, ReLU and dropout in its epilogue: the product's flops, SB1 and LINW1 in, DROP2 out
     w['lin1+bad'] = ('mfma',) + ffn
+    w['dXlin2+bdrlb'] = ('mfma', ffn[0], ffn[1] + 2 * tok * U)      # the product's bytes plus the gate (DROP2) read
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

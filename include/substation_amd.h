@@ -193,7 +193,10 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * traffic in each of the two launches at B=8, L=512, E=1024.  Outputs and gradients
  * are bit-identical to those with the option off.  With SUB_OPT_FUSE_EPILOGUES on
  * and DROP2 in BJU order, bias, ReLU and dropout then run in the epilogue of the
- * lin1 product (profiling name `lin1+bad`) and SB1_LINW1 is not written either.
+ * lin1 product (profiling name `lin1+bad`) and SB1_LINW1 is not written either;
+ * in encoder_backward bdrlb runs in the epilogue of the dXlin2 product
+ * (`dXlin2+bdrlb`), DDROP2 is not written and DLINB1 sums its terms in another
+ * order.
  * Set it to 0 before the forward call when LIN1, DROP2MASK or SB1_LINW1 are
  * wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6

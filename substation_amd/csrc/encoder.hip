@@ -150,7 +150,7 @@ struct GemmPlan {
 // G_QKV_BIAS: QKV projection writing KKQQVV directly with BKQV added in the
 // epilogue (replaces QKV-fused + aib).  G_DXQKV_RESID: input-gradient projection
 // writing DX directly with DRESID1 added (replaces dXQKV-fused + bei).
-enum G { G_QKV_BIAS, G_DXQKV_RESID, G_LIN1_BAD, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
+enum G { G_QKV_BIAS, G_DXQKV_RESID, G_LIN1_BAD, G_DXLIN2_BDRLB, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
          G_DWOUT, G_DXOUT, G_DX1GAMMA, G_DX2GAMMA, G_DX1QKT, G_DX2QKT, G_DXQKV, G_DWQKV, G_COUNT };
 
 struct ProfEntry { const char* name; hipEvent_t a, b; };
@@ -385,6 +385,15 @@ void configure(Handle& h, const sub_config* c) {
                gemm_relu_dropout_ok(p.shape, (const void*)16, (const void*)16, (const void*)16, ep);
     }
 
+    // dXlin2 with the ReLU layer's bdrlb in its epilogue (gate read off DROP2, writes DLIN1 and partial column sums for
+    // DLINB1; DDROP2 is not produced)
+    plan_fused(G_DXLIN2_BDRLB, h.lb[DLIN2], h.lp[LINW2], h.lb[DLIN1], h.lf[DROP2]);
+    if (h.gemm[G_DXLIN2_BDRLB].ok) {
+        GemmPlan& p = h.gemm[G_DXLIN2_BDRLB];
+        GemmEpilogue ep; ep.gate = (const half_t*)16; ep.colsum = (float*)16; ep.sbM = p.sM; ep.sbN = p.sN;
+        p.ok = p.sb[0] == 0 && gemm_relu_dropout_ok(p.shape, (const void*)16, (const void*)16, (const void*)16, ep);
+    }
+
     {   // scratch of the five column reductions of one backward pass, side by side
         Space si = make_space(sz, {dB, dJ}, dI), su = make_space(sz, {dB, dJ}, dU);
         Space sq = make_space(sz, {dQ, dH, dB, dJ}, dP);
@@ -401,6 +410,8 @@ void configure(Handle& h, const sub_config* c) {
         // the attention kernels' partial sums for the projection-bias gradient stand in for baib's
         const size_t attn_bias = (size_t)(3 * sz.n[dH] * sz.n[dB] * ((sz.n[dJ] + 127) / 128) * sz.n[dP]);
         if (attn_bias > (baib > baib2 ? baib : baib2)) h.ws_need_bwd += attn_bias;
+        // the partial column sums of dXlin2's epilogue (one row per 128 tokens)
+        h.ws_need_bwd += (size_t)((sz.n[dB] * sz.n[dJ] + 127) / 128) * sz.n[dU] + 64;
     }
     h.gws_need = 0;
     for (int i = 0; i < G_COUNT; ++i) {
@@ -884,9 +895,30 @@ void backward(Handle& h, const BwdPtrs& t) {
                      F[DROP3MASK], h.lf[DROP3MASK], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2]);
         }
     }
-    run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
+    const bool fuse_bdrlb = relu_from_output(h) && h.fuse_epilogues && h.gemm[G_DXLIN2_BDRLB].ok && aligned16(F[DROP2]) &&
+                            aligned16(D[DLIN1]) && aligned16(D[DLIN2]) && aligned16(W[LINW2]);
+    if (fuse_bdrlb) {
+        // product, gate and the column sums of the result in one launch: DDROP2 is not produced
+        ProfScope ps(h, "dXlin2+bdrlb");
+        const GemmPlan& p = h.gemm[G_DXLIN2_BDRLB];
+        const int ntc = (int)(p.shape.M / 128), U = (int)p.shape.N;
+        float* ws = take_ws(h, (size_t)ntc * U);
+        GemmEpilogue ep;
+        ep.gate = (const half_t*)F[DROP2]; ep.sbM = p.sM; ep.sbN = p.sN; ep.colsum = ws;
+        launch_gemm(p.shape, (const half_t*)D[DLIN2], (const half_t*)W[LINW2], (half_t*)D[DLIN1], p.alpha, ep, h.stream);
+        FinishJob job{ws, FinishArgs{{(half_t*)DW[LINB1], nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};
+        if (h.deferring) {
+            if (h.deferred.n >= kMaxFinishJobs) fail("encoder_backward: too many deferred reductions");
+            h.deferred.j[h.deferred.n++] = job;
+        } else {
+            FinishJobs one; one.n = 1; one.j[0] = job;
+            launch_colfinish(one, h.stream);
+        }
+    } else {
+        run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
+    }
     run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
-    {
+    if (!fuse_bdrlb) {
         ProfScope ps(h, "bdrlb");
         if (relu_from_output(h))
             op_bdrlb_from_output(h, D[DDROP2], h.lb[DDROP2], F[DROP2], h.lf[DROP2], D[DLIN1], h.lb[DLIN1], DW[LINB1]);

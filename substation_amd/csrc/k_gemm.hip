@@ -35,6 +35,8 @@ struct GemmArgs {
     float* partial;               // [split][batch][M][N]
     int relu_dropout = 0;         // epilogue of the asynchronous kernel: ReLU and dropout after the addend
     PhiloxKey key;
+    const half_t* gate = nullptr; // or: zero where gate <= 0 (strides of `bias`), column sums per 128-row slab
+    float* colsum = nullptr;
 };
 
 // ---------------------------------------------------------------------------
@@ -654,6 +656,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     half_t* stage = st0 + wave * STAGE_WAVE;
     PhiloxKey rd_key = g.key;
     if (g.relu_dropout) rd_key = resolved(g.key);
+    float colsum[8];              // gate mode: this lane's 8 columns summed over its rows of the wave's slab
+#pragma unroll
+    for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
     half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
     const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
     constexpr int LPR = 4 * TN;
@@ -681,6 +686,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
             }
+            if (g.gate) {
+                // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
+                const h8 gt = *reinterpret_cast<const h8*>(g.gate + (long)mm * g.sbM + nn);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    val[e] = (float)gt[e] > 0.f ? val[e] : (half_t)0.0f;
+                    colsum[e] += (float)val[e];
+                }
+            }
             if (g.relu_dropout) {
                 // what the bias-activation-dropout operator does to the rounded sum, with the
                 // same keep bits (the element index is the offset into the dense output)
@@ -690,6 +704,19 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                     val[e] = ((bits >> e) & 1u) ? (half_t)fmaxf((float)val[e], 0.f) : (half_t)0.0f;
             }
             *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
+        }
+    }
+    if (g.gate) {
+        // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
+        // row of partial sums per 128-row slab of the output (a finishing launch adds the slabs)
+#pragma unroll
+        for (int o = LPR; o < 64; o <<= 1)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) colsum[e] += __shfl_xor(colsum[e], o);
+        if (lane < LPR) {
+            float* dst = g.colsum + ((long)tile_m * 2 + wm) * g.N + n0 + wn * 32 * TN + lane * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) dst[e] = colsum[e];
         }
     }
 }
@@ -758,6 +785,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     for (int i = 0; i < 3; ++i) { a.sCb[i] = s.sCb[i]; a.sbb[i] = ep.sbb[i]; }
     a.alpha = alpha; a.bias = ep.bias;
     a.relu_dropout = ep.relu_dropout ? 1 : 0; a.key = ep.key;
+    a.gate = ep.gate; a.colsum = ep.colsum;
     a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;
@@ -776,6 +804,7 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     if (a.bias && !(a.sbN == 1 && mult8(a.sbM) && mult8(a.sbb[0]) && mult8(a.sbb[1]) && mult8(a.sbb[2]) &&
                     al16(a.bias)))
         return 0;
+    if (a.gate && !(a.sbN == 1 && mult8(a.sbM) && al16(a.gate) && !a.bias && a.colsum)) return 0;
     // every 16-byte access must be aligned and whole
     bool ok = mult8(a.N) && mult8(a.sCM) && mult8(a.sCb[0]) && mult8(a.sCb[1]) && mult8(a.sCb[2]);
     ok = ok && mult8(a.sAK0) && mult8(a.sAb[0]) && mult8(a.sAb[1]) && mult8(a.sAb[2]);
@@ -962,7 +991,7 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             c.a.partial = ws;
         }
         const int tile = force ? force : pick_tile(c.a, batch, akc, bkc);
-        if (ep.relu_dropout && (tile != 44 || batch != 1 || s.sCN != 1 || s.sCM != s.N))
+        if ((ep.relu_dropout || ep.gate) && (tile != 44 || batch != 1 || s.sCN != 1 || s.sCM != s.N))
             fail("gemm: the ReLU-dropout epilogue needs the 256x256 asynchronous kernel (see gemm_relu_dropout_ok)");
         const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
         if (tile == 44) launch_mfma<4, 4, true>(c.a, akc, bkc, batch, true, st);
@@ -970,7 +999,7 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
         else if (tile == 21) launch_mfma<2, 1, false>(c.a, akc, bkc, batch, false, st);
         else launch_mfma<2, 2, true>(c.a, akc, bkc, batch, dma, st);
     } else {
-        if (ep.relu_dropout) fail("gemm: the ReLU-dropout epilogue needs the MFMA kernel");
+        if (ep.relu_dropout || ep.gate) fail("gemm: the ReLU-dropout epilogue needs the MFMA kernel");
         long total = batch * (long)c.a.M * c.a.N;
         long blocks = (total + 255) / 256;
         if (blocks > 0x7fffffffL) fail("gemm: problem too large for the scalar kernel");

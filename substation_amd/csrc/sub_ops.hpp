@@ -167,6 +167,11 @@ struct GemmEpilogue {
     // index being the offset into C (C dense in canonical order).  See gemm_relu_dropout_ok.
     bool relu_dropout = false;
     PhiloxKey key;
+    // or: out = gate > 0 ? x : 0 with `gate` laid out like an addend (strides sbM, sbN, sbb), and the
+    // column sums of out over the rows of every 128-row slab as fp32 rows of `colsum` ([M / 128][N]);
+    // same conditions as relu_dropout (gemm_relu_dropout_ok)
+    const half_t* gate = nullptr;
+    float* colsum = nullptr;
 };
 // `ws` (optional): fp32 scratch of ws_floats elements for splitting the
 // contraction of small-output products across workgroups.

@@ -34,6 +34,7 @@ OPERATORS = [
     ('blnrd1', 'bwd', ('DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
     ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
     ('dWlin2', 'bwd', ('DLIN2', 'DROP2', 'LINW2')),
+    ('dXlin2+bdrlb', 'bwd', ('DLIN2', 'LINW2', 'DROP2', 'DLIN1')),
     ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DROP2', 'DLIN1')),      # ReLU: the gate is read off DROP2
     ('dXlin1+dWlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1', 'SB1')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
@@ -72,6 +73,7 @@ ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     ('dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei'),
     ('lin1+bad', 'lin1', 'bad'),
+    ('dXlin2+bdrlb', 'dXlin2', 'bdrlb'),
     ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
     ('dXout+dWout', 'dXout', 'dWout'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),

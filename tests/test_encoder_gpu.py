@@ -465,9 +465,10 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     """ReLU layers (the default of the module, as in the reference) read the gate
     of dropout and ReLU in the backward pass off DROP2 = relu(LIN1) * mask, which
     is positive exactly where the mask kept a positive LIN1; LIN1 and DROP2MASK are
-    then neither written nor read.  Output and every gradient must equal, bit for
-    bit, those with the option off (block_bdrlb.cuh:72: gate from DROP2MASK and
-    LIN1), and the two tensors must really be left alone."""
+    then neither written nor read, and the two operators run in the epilogues of
+    the products before them.  Output and every gradient must equal, bit for bit,
+    those with the option off (block_bdrlb.cuh:72: gate from DROP2MASK and LIN1);
+    the bias gradient that is a column sum over 4096 terms agrees to rounding."""
     from substation_amd import Encoder, layouts as L
     lay = L.mi355x_layouts()
     B, Ls, H, E = dims
@@ -486,11 +487,17 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
         Y = enc(X)
         Y.backward(DY)
         torch.cuda.synchronize()
-        outs.append([Y.detach().clone(), X.grad.clone()] + [q.grad.clone() for q in enc.parameters()])
-    for a, b in zip(*outs):
+        outs.append([('Y', Y.detach().clone()), ('DX', X.grad.clone())] +
+                    [('D' + n, q.grad.clone()) for n, q in enc.named_parameters()])
+    for (name, a), (_, b) in zip(*outs):
         assert torch.isfinite(a.float()).all()
-        assert torch.equal(a, b)
-    assert float(outs[0][1].abs().max()) > 0
+        if name == 'DLINB1':
+            # its column sums are formed in the epilogue of the product before it when the
+            # option is on: the same terms added in another order
+            assert_close(b.float().cpu().numpy(), a.float().cpu().numpy(), tol=2e-3, name=name)
+        else:
+            assert torch.equal(a, b), name
+    assert float(outs[0][1][1].abs().max()) > 0
 
 
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
