@@ -38,11 +38,11 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91469343, 'attention': 38114651, 'out': 33767869, 'bdrln1': 59008853,
-    'lin1': 88315355, 'bad': 67316332, 'lin2': 109257713, 'bdrln2': 59011779,
-    'bsb+blnrd1': 61022518, 'dXlin2': 84115563, 'dWlin2': 109268080, 'bdrlb': 101781592,
-    'dXlin1+dWlin1': 300874502, 'ebsb+blnrd2+baob': 79940530, 'dXout+dWout': 120659452, 'dWout split-k sum': 18967854,
-    'attention-bwd-dQ': 55315797, 'attention-bwd-dKdV': 55518614, 'dXQKV-fused+dWQKV-fused': 288128157, 'column-sum finish': 7831768,
+    'QKV-fused': 92578043, 'attention': 38114728, 'out': 33951168, 'bdrln1': 59014518,
+    'lin1+bad': 89917703, 'lin2': 109441059, 'bdrln2': 59012470, 'bsb+blnrd1': 61022656,
+    'dXlin2+bdrlb': 118510741, 'dWlin2': 109268276, 'dXlin1+dWlin1': 300746430, 'ebsb+blnrd2+baob': 79940171,
+    'dXout+dWout': 120967229, 'dWout split-k sum': 18967868, 'attention-bwd-dQ': 55316239, 'attention-bwd-dKdV': 55518648,
+    'dXQKV-fused+dWQKV-fused': 286639594, 'column-sum finish': 7307979,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',

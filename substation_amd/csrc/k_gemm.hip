@@ -500,7 +500,11 @@ struct DTile {
 // drawing on L2 that takes long (measured: the loads of a step alone cost about as
 // much time as its multiplications, and with one wave per SIMD the two add up);
 // while one wave of a SIMD sits in the issue of its loads the other multiplies.
-template <int TM, int TN, bool AKC, bool BKC, int S, int NW>
+// EPI: what the epilogue does after the scaling and the optional addend.  A template
+// parameter so that the plain kernel does not carry the registers of the others.
+enum { EPI_PLAIN = 0, EPI_RELU_DROPOUT = 1, EPI_GATE_COLSUM = 2 };
+
+template <int TM, int TN, bool AKC, bool BKC, int S, int NW, int EPI = EPI_PLAIN>
 __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     static_assert(S == 2 || S == 3, "two or three LDS stages");
     static_assert(NW == 4 || NW == 8, "four or eight waves");
@@ -655,7 +659,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 
     half_t* stage = st0 + wave * STAGE_WAVE;
     PhiloxKey rd_key = g.key;
-    if (g.relu_dropout) rd_key = resolved(g.key);
+    if (EPI == EPI_RELU_DROPOUT) rd_key = resolved(g.key);
     float colsum[8];              // gate mode: this lane's 8 columns summed over its rows of the wave's slab
 #pragma unroll
     for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
@@ -686,7 +690,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
             }
-            if (g.gate) {
+            if (EPI == EPI_GATE_COLSUM) {
                 // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
                 const h8 gt = *reinterpret_cast<const h8*>(g.gate + (long)mm * g.sbM + nn);
 #pragma unroll
@@ -695,7 +699,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                     colsum[e] += (float)val[e];
                 }
             }
-            if (g.relu_dropout) {
+            if (EPI == EPI_RELU_DROPOUT) {
                 // what the bias-activation-dropout operator does to the rounded sum, with the
                 // same keep bits (the element index is the offset into the dense output)
                 const uint32_t bits = keep_bits8(rd_key, (uint64_t)mm * (uint64_t)g.sCM + (uint64_t)nn);
@@ -706,7 +710,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
         }
     }
-    if (g.gate) {
+    if (EPI == EPI_GATE_COLSUM) {
         // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
         // row of partial sums per 128-row slab of the output (a finishing launch adds the slabs)
 #pragma unroll
@@ -841,12 +845,27 @@ void launch_mfma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t 
     else hipLaunchKernelGGL((k_gemm_mfma<TM, TN, false, false, FULL>), grid, dim3(256), 0, st, a);
 }
 
+template <int TM, int TN, int S, int NW, int EPI>
+void launch_dma3(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
+    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true, S, NW, EPI>), grid, dim3(NW * 64), 0, st, a);
+    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false, S, NW, EPI>), grid, dim3(NW * 64), 0, st, a);
+    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true, S, NW, EPI>), grid, dim3(NW * 64), 0, st, a);
+    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false, S, NW, EPI>), grid, dim3(NW * 64), 0, st, a);
+}
+
 template <int TM, int TN, int S, int NW>
 void launch_dma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
-    if (akc && bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, true, S, NW>), grid, dim3(NW * 64), 0, st, a);
-    else if (akc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, true, false, S, NW>), grid, dim3(NW * 64), 0, st, a);
-    else if (bkc) hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, true, S, NW>), grid, dim3(NW * 64), 0, st, a);
-    else hipLaunchKernelGGL((k_gemm_dma<TM, TN, false, false, S, NW>), grid, dim3(NW * 64), 0, st, a);
+    if (a.relu_dropout || a.gate) {
+        // only the eight-wave 256x256 kernel carries these epilogues
+        if constexpr (NW == 8) {
+            if (a.gate) launch_dma3<TM, TN, S, NW, EPI_GATE_COLSUM>(a, akc, bkc, grid, st);
+            else launch_dma3<TM, TN, S, NW, EPI_RELU_DROPOUT>(a, akc, bkc, grid, st);
+            return;
+        } else {
+            fail("gemm: this kernel variant has no ReLU-dropout or gate epilogue");
+        }
+    }
+    launch_dma3<TM, TN, S, NW, EPI_PLAIN>(a, akc, bkc, grid, st);
 }
 
 template <int TM, int TN>
