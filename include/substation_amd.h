@@ -197,8 +197,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * in encoder_backward bdrlb runs in the epilogue of the dXlin2 product
  * (`dXlin2+bdrlb`), DDROP2 is not written and DLINB1 sums its terms in another
  * order.
- * Set it to 0 before the forward call when LIN1, DROP2MASK or SB1_LINW1 are
- * wanted (debug capture). */
+ * Set it to 0 before the forward call when LIN1, DROP2MASK, SB1_LINW1 or
+ * DDROP2 are wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
