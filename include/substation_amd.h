@@ -205,6 +205,9 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * (given 16-byte aligned tensors).  No counterpart in the reference. */
 int sub_attention_in_registers(void* handle, int* planned);
 int sub_set_option(void* handle, int option, int value);
+/* The present value of an option (a caller that sized LIN1 and DROP2MASK down,
+ * see SUB_OPT_RELU_FROM_OUTPUT, checks it before every call). */
+int sub_get_option(void* handle, int option, int* value);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same
  * order, without the handle (n must be 37 resp. 64). */

@@ -9,7 +9,7 @@ reference draws none on the attention probabilities of this layer and neither
 does this.  LayerNorm uses ``rsqrt(var + eps)`` like the device path
 (``ln_mode='numpy'`` gives the script's ``std + eps``).
 
-Pinned by tests/test_decoder_oracle.py against ``torch.nn.TransformerDecoderLayer``
+Pinned by tests/test_oracle_decoder.py against ``torch.nn.TransformerDecoderLayer``
 in fp64 (post-norm, forward and every gradient including the one of the encoder
 output), which is what the reference's own test/test_transformer_torch.py does for
 its layers.

@@ -58,6 +58,7 @@ SIGNATURES = {
     'sub_set_rng_counter': (_I, [_VP, _VP]),
     'sub_last_error': (_CP, []),
     'sub_set_option': (_I, [_VP, _I, _I]),
+    'sub_get_option': (_I, [_VP, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
     'sub_attention_in_registers': (_I, [_VP, ctypes.POINTER(_I)]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
@@ -187,6 +188,11 @@ class Handle:
 
     def set_option(self, option, value):
         check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')
+
+    def get_option(self, option):
+        v = ctypes.c_int(0)
+        check(self.lib.sub_get_option(self.ptr, option, ctypes.byref(v)), 'sub_get_option')
+        return v.value
 
     def attention_in_registers(self):
         """True when self-attention will run with the scores kept in registers."""

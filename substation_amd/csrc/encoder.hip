@@ -1179,6 +1179,20 @@ int encoder_backward(void* handle, void* DY,
     return sub_encoder_backward(handle, p, (int)(sizeof(p) / sizeof(p[0])));
 }
 
+int sub_get_option(void* handle, int option, int* value) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        if (!value) fail("sub_get_option: null result pointer");
+        if (option == SUB_OPT_FUSE_EPILOGUES) *value = h.fuse_epilogues;
+        else if (option == SUB_OPT_FUSE_LN_BACKWARD) *value = h.fuse_ln_backward;
+        else if (option == SUB_OPT_FUSE_SCORES) *value = h.fuse_scores;
+        else if (option == SUB_OPT_FUSE_ATTENTION) *value = h.fuse_attention;
+        else if (option == SUB_OPT_PAIR_PRODUCTS) *value = h.pair_products;
+        else if (option == SUB_OPT_RELU_FROM_OUTPUT) *value = h.relu_from_output;
+        else fail("sub_get_option: unknown option");
+    });
+}
+
 int sub_set_option(void* handle, int option, int value) {
     return guarded([&] {
         Handle& h = as_handle(handle);

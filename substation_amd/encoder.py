@@ -36,8 +36,11 @@ class Encoder(torch.nn.Module):
                  activation_dropout_probability, residual2_dropout_probability,
                  enable_debug=False, profiling=False, *, activation='relu', seed=0,
                  intermediate_size=None, compact_attention=False, persistent_workspace=False,
-                 canonical_state_dict=False):
-        """``persistent_workspace``: the intermediates are allocated once and reused
+                 canonical_state_dict=False, compact_activation=False):
+        """``compact_activation``: with ReLU the backward pass reads its gate off the
+        dropout output, so the pre-activation LIN1 and DROP2MASK are neither written
+        nor read; allocate 8 elements for each instead of B*L*4E (at B=8 L=512
+        E=1024: 64 MiB less per layer call).  ``persistent_workspace``: the intermediates are allocated once and reused
         by every call instead of 37 ``torch.empty`` per iteration
         (pytorch_module/encoder.py:78-85,113-119); a forward call then overwrites
         what an earlier forward call saved for its backward pass, which backward()
@@ -108,6 +111,12 @@ class Encoder(torch.nn.Module):
         if self.compact_attention:
             compact = {'BETA': 8, 'ATTN_DROP': 8, 'DATTN_DROP': 8, 'DBETA': 8,
                        'ALPHA': rows * 4, 'ATTN_DROP_MASK': rows * max(max_seq_len // 16, 1)}
+        # compact_activation: as above for the two feed-forward tensors that the ReLU
+        # path leaves untouched while option 6 is on; forward() and backward() check it.
+        self.compact_activation = bool(compact_activation and not enable_debug and activation == 'relu'
+                                       and self._handle.get_option(_lib.OPT_RELU_FROM_OUTPUT))
+        if self.compact_activation:
+            compact.update({'LIN1': 8, 'DROP2MASK': 8})
         self.persistent_workspace = bool(persistent_workspace)
         self.canonical_state_dict = bool(canonical_state_dict)
         self._workspace = {}           # 'forward_interm' / 'backward_interm' -> tensors, when persistent
@@ -152,6 +161,7 @@ class Encoder(torch.nn.Module):
                 if module.compact_attention and not handle.attention_in_registers():
                     raise RuntimeError('this Encoder was built with compact_attention=True but the attention '
                                        'kernels that keep the scores in registers are switched off')
+                module._check_compact_activation()
                 dev = X.device
                 X = X.contiguous()
                 # same element count as X, shaped in the output's own dimension order
@@ -179,6 +189,7 @@ class Encoder(torch.nn.Module):
                 if module.persistent_workspace and ctx.generation != module._generation:
                     raise RuntimeError('persistent_workspace: forward() ran again before this backward pass; '
                                        'what it had saved has been overwritten')
+                module._check_compact_activation()
                 dev = DY.device
                 DY = DY.contiguous()
                 DX = torch.empty(in_shape, device=dev, dtype=DY.dtype)
@@ -199,6 +210,12 @@ class Encoder(torch.nn.Module):
                 return (DX, *param_gradients)
 
         self.encoder_func = EncoderFunction
+
+    def _check_compact_activation(self):
+        if self.compact_activation and not self._handle.get_option(_lib.OPT_RELU_FROM_OUTPUT):
+            raise RuntimeError('this Encoder was built with compact_activation=True but the ReLU gate from '
+                               'the dropout output (option 6) is switched off: LIN1 and DROP2MASK would be '
+                               'written through 8-element buffers')
 
     def _canonical_perm(self, name, layout):
         canon = _lay.CANONICAL[name]
@@ -303,7 +320,7 @@ class EncoderStack(torch.nn.Module):
                  softmax_dropout_probability, residual1_dropout_probability,
                  activation_dropout_probability, residual2_dropout_probability, *, activation='relu', seed=0,
                  intermediate_size=None, compact_attention=True, persistent_workspace=True,
-                 canonical_state_dict=True, profiling=False):
+                 canonical_state_dict=True, profiling=False, compact_activation=True):
         super().__init__()
         if layouts['input'][1] != layouts['output'][1]:
             raise ValueError(f"layers stack only when the output layout ({layouts['output'][1]}) equals the "
@@ -315,7 +332,7 @@ class EncoderStack(torch.nn.Module):
                     activation_dropout_probability, residual2_dropout_probability, profiling=profiling,
                     activation=activation, seed=seed + i, intermediate_size=intermediate_size,
                     compact_attention=compact_attention, persistent_workspace=persistent_workspace,
-                    canonical_state_dict=canonical_state_dict)
+                    canonical_state_dict=canonical_state_dict, compact_activation=compact_activation)
             for i in range(num_layers)])
         shared = {}
         for layer in self.layers:

@@ -500,6 +500,64 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     assert float(outs[0][1][1].abs().max()) > 0
 
 
+def test_compact_activation_buffers_give_the_same_results_and_refuse_the_other_gate():
+    """compact_activation=True allocates 8 elements for LIN1 and DROP2MASK, which
+    the ReLU path with the gate taken from DROP2 neither writes nor reads: results
+    are bit-identical with the fused epilogues and with the separate operators,
+    GELU layers ignore the request, and switching the gate back to LIN1 and
+    DROP2MASK is refused before anything is launched."""
+    from substation_amd import Encoder, EncoderStack, layouts as L
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = 2, 256, 4, 256
+    for fuse_epilogues in (1, 0):
+        outs = []
+        for compact in (False, True):
+            torch.manual_seed(0)
+            enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                          compact_activation=compact).cuda()
+            assert enc.compact_activation == compact
+            enc._handle.set_option(1, fuse_epilogues)
+            enc.set_rng(SEED, 0)
+            g = torch.Generator().manual_seed(5)
+            X = (0.5 * torch.randn(B, Ls, E, generator=g)).half().cuda().requires_grad_(True)
+            DY = torch.randn(B, Ls, E, generator=g).half().cuda()
+            with torch.no_grad():
+                for q in enc.parameters():
+                    q.mul_(0.1)
+            for _ in range(2):
+                X.grad = None
+                Y = enc(X)
+                Y.backward(DY)
+            torch.cuda.synchronize()
+            outs.append([Y.detach().clone(), X.grad.clone()] + [q.grad.clone() for q in enc.parameters()])
+        for a, b in zip(*outs):
+            assert torch.isfinite(a.float()).all()
+            assert torch.equal(a, b)
+    Y = enc(X)
+    enc._handle.set_option(6, 0)
+    with pytest.raises(RuntimeError, match='compact_activation'):
+        Y.backward(DY)
+    with pytest.raises(RuntimeError, match='compact_activation'):
+        enc(X)
+    gelu = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED, activation='gelu',
+                   compact_activation=True)
+    assert not gelu.compact_activation
+    # two layers with every compact buffer against two with none: same output
+    ys = []
+    for compact in (True, False):
+        torch.manual_seed(1)
+        stack = EncoderStack(2, B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                             compact_attention=compact, compact_activation=compact).cuda()
+        stack.set_rng(SEED, 0)
+        Xs = X.detach().clone().requires_grad_(True)
+        Ys = stack(Xs)
+        Ys.backward(DY)
+        torch.cuda.synchronize()
+        ys.append((Ys.detach().clone(), Xs.grad.clone(), stack.workspace_bytes()))
+    assert torch.equal(ys[0][0], ys[1][0]) and torch.equal(ys[0][1], ys[1][1])
+    assert ys[0][2] < ys[1][2] - 2 * 2 * (B * Ls * 4 * E * 2 - 16)
+
+
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
     """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
     the library's one-time allocations) and replayed with eager work in between:
