@@ -460,7 +460,9 @@ def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback()
         enc(X)
 
 
-@pytest.mark.parametrize('dims', [(2, 256, 4, 256), (8, 512, 16, 1024)])
+@pytest.mark.parametrize('dims', [(2, 256, 4, 256), (8, 512, 16, 1024),
+                                  (15, 256, 8, 512, 4352),      # 15 x 17 tiles of 256 x 256: odd counts both ways
+                                  (16, 512, 8, 512, 2048)])     # 32 x 8 tiles
 def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     """ReLU layers (the default of the module, as in the reference) read the gate
     of dropout and ReLU in the backward pass off DROP2 = relu(LIN1) * mask, which
@@ -471,11 +473,13 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     the bias gradient that is a column sum over 4096 terms agrees to rounding."""
     from substation_amd import Encoder, layouts as L
     lay = L.mi355x_layouts()
-    B, Ls, H, E = dims
+    B, Ls, H, E = dims[:4]
+    U = dims[4] if len(dims) > 4 else None
     outs = []
     for from_output in (0, 1):
         torch.manual_seed(0)
-        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED).cuda()
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                      intermediate_size=U).cuda()
         enc._handle.set_option(6, from_output)
         enc.set_rng(SEED, 0)
         g = torch.Generator().manual_seed(5)
