@@ -38,11 +38,11 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 92578043, 'attention': 38114728, 'out': 33951168, 'bdrln1': 59014518,
-    'lin1+bad': 89917703, 'lin2': 109441059, 'bdrln2': 59012470, 'bsb+blnrd1': 61022656,
-    'dXlin2+bdrlb': 118510741, 'dWlin2': 109268276, 'dXlin1+dWlin1': 300746430, 'ebsb+blnrd2+baob': 79940171,
-    'dXout+dWout': 120967229, 'dWout split-k sum': 18967868, 'attention-bwd-dQ': 55316239, 'attention-bwd-dKdV': 55518648,
-    'dXQKV-fused+dWQKV-fused': 286639594, 'column-sum finish': 7307979,
+    'QKV-fused': 91465052, 'attention': 38114745, 'out': 33775039, 'bdrln1': 59010189,
+    'lin1+bad': 87706765, 'lin2': 109264945, 'bdrln2': 59010153, 'bsb+blnrd1': 61022887,
+    'dXlin2+bdrlb': 118258890, 'dWlin2': 109266152, 'dXlin1+dWlin1': 300456232, 'ebsb+blnrd2+baob': 79940078,
+    'dXout+dWout': 121444063, 'dWout split-k sum': 18966832, 'attention-bwd-dQ': 55316441, 'attention-bwd-dKdV': 55518618,
+    'dXQKV-fused+dWQKV-fused': 293626205,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',

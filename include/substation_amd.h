@@ -200,6 +200,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * Set it to 0 before the forward call when LIN1, DROP2MASK, SB1_LINW1 or
  * DDROP2 are wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6
+/* SUB_OPT_FINISH_IN_PAIR (default 1): the second stage of the column sums of
+ * encoder_backward (adding the per-chunk fp32 partials of the bias and
+ * LayerNorm-parameter gradients) runs in extra workgroups of the last pair of
+ * products of the pass, which its last, partly filled round of tiles leaves
+ * room for, instead of in a launch of its own.  Same code, same order of
+ * additions: results are bit-identical.  Needs SUB_OPT_PAIR_PRODUCTS and the
+ * in-register attention (whose kernels produce the DBKQV partials). */
+#define SUB_OPT_FINISH_IN_PAIR 7
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

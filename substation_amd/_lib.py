@@ -20,6 +20,7 @@ OPT_FUSE_SCORES = 3
 OPT_FUSE_ATTENTION = 4
 OPT_PAIR_PRODUCTS = 5
 OPT_RELU_FROM_OUTPUT = 6
+OPT_FINISH_IN_PAIR = 7
 FUSE_REQUIRED = 2
 
 

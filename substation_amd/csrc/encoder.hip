@@ -188,6 +188,7 @@ struct Handle {
     bool fuse_scores = true;
     int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
+    bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
@@ -454,7 +455,7 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
 // gradient next to it) in one launch where they qualify, else one after the other.
 void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1, const char* name1,
                    const void* addend1, int id2, const void* A2, const void* B2, void* C2, const char* name2,
-                   const char* pair_name) {
+                   const char* pair_name, FinishJobs* tail = nullptr) {
     if (h.pair_products) {
         ProfScope ps(h, pair_name);
         const GemmPlan& p1 = h.gemm[id1];
@@ -467,7 +468,7 @@ void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1,
         ensure_gws(h, h.gws_need);
         if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha, e1, p2.shape,
                              (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream, h.gws,
-                             h.gws_floats))
+                             h.gws_floats, tail))
             return;
         ps.cancel();
     }
@@ -1012,13 +1013,17 @@ void backward(Handle& h, const BwdPtrs& t) {
     }
     const bool fuse_dx = h.fuse_epilogues && h.gemm[G_DXQKV_RESID].ok && aligned16(D[DRESID1]) &&
                          aligned16(t.DX);
+    // The last products of the pass finish the deferred column sums in workgroups of
+    // their own launch when every producer of those sums has been launched by now
+    // (baib below would add one more).
+    FinishJobs* tail = h.deferring && attn_bias && h.finish_in_pair ? &h.deferred : nullptr;
     if (fuse_dx) {
         // DX = WKQV.DKKQQVV + DRESID1 in one pass; DXATT is not written
         run_gemm_pair(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1],
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused");
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail);
     } else {
         run_gemm_pair(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused", nullptr,
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused");
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail);
     }
     if (!attn_bias) {
         ProfScope ps(h, "baib");
@@ -1189,6 +1194,7 @@ int sub_get_option(void* handle, int option, int* value) {
         else if (option == SUB_OPT_FUSE_ATTENTION) *value = h.fuse_attention;
         else if (option == SUB_OPT_PAIR_PRODUCTS) *value = h.pair_products;
         else if (option == SUB_OPT_RELU_FROM_OUTPUT) *value = h.relu_from_output;
+        else if (option == SUB_OPT_FINISH_IN_PAIR) *value = h.finish_in_pair;
         else fail("sub_get_option: unknown option");
     });
 }
@@ -1201,6 +1207,7 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_FUSE_SCORES) h.fuse_scores = value != 0;
         else if (option == SUB_OPT_PAIR_PRODUCTS) h.pair_products = value != 0;
         else if (option == SUB_OPT_RELU_FROM_OUTPUT) h.relu_from_output = value != 0;
+        else if (option == SUB_OPT_FINISH_IN_PAIR) h.finish_in_pair = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;

@@ -8,6 +8,7 @@
 // reduces its token chunk for a strip of features into fp32 partials
 // (deterministically, no atomics), and a small second kernel adds the partials.
 #include "sub_ops.hpp"
+#include "sub_finish.hpp"
 
 namespace sub {
 
@@ -201,35 +202,9 @@ __global__ __launch_bounds__(BLOCK) void k_colreduce(RowSpace rs, ColArgs a, flo
 // Adds the ntc partials of every (sum, kept index, feature) of up to
 // kMaxFinishJobs operators in one launch: blockIdx.y selects the operator, 32
 // features x 8 slices per block, the slices combined through LDS.
-__global__ __launch_bounds__(BLOCK) void k_colfinish(FinishJobs jobs) {
+__global__ __launch_bounds__(kFinishThreads) void k_colfinish(FinishJobs jobs) {
     __shared__ float red[8][33];
-    const FinishJob& j = jobs.j[blockIdx.y];
-    const int fl = threadIdx.x & 31, sl = threadIdx.x >> 5;
-    long idx = (long)blockIdx.x * 32 + fl;
-    const bool ok = idx < (long)j.ns * j.nbatch * j.R;
-    int s = 0, f = 0, z = 0;
-    float t = 0.f;
-    if (ok) {
-        long sz = idx / j.R; f = (int)(idx - sz * j.R);
-        s = (int)(sz / j.nbatch); z = (int)(sz - (long)s * j.nbatch);
-        const float* p = j.ws + sz * j.ntc * j.R + f;
-        // eight independent loads per round trip instead of one
-        for (int c = sl; c < j.ntc; c += 64) {
-            float v[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = c + 8 * k < j.ntc ? p[(long)(c + 8 * k) * j.R] : 0.f;
-#pragma unroll
-            for (int k = 0; k < 8; ++k) t += v[k];
-        }
-    }
-    red[sl][fl] = t;
-    __syncthreads();
-    if (sl == 0 && ok) {
-        float tot = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) tot += red[i][fl];
-        j.fo.out[s][(long)(z / j.fo.n1) * j.fo.ob0 + (long)(z % j.fo.n1) * j.fo.ob1 + (long)f * j.fo.of] = (half_t)tot;
-    }
+    finish_block(jobs.j[blockIdx.y], blockIdx.x, red);
 }
 
 struct ColPlan {
@@ -320,12 +295,7 @@ __global__ __launch_bounds__(BLOCK) void k_rowgroup_sum(RowSpace rs, View d, Vie
 
 void launch_colfinish(const FinishJobs& jobs, hipStream_t st) {
     if (jobs.n == 0) return;
-    long maxn = 0;
-    for (int i = 0; i < jobs.n; ++i) {
-        long n = (long)jobs.j[i].ns * jobs.j[i].nbatch * jobs.j[i].R;
-        if (n > maxn) maxn = n;
-    }
-    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)((maxn + 31) / 32), jobs.n), dim3(BLOCK), 0, st, jobs);
+    hipLaunchKernelGGL(k_colfinish, dim3((unsigned)finish_groups(jobs), jobs.n), dim3(kFinishThreads), 0, st, jobs);
     check_launch("column-sum finish");
 }
 

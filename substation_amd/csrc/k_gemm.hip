@@ -14,6 +14,7 @@
 #include <cstdlib>
 
 #include "sub_ops.hpp"
+#include "sub_finish.hpp"
 
 namespace sub {
 
@@ -399,12 +400,22 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 // its output write -- the other one runs.  Alone, each product would leave a
 // single wave on every SIMD.
 template <bool A1, bool B1, bool A2, bool B2>
-__global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2) {
+__global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2,
+                                                   FinishJobs tail, unsigned tail_groups) {
     constexpr int L1 = mfma_lds_halves<2, 2, A1, B1>(), L2 = mfma_lds_halves<2, 2, A2, B2>();
     __shared__ __attribute__((aligned(16))) half_t lds[L1 > L2 ? L1 : L2];
+    static_assert(sizeof(lds) >= 8 * 33 * sizeof(float) && kFinishThreads == 256, "finish_block needs this much");
     // n1, n2: workgroups of the two products (multiples of 8).  While both have
     // some left they alternate in groups of 8; the rest belongs to the larger one.
     const unsigned b = blockIdx.x, both = 2 * (n1 < n2 ? n1 : n2);
+    if (b >= n1 + n2) {
+        // Workgroups past the tiles finish column sums of earlier launches: they are
+        // dispatched last, into the places the final, partly filled round of tiles
+        // leaves free, and spare the pass a launch of their own.
+        const unsigned t = b - (n1 + n2);
+        finish_block(tail.j[t / tail_groups], t % tail_groups, reinterpret_cast<float (*)[33]>(lds));
+        return;
+    }
     if (b < both) {
         const unsigned id = ((b >> 4) << 3) | (b & 7);
         if ((b >> 3) & 1) gemm_mfma_body<2, 2, A2, B2, true>(g2, id, n2, lds);
@@ -950,7 +961,7 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
 bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws,
-                      size_t ws_floats) {
+                      size_t ws_floats, FinishJobs* tail) {
     static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
     if (off) return false;
     const GemmShape* sh[2] = {&s1, &s2};
@@ -972,16 +983,25 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
         if (pick_tile(a, batch, akc[i], bkc[i]) != 22) return false;
         if (akc[i] && bkc[i]) return false;                  // the asynchronous kernel's products stay on their own
     }
-    dim3 grid((unsigned)(n[0] + n[1]));
+    // column sums of earlier launches, finished by workgroups after the tiles (none of them
+    // may be a sum that this launch itself contributes to)
+    FinishJobs tj;
+    unsigned tg = 1;
+    if (tail && tail->n > 0) {
+        const long groups = finish_groups(*tail);
+        if (groups * tail->n <= 4096) { tj = *tail; tg = (unsigned)groups; }
+    }
+    dim3 grid((unsigned)(n[0] + n[1] + (long)tj.n * tg));
     const unsigned n1 = (unsigned)n[0], n2 = (unsigned)n[1];
     if (akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
     else if (!akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
     else if (akc[0] && !bkc[0] && akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2);
+        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
     else
         return false;
+    if (tj.n > 0) tail->n = 0;         // taken: nothing left for the caller to finish
     for (int i = 0; i < 2; ++i)
         if (c[i].a.splits > 1) {
             const long batch = sh[i]->batch(), nq = batch * (long)c[i].a.M * (c[i].a.N / 4);

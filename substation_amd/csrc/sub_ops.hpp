@@ -182,11 +182,13 @@ void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C
 bool gemm_relu_dropout_ok(const GemmShape& g, const void* A, const void* B, const void* C, const GemmEpilogue& ep);
 // Two independent contractions in one launch, their workgroups interleaved so that
 // every CU works on both at once.  Returns false, having launched nothing, when
-// the pair does not qualify (then call launch_gemm for each).
+// the pair does not qualify (then call launch_gemm for each).  `tail` (optional):
+// deferred column sums of EARLIER launches, finished by extra workgroups of this
+// launch; tail->n is set to 0 when they were taken, else it is left as it was.
 bool launch_gemm_pair(const GemmShape& g1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& g2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws = nullptr,
-                      size_t ws_floats = 0);
+                      size_t ws_floats = 0, FinishJobs* tail = nullptr);
 // Scratch (in floats) that launch_gemm can make use of for this shape; 0 if none.
 size_t gemm_splitk_ws_floats(const GemmShape& g);
 // Which kernel launch_gemm would pick: 0 = scalar fallback, 1 = MFMA.

@@ -504,6 +504,47 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     assert float(outs[0][1][1].abs().max()) > 0
 
 
+@pytest.mark.parametrize('dims,activation', [((8, 512, 16, 1024), 'relu'), ((4, 512, 8, 512), 'gelu'),
+                                             ((2, 256, 4, 256), 'relu')])
+def test_column_sums_finished_inside_the_last_pair_launch_are_bit_identical(dims, activation):
+    """The second stage of the column sums (bias and LayerNorm-parameter gradients)
+    runs in extra workgroups of the last pair of products of the backward pass
+    (option 7) instead of in a launch of its own: every gradient must be equal bit
+    for bit, twice in a row (the deferred list is rebuilt per call).  The smallest
+    case does not qualify for a pair launch and takes the separate launch either
+    way."""
+    from substation_amd import Encoder, layouts as L
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = dims
+    outs = []
+    for in_pair in (0, 1):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                      activation=activation).cuda()
+        enc._handle.set_option(7, in_pair)
+        assert enc._handle.get_option(7) == in_pair
+        g = torch.Generator().manual_seed(5)
+        X = (0.5 * torch.randn(B, Ls, E, generator=g)).half().cuda().requires_grad_(True)
+        DY = torch.randn(B, Ls, E, generator=g).half().cuda()
+        with torch.no_grad():
+            for q in enc.parameters():
+                q.mul_(0.1)
+        got = []
+        for step in range(2):
+            enc.set_rng(SEED, step)
+            X.grad = None
+            enc.zero_grad()
+            Y = enc(X)
+            Y.backward(DY)
+            torch.cuda.synchronize()
+            got += [('DX', X.grad.clone())] + [('D' + n, q.grad.clone()) for n, q in enc.named_parameters()]
+        outs.append(got)
+    for (name, a), (_, b) in zip(*outs):
+        assert torch.isfinite(a.float()).all()
+        assert torch.equal(a, b), name
+    assert all(float(a.abs().max()) > 0 for name, a in outs[1] if name in ('DBKQV', 'DBO', 'DS1', 'DB2', 'DLINB1'))
+
+
 def test_compact_activation_buffers_give_the_same_results_and_refuse_the_other_gate():
     """compact_activation=True allocates 8 elements for LIN1 and DROP2MASK, which
     the ReLU path with the gate taken from DROP2 neither writes nor reads: results
