@@ -38,11 +38,10 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91465052, 'attention': 38114745, 'out': 33775039, 'bdrln1': 59010189,
-    'lin1+bad': 87706765, 'lin2': 109264945, 'bdrln2': 59010153, 'bsb+blnrd1': 61022887,
-    'dXlin2+bdrlb': 118258890, 'dWlin2': 109266152, 'dXlin1+dWlin1': 300456232, 'ebsb+blnrd2+baob': 79940078,
-    'dXout+dWout': 121444063, 'dWout split-k sum': 18966832, 'attention-bwd-dQ': 55316441, 'attention-bwd-dKdV': 55518618,
-    'dXQKV-fused+dWQKV-fused': 293626205,
+    'QKV-fused': 91469435, 'attention': 38114643, 'out': 33775066, 'bdrln1': 59009787,
+    'lin1+bad': 87713311, 'lin2': 109265032, 'bdrln2': 59008177, 'bsb+blnrd1': 61023087,
+    'dXlin2+bdrlb': 118261081, 'dWlin2': 109276643, 'dXlin1+dWlin1': 299326771, 'ebsb+blnrd2+baob': 79940204,
+    'dXout+dWout': 120625292, 'attention-bwd-dQ': 55318264, 'attention-bwd-dKdV': 55518659, 'dXQKV-fused+dWQKV-fused': 316609906,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',

@@ -204,7 +204,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * encoder_backward (adding the per-chunk fp32 partials of the bias and
  * LayerNorm-parameter gradients) runs in extra workgroups of the last pair of
  * products of the pass, which its last, partly filled round of tiles leaves
- * room for, instead of in a launch of its own.  Same code, same order of
+ * room for, instead of in a launch of its own; the sum of the split-k partials
+ * of the dWout product waits for that launch too.  Same code, same order of
  * additions: results are bit-identical.  Needs SUB_OPT_PAIR_PRODUCTS and the
  * in-register attention (whose kernels produce the DBKQV partials). */
 #define SUB_OPT_FINISH_IN_PAIR 7

@@ -188,6 +188,7 @@ struct Handle {
     bool fuse_scores = true;
     int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
+    SplitSum pending_sum;             // dWout's split-k sum between its launch and the last pair of the backward pass
     bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     std::vector<ProfEntry> prof;
@@ -455,7 +456,8 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
 // gradient next to it) in one launch where they qualify, else one after the other.
 void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1, const char* name1,
                    const void* addend1, int id2, const void* A2, const void* B2, void* C2, const char* name2,
-                   const char* pair_name, FinishJobs* tail = nullptr) {
+                   const char* pair_name, FinishJobs* tail = nullptr, SplitSum* defer_sum = nullptr,
+                   SplitSum* run_sum = nullptr) {
     if (h.pair_products) {
         ProfScope ps(h, pair_name);
         const GemmPlan& p1 = h.gemm[id1];
@@ -468,10 +470,14 @@ void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1,
         ensure_gws(h, h.gws_need);
         if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha, e1, p2.shape,
                              (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream, h.gws,
-                             h.gws_floats, tail))
+                             h.gws_floats, tail, defer_sum, run_sum)) {
+            if (run_sum) launch_split_sum(*run_sum, h.stream);      // did not fit into that launch
             return;
+        }
         ps.cancel();
     }
+    // the products below may split their contractions over the same scratch
+    if (run_sum) launch_split_sum(*run_sum, h.stream);
     run_gemm(h, id1, A1, B1, C1, name1, addend1);
     run_gemm(h, id2, A2, B2, C2, name2);
 }
@@ -874,6 +880,7 @@ void backward(Handle& h, const BwdPtrs& t) {
     h.deferring = !h.profiling;
     h.ws_cursor = 0;
     h.deferred.n = 0;
+    h.pending_sum.pending = false;
     struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
     void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
     bool fused = false;
@@ -954,13 +961,18 @@ void backward(Handle& h, const BwdPtrs& t) {
             op_baob(h, D[DATT], h.lb[DATT], DW[BO]);
         }
     }
+    AttnArgs at;
+    const bool attn_fused = attention_fused(h, F, at);
+    // With the attention in registers nothing between here and the last pair of
+    // products touches the split-k scratch: the sum of dWout's partials can wait and
+    // run in workgroups of that launch.
     run_gemm_pair(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout", nullptr,
-                  G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout", "dXout+dWout");
+                  G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout", "dXout+dWout", nullptr,
+                  h.deferring && attn_fused && h.finish_in_pair ? &h.pending_sum : nullptr);
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
-    AttnArgs at;
     bool attn_bias = false;
-    if (attention_fused(h, F, at)) {
+    if (attn_fused) {
         if (!attn_side(D[DGAMMA], h.lb[DGAMMA], dJ, at.d_o) || !attn_side(DQQ, h.lDQQ, dJ, at.dq) ||
             !attn_side(DKK, h.lDKK, dK, at.dk) || !attn_side(DVV, h.lDKK, dK, at.dv))
             fail("encoder_backward: attention layouts changed since the forward pass");
@@ -1020,10 +1032,12 @@ void backward(Handle& h, const BwdPtrs& t) {
     if (fuse_dx) {
         // DX = WKQV.DKKQQVV + DRESID1 in one pass; DXATT is not written
         run_gemm_pair(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1],
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail);
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail, nullptr,
+                      &h.pending_sum);
     } else {
         run_gemm_pair(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused", nullptr,
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail);
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail, nullptr,
+                      &h.pending_sum);
     }
     if (!attn_bias) {
         ProfScope ps(h, "baib");

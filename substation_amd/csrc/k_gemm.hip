@@ -12,6 +12,7 @@
 // accumulators (4 consecutive n per lane), staged through LDS and written as
 // full 128-bit rows.
 #include <cstdlib>
+#include <cstring>
 
 #include "sub_ops.hpp"
 #include "sub_finish.hpp"
@@ -399,9 +400,12 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 // one of them waits -- for its operands, at its barrier, in its first fetch or
 // its output write -- the other one runs.  Alone, each product would leave a
 // single wave on every SIMD.
+__device__ __forceinline__ void splitk_sum_block(const GemmArgs& g, long nb_total, long block);
+
 template <bool A1, bool B1, bool A2, bool B2>
 __global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2,
-                                                   FinishJobs tail, unsigned tail_groups) {
+                                                   FinishJobs tail, unsigned tail_groups, unsigned tail_blocks,
+                                                   GemmArgs gsum, long sum_batches) {
     constexpr int L1 = mfma_lds_halves<2, 2, A1, B1>(), L2 = mfma_lds_halves<2, 2, A2, B2>();
     __shared__ __attribute__((aligned(16))) half_t lds[L1 > L2 ? L1 : L2];
     static_assert(sizeof(lds) >= 8 * 33 * sizeof(float) && kFinishThreads == 256, "finish_block needs this much");
@@ -409,11 +413,14 @@ __global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, uns
     // some left they alternate in groups of 8; the rest belongs to the larger one.
     const unsigned b = blockIdx.x, both = 2 * (n1 < n2 ? n1 : n2);
     if (b >= n1 + n2) {
-        // Workgroups past the tiles finish column sums of earlier launches: they are
-        // dispatched last, into the places the final, partly filled round of tiles
-        // leaves free, and spare the pass a launch of their own.
+        // Workgroups past the tiles finish column sums of earlier launches, then add the
+        // split-k partials of an earlier product: they are dispatched last, into the
+        // places the tiles leave free on the CUs, and spare the pass two small launches.
         const unsigned t = b - (n1 + n2);
-        finish_block(tail.j[t / tail_groups], t % tail_groups, reinterpret_cast<float (*)[33]>(lds));
+        if (t < tail_blocks)
+            finish_block(tail.j[t / tail_groups], t % tail_groups, reinterpret_cast<float (*)[33]>(lds));
+        else
+            splitk_sum_block(gsum, sum_batches, t - tail_blocks);
         return;
     }
     if (b < both) {
@@ -737,9 +744,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 }
 
 // Adds the k-split partials: C[b,m,n] = fp16(alpha * sum_s P[s][b][m][n]) (+ addend).
-__global__ __launch_bounds__(256) void k_gemm_splitk_reduce(GemmArgs g, long nb_total) {
+__device__ __forceinline__ void splitk_sum_block(const GemmArgs& g, long nb_total, long block) {
     const long quads = (long)g.N / 4;
-    long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    long idx = block * 256 + threadIdx.x;
     if (idx >= nb_total * g.M * quads) return;
     int nq = (int)(idx % quads); long rr = idx / quads;
     int m = (int)(rr % g.M); long bz = rr / g.M;
@@ -764,6 +771,10 @@ __global__ __launch_bounds__(256) void k_gemm_splitk_reduce(GemmArgs g, long nb_
         for (int e = 0; e < 4; ++e) o[e] = (half_t)((float)o[e] + (float)ad[e]);
     }
     *reinterpret_cast<h4*>(c) = o;
+}
+
+__global__ __launch_bounds__(256) void k_gemm_splitk_reduce(GemmArgs g, long nb_total) {
+    splitk_sum_block(g, nb_total, blockIdx.x);
 }
 
 inline bool mult8(long x) { return (x & 7) == 0; }
@@ -961,9 +972,16 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
 bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws,
-                      size_t ws_floats, FinishJobs* tail) {
+                      size_t ws_floats, FinishJobs* tail, SplitSum* defer_sum, SplitSum* run_sum) {
+    static_assert(sizeof(GemmArgs) <= sizeof(SplitSum::args), "SplitSum holds a product's kernel arguments");
     static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
     if (off) return false;
+    const float* const ws_base = ws;
+    if (run_sum && run_sum->pending && ws) {
+        // this launch's own partials go behind the ones still waiting for their sum
+        if (run_sum->floats >= ws_floats) { ws = nullptr; ws_floats = 0; }
+        else { ws += run_sum->floats; ws_floats -= run_sum->floats; }
+    }
     const GemmShape* sh[2] = {&s1, &s2};
     Canon c[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
     bool akc[2], bkc[2], split_used = false;
@@ -991,24 +1009,50 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
         const long groups = finish_groups(*tail);
         if (groups * tail->n <= 4096) { tj = *tail; tg = (unsigned)groups; }
     }
-    dim3 grid((unsigned)(n[0] + n[1] + (long)tj.n * tg));
+    const unsigned tb = (unsigned)tj.n * tg;
+    GemmArgs gsum{};
+    long sum_batches = 0, sum_blocks = 0;
+    if (run_sum && run_sum->pending) {
+        memcpy(&gsum, run_sum->args, sizeof(GemmArgs));
+        const long blocks = (run_sum->nb_total * (long)gsum.M * (gsum.N / 4) + 255) / 256;
+        if (blocks <= 8192) { sum_batches = run_sum->nb_total; sum_blocks = blocks; }
+    }
+    dim3 grid((unsigned)(n[0] + n[1] + tb + sum_blocks));
     const unsigned n1 = (unsigned)n[0], n2 = (unsigned)n[1];
     if (akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
+        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
     else if (!akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
+        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
     else if (akc[0] && !bkc[0] && akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg);
+        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
     else
         return false;
     if (tj.n > 0) tail->n = 0;         // taken: nothing left for the caller to finish
+    if (sum_blocks > 0) run_sum->pending = false;
     for (int i = 0; i < 2; ++i)
         if (c[i].a.splits > 1) {
             const long batch = sh[i]->batch(), nq = batch * (long)c[i].a.M * (c[i].a.N / 4);
+            if (defer_sum && !defer_sum->pending && c[i].a.partial == ws_base) {
+                memcpy(defer_sum->args, &c[i].a, sizeof(GemmArgs));
+                defer_sum->nb_total = batch;
+                defer_sum->floats = (size_t)batch * c[i].a.M * c[i].a.N * c[i].a.splits;
+                defer_sum->pending = true;
+                continue;
+            }
             hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, c[i].a, batch);
         }
     check_launch("gemm pair");
     return true;
+}
+
+void launch_split_sum(SplitSum& s, hipStream_t st) {
+    if (!s.pending) return;
+    GemmArgs g;
+    memcpy(&g, s.args, sizeof(GemmArgs));
+    const long nq = s.nb_total * (long)g.M * (g.N / 4);
+    hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, g, s.nb_total);
+    check_launch("split-k sum");
+    s.pending = false;
 }
 
 void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C, float alpha,
