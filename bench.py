@@ -38,10 +38,10 @@ CONFIGS = {
 # WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
 # profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
 MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91469435, 'attention': 38114643, 'out': 33775066, 'bdrln1': 59009787,
-    'lin1+bad': 87713311, 'lin2': 109265032, 'bdrln2': 59008177, 'bsb+blnrd1': 61023087,
-    'dXlin2+bdrlb': 118261081, 'dWlin2': 109276643, 'dXlin1+dWlin1': 299326771, 'ebsb+blnrd2+baob': 79940204,
-    'dXout+dWout': 120625292, 'attention-bwd-dQ': 55318264, 'attention-bwd-dKdV': 55518659, 'dXQKV-fused+dWQKV-fused': 316609906,
+    'QKV-fused': 91452057, 'attention': 38114912, 'out': 33775005, 'bdrln1': 59014043,
+    'lin1+bad': 87734212, 'lin2': 109264774, 'bdrln2': 59016749, 'bsb+blnrd1': 61022384,
+    'dXlin2+bdrlb': 118260844, 'dWlin2': 109269143, 'dXlin1+dWlin1': 298726901, 'ebsb+blnrd2+baob': 79940065,
+    'dXout': 33752717, 'attention-bwd-dQ': 55316836, 'attention-bwd-dKdV': 55518567, 'dXQKV-fused+dWQKV-fused+dWout': 373479999,
 }
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
@@ -91,6 +91,8 @@ def algorithmic_work(B, L, H, E, relu_from_output=True):
     w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
     w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
     w['dXout+dWout'] = ('mfma', 2 * outp[0], 2 * outp[1])
+    # the last launch of the backward pass with dWout's tiles in the places it leaves free
+    w['dXQKV-fused+dWQKV-fused+dWout'] = ('mfma', 2 * proj[0] + outp[0], 2 * proj[1] + outp[1])
     # lin1 with bias, ReLU and dropout in its epilogue: the product's flops, SB1 and LINW1 in, DROP2 out
     w['lin1+bad'] = ('mfma',) + ffn
     w['dXlin2+bdrlb'] = ('mfma', ffn[0], ffn[1] + 2 * tok * U)      # the product's bytes plus the gate (DROP2) read

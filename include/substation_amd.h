@@ -204,9 +204,12 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * encoder_backward (adding the per-chunk fp32 partials of the bias and
  * LayerNorm-parameter gradients) runs in extra workgroups of the last pair of
  * products of the pass, which its last, partly filled round of tiles leaves
- * room for, instead of in a launch of its own; the sum of the split-k partials
- * of the dWout product waits for that launch too.  Same code, same order of
- * additions: results are bit-identical.  Needs SUB_OPT_PAIR_PRODUCTS and the
+ * room for, instead of in a launch of its own (same code, same order of
+ * additions: bit-identical).  Where that launch also has room for the tiles of
+ * the dWout product, dWout runs there with its contraction in one piece and
+ * dXout runs alone (DWO then sums its terms in another order than with the
+ * option off: equal to rounding).  Profiling names: `dXout`,
+ * `dXQKV-fused+dWQKV-fused+dWout`.  Needs SUB_OPT_PAIR_PRODUCTS and the
  * in-register attention (whose kernels produce the DBKQV partials). */
 #define SUB_OPT_FINISH_IN_PAIR 7
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are

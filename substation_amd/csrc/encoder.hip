@@ -188,7 +188,6 @@ struct Handle {
     bool fuse_scores = true;
     int fuse_attention = 1;           // 0 off, 1 where possible, 2 required
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
-    SplitSum pending_sum;             // dWout's split-k sum between its launch and the last pair of the backward pass
     bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     std::vector<ProfEntry> prof;
@@ -454,32 +453,43 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
 
 // Two products that do not depend on one another (a data gradient and the weight
 // gradient next to it) in one launch where they qualify, else one after the other.
+GemmEpilogue addend_epilogue(const GemmPlan& p, const void* addend) {
+    GemmEpilogue e;
+    if (addend) {
+        e.bias = (const half_t*)addend; e.sbM = p.sM; e.sbN = p.sN;
+        for (int i = 0; i < 3; ++i) e.sbb[i] = p.sb[i];
+    }
+    return e;
+}
+
 void run_gemm_pair(Handle& h, int id1, const void* A1, const void* B1, void* C1, const char* name1,
                    const void* addend1, int id2, const void* A2, const void* B2, void* C2, const char* name2,
-                   const char* pair_name, FinishJobs* tail = nullptr, SplitSum* defer_sum = nullptr,
-                   SplitSum* run_sum = nullptr) {
+                   const char* pair_name, FinishJobs* tail = nullptr, PairThird* third = nullptr) {
     if (h.pair_products) {
         ProfScope ps(h, pair_name);
         const GemmPlan& p1 = h.gemm[id1];
         const GemmPlan& p2 = h.gemm[id2];
-        GemmEpilogue e1, e2;
-        if (addend1) {
-            e1.bias = (const half_t*)addend1; e1.sbM = p1.sM; e1.sbN = p1.sN;
-            for (int i = 0; i < 3; ++i) e1.sbb[i] = p1.sb[i];
-        }
         ensure_gws(h, h.gws_need);
-        if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha, e1, p2.shape,
-                             (const half_t*)A2, (const half_t*)B2, (half_t*)C2, p2.alpha, e2, h.stream, h.gws,
-                             h.gws_floats, tail, defer_sum, run_sum)) {
-            if (run_sum) launch_split_sum(*run_sum, h.stream);      // did not fit into that launch
+        if (launch_gemm_pair(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, p1.alpha,
+                             addend_epilogue(p1, addend1), p2.shape, (const half_t*)A2, (const half_t*)B2,
+                             (half_t*)C2, p2.alpha, GemmEpilogue{}, h.stream, h.gws, h.gws_floats, tail, third))
             return;
-        }
         ps.cancel();
     }
-    // the products below may split their contractions over the same scratch
-    if (run_sum) launch_split_sum(*run_sum, h.stream);
     run_gemm(h, id1, A1, B1, C1, name1, addend1);
     run_gemm(h, id2, A2, B2, C2, name2);
+}
+
+// Would run_gemm_pair with these arguments take `third` into its launch?
+bool pair_takes_third(Handle& h, int id1, const void* A1, const void* B1, void* C1, const void* addend1, int id2,
+                      const void* A2, const void* B2, void* C2, const PairThird& third) {
+    if (!h.pair_products) return false;
+    const GemmPlan& p1 = h.gemm[id1];
+    const GemmPlan& p2 = h.gemm[id2];
+    ensure_gws(h, h.gws_need);
+    return gemm_pair_takes_third(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1,
+                                 addend_epilogue(p1, addend1), p2.shape, (const half_t*)A2, (const half_t*)B2,
+                                 (half_t*)C2, GemmEpilogue{}, h.gws, h.gws_floats, third);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -880,7 +890,6 @@ void backward(Handle& h, const BwdPtrs& t) {
     h.deferring = !h.profiling;
     h.ws_cursor = 0;
     h.deferred.n = 0;
-    h.pending_sum.pending = false;
     struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
     void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
     bool fused = false;
@@ -963,12 +972,28 @@ void backward(Handle& h, const BwdPtrs& t) {
     }
     AttnArgs at;
     const bool attn_fused = attention_fused(h, F, at);
-    // With the attention in registers nothing between here and the last pair of
-    // products touches the split-k scratch: the sum of dWout's partials can wait and
-    // run in workgroups of that launch.
-    run_gemm_pair(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout", nullptr,
-                  G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout", "dXout+dWout", nullptr,
-                  h.deferring && attn_fused && h.finish_in_pair ? &h.pending_sum : nullptr);
+    const bool fuse_dx = h.fuse_epilogues && h.gemm[G_DXQKV_RESID].ok && aligned16(D[DRESID1]) &&
+                         aligned16(t.DX);
+    // dWout (64 tiles of 128 x 128 at the bench workload, too few for a launch of its
+    // own without splitting its contraction) needs nothing but DATT and feeds nothing:
+    // when the last pair of products of the pass has room for its tiles it runs there,
+    // unsplit, and dXout runs alone here.
+    PairThird dwout;
+    bool dwout_later = false;
+    if (h.finish_in_pair && attn_fused) {
+        const GemmPlan& p3 = h.gemm[G_DWOUT];
+        dwout.shape = &p3.shape; dwout.A = (const half_t*)F[GAMMA]; dwout.B = (const half_t*)D[DATT];
+        dwout.C = (half_t*)DW[WO]; dwout.alpha = p3.alpha;
+        dwout_later = fuse_dx ? pair_takes_third(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, D[DRESID1], G_DWQKV,
+                                                 t.X, D[DKKQQVV], DW[WKQV], dwout)
+                              : pair_takes_third(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], nullptr, G_DWQKV, t.X,
+                                                 D[DKKQQVV], DW[WKQV], dwout);
+    }
+    if (dwout_later)
+        run_gemm(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout");
+    else
+        run_gemm_pair(h, G_DXOUT, W[WO], D[DATT], D[DGAMMA], "dXout", nullptr,
+                      G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout", "dXout+dWout");
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
     half_t* DKK = sub_q(D[DKKQQVV], h, 0); half_t* DQQ = sub_q(D[DKKQQVV], h, 1); half_t* DVV = sub_q(D[DKKQQVV], h, 2);
     bool attn_bias = false;
@@ -1023,22 +1048,21 @@ void backward(Handle& h, const BwdPtrs& t) {
         run_gemm(h, G_DX1QKT, KK, D[DBETA], DQQ, "dX1QKT");
         run_gemm(h, G_DX2QKT, QQ, D[DBETA], DKK, "dX2QKT");
     }
-    const bool fuse_dx = h.fuse_epilogues && h.gemm[G_DXQKV_RESID].ok && aligned16(D[DRESID1]) &&
-                         aligned16(t.DX);
     // The last products of the pass finish the deferred column sums in workgroups of
     // their own launch when every producer of those sums has been launched by now
     // (baib below would add one more).
     FinishJobs* tail = h.deferring && attn_bias && h.finish_in_pair ? &h.deferred : nullptr;
+    PairThird* third = dwout_later ? &dwout : nullptr;
+    const char* last_name = dwout_later ? "dXQKV-fused+dWQKV-fused+dWout" : "dXQKV-fused+dWQKV-fused";
     if (fuse_dx) {
         // DX = WKQV.DKKQQVV + DRESID1 in one pass; DXATT is not written
         run_gemm_pair(h, G_DXQKV_RESID, W[WKQV], D[DKKQQVV], t.DX, "dXQKV-fused", D[DRESID1],
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail, nullptr,
-                      &h.pending_sum);
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", last_name, tail, third);
     } else {
         run_gemm_pair(h, G_DXQKV, W[WKQV], D[DKKQQVV], D[DXATT], "dXQKV-fused", nullptr,
-                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", "dXQKV-fused+dWQKV-fused", tail, nullptr,
-                      &h.pending_sum);
+                      G_DWQKV, t.X, D[DKKQQVV], DW[WKQV], "dWQKV-fused", last_name, tail, third);
     }
+    if (dwout_later && !dwout.taken) run_gemm(h, G_DWOUT, F[GAMMA], D[DATT], DW[WO], "dWout");
     if (!attn_bias) {
         ProfScope ps(h, "baib");
         op_baib(h, D[DKKQQVV], h.lb[DKKQQVV], DW[BKQV], h.lp[BKQV]);

@@ -400,12 +400,9 @@ __global__ __launch_bounds__(256) void k_gemm_mfma(GemmArgs g) {
 // one of them waits -- for its operands, at its barrier, in its first fetch or
 // its output write -- the other one runs.  Alone, each product would leave a
 // single wave on every SIMD.
-__device__ __forceinline__ void splitk_sum_block(const GemmArgs& g, long nb_total, long block);
-
 template <bool A1, bool B1, bool A2, bool B2>
-__global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2,
-                                                   FinishJobs tail, unsigned tail_groups, unsigned tail_blocks,
-                                                   GemmArgs gsum, long sum_batches) {
+__global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2, GemmArgs g3,
+                                                   unsigned n3, FinishJobs tail, unsigned tail_groups) {
     constexpr int L1 = mfma_lds_halves<2, 2, A1, B1>(), L2 = mfma_lds_halves<2, 2, A2, B2>();
     __shared__ __attribute__((aligned(16))) half_t lds[L1 > L2 ? L1 : L2];
     static_assert(sizeof(lds) >= 8 * 33 * sizeof(float) && kFinishThreads == 256, "finish_block needs this much");
@@ -413,14 +410,17 @@ __global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, uns
     // some left they alternate in groups of 8; the rest belongs to the larger one.
     const unsigned b = blockIdx.x, both = 2 * (n1 < n2 ? n1 : n2);
     if (b >= n1 + n2) {
-        // Workgroups past the tiles finish column sums of earlier launches, then add the
-        // split-k partials of an earlier product: they are dispatched last, into the
-        // places the tiles leave free on the CUs, and spare the pass two small launches.
         const unsigned t = b - (n1 + n2);
-        if (t < tail_blocks)
-            finish_block(tail.j[t / tail_groups], t % tail_groups, reinterpret_cast<float (*)[33]>(lds));
-        else
-            splitk_sum_block(gsum, sum_batches, t - tail_blocks);
+        if (t < n3) {
+            // a third product (n3 workgroups, a multiple of 8, read like the second one)
+            // in the places that the pair leaves free with two workgroups per CU
+            gemm_mfma_body<2, 2, A2, B2, true>(g3, t, n3, lds);
+        } else {
+            // Workgroups past the tiles finish column sums of earlier launches: they are
+            // dispatched last, into places that tiles leave free or vacate first, and
+            // spare the pass a launch of their own.
+            finish_block(tail.j[(t - n3) / tail_groups], (t - n3) % tail_groups, reinterpret_cast<float (*)[33]>(lds));
+        }
         return;
     }
     if (b < both) {
@@ -965,6 +965,73 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
     return per * splits;
 }
 
+namespace {
+
+// What launch_gemm_pair would launch: the two products as the kernel takes them and,
+// when one is offered and fits, a third one behind them.
+struct PairSel {
+    Canon c[2], c3;
+    long n[2] = {0, 0}, n3 = 0;
+    int variant = -1;          // instantiated orientation of the pair
+};
+
+bool pair_select(const GemmShape* const sh[2], const Canon cin[2], float* ws, size_t ws_floats,
+                 const PairThird* third, PairSel& out) {
+    bool akc[2], bkc[2], split_used = false;
+    int nkt[2];
+    for (int i = 0; i < 2; ++i) {
+        out.c[i] = cin[i];
+        const long batch = sh[i]->batch();
+        if (batch == 0 || pick_kind(out.c[i], akc[i], bkc[i]) != 1) return false;
+        GemmArgs& a = out.c[i].a;
+        if (a.M % 128 || a.N % 128 || a.K1 % BK) return false;
+        out.n[i] = (long)(a.M / 128) * (a.N / 128) * batch;
+        // a small output has its contraction split, as on its own (the scratch serves one product)
+        if (ws && !split_used && out.n[i] < 128 && (size_t)batch * a.M * a.N <= kSplitMaxOut) {
+            a.splits = pick_splits(a, batch, ws_floats);
+            if (a.splits > 1) { a.partial = ws; split_used = true; out.n[i] *= a.splits; }
+        }
+        if (out.n[i] % 8 || out.n[i] < 128 || out.n[i] > 384) return false;
+        if (pick_tile(a, batch, akc[i], bkc[i]) != 22) return false;
+        if (akc[i] && bkc[i]) return false;                  // the asynchronous kernel's products stay on their own
+        nkt[i] = a.K0 * (a.K1 / BK) / a.splits;
+    }
+    if (akc[0] && !bkc[0] && !akc[1] && !bkc[1]) out.variant = 0;
+    else if (!akc[0] && !bkc[0] && !akc[1] && !bkc[1]) out.variant = 1;
+    else if (akc[0] && !bkc[0] && akc[1] && !bkc[1]) out.variant = 2;
+    else return false;
+    // A third product rides along when its whole tiles fit into the places the pair
+    // leaves free (two workgroups per CU), it is read the way the second one is, and
+    // its contraction is not longer than theirs: the launch then takes no longer.
+    out.n3 = 0;
+    if (third && third->shape) {
+        const long batch = third->shape->batch();
+        out.c3 = canonicalise(*third->shape, third->A, third->B, third->C, third->alpha, GemmEpilogue{});
+        bool a3 = false, b3 = false;
+        const GemmArgs& a = out.c3.a;
+        if (batch > 0 && pick_kind(out.c3, a3, b3) == 1 && a.M % 128 == 0 && a.N % 128 == 0 && a.K1 % BK == 0 &&
+            a3 == akc[1] && b3 == bkc[1]) {
+            const long n3 = (long)(a.M / 128) * (a.N / 128) * batch;
+            const int nkt3 = a.K0 * (a.K1 / BK);
+            if (n3 % 8 == 0 && out.n[0] + out.n[1] + n3 <= 512 && nkt3 <= (nkt[0] > nkt[1] ? nkt[0] : nkt[1]))
+                out.n3 = n3;
+        }
+    }
+    return true;
+}
+
+}  // namespace
+
+bool gemm_pair_takes_third(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1,
+                           const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
+                           half_t* C2, const GemmEpilogue& ep2, float* ws, size_t ws_floats,
+                           const PairThird& third) {
+    const GemmShape* sh[2] = {&s1, &s2};
+    const Canon c[2] = {canonicalise(s1, A1, B1, C1, 1.f, ep1), canonicalise(s2, A2, B2, C2, 1.f, ep2)};
+    PairSel sel;
+    return pair_select(sh, c, ws, ws_floats, &third, sel) && sel.n3 > 0;
+}
+
 // Two independent products in one launch (see k_gemm_pair).  Returns false, having
 // launched nothing, unless both are products the register-staged kernel would take
 // as whole 128x128 tiles with about one tile per CU, in an operand orientation
@@ -972,35 +1039,13 @@ size_t gemm_splitk_ws_floats(const GemmShape& s) {
 bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws,
-                      size_t ws_floats, FinishJobs* tail, SplitSum* defer_sum, SplitSum* run_sum) {
-    static_assert(sizeof(GemmArgs) <= sizeof(SplitSum::args), "SplitSum holds a product's kernel arguments");
+                      size_t ws_floats, FinishJobs* tail, PairThird* third) {
     static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
     if (off) return false;
-    const float* const ws_base = ws;
-    if (run_sum && run_sum->pending && ws) {
-        // this launch's own partials go behind the ones still waiting for their sum
-        if (run_sum->floats >= ws_floats) { ws = nullptr; ws_floats = 0; }
-        else { ws += run_sum->floats; ws_floats -= run_sum->floats; }
-    }
     const GemmShape* sh[2] = {&s1, &s2};
-    Canon c[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
-    bool akc[2], bkc[2], split_used = false;
-    long n[2];
-    for (int i = 0; i < 2; ++i) {
-        const long batch = sh[i]->batch();
-        if (batch == 0 || pick_kind(c[i], akc[i], bkc[i]) != 1) return false;
-        const GemmArgs& a = c[i].a;
-        if (a.M % 128 || a.N % 128 || a.K1 % BK) return false;
-        n[i] = (long)(a.M / 128) * (a.N / 128) * batch;
-        // a small output has its contraction split, as on its own (the scratch serves one product)
-        if (ws && !split_used && n[i] < 128 && (size_t)batch * a.M * a.N <= kSplitMaxOut) {
-            c[i].a.splits = pick_splits(a, batch, ws_floats);
-            if (c[i].a.splits > 1) { c[i].a.partial = ws; split_used = true; n[i] *= c[i].a.splits; }
-        }
-        if (n[i] % 8 || n[i] < 128 || n[i] > 384) return false;
-        if (pick_tile(a, batch, akc[i], bkc[i]) != 22) return false;
-        if (akc[i] && bkc[i]) return false;                  // the asynchronous kernel's products stay on their own
-    }
+    const Canon cin[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
+    PairSel sel;
+    if (!pair_select(sh, cin, ws, ws_floats, third, sel)) return false;
     // column sums of earlier launches, finished by workgroups after the tiles (none of them
     // may be a sum that this launch itself contributes to)
     FinishJobs tj;
@@ -1009,50 +1054,27 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
         const long groups = finish_groups(*tail);
         if (groups * tail->n <= 4096) { tj = *tail; tg = (unsigned)groups; }
     }
-    const unsigned tb = (unsigned)tj.n * tg;
-    GemmArgs gsum{};
-    long sum_batches = 0, sum_blocks = 0;
-    if (run_sum && run_sum->pending) {
-        memcpy(&gsum, run_sum->args, sizeof(GemmArgs));
-        const long blocks = (run_sum->nb_total * (long)gsum.M * (gsum.N / 4) + 255) / 256;
-        if (blocks <= 8192) { sum_batches = run_sum->nb_total; sum_blocks = blocks; }
-    }
-    dim3 grid((unsigned)(n[0] + n[1] + tb + sum_blocks));
-    const unsigned n1 = (unsigned)n[0], n2 = (unsigned)n[1];
-    if (akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
-    else if (!akc[0] && !bkc[0] && !akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
-    else if (akc[0] && !bkc[0] && akc[1] && !bkc[1])
-        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, c[0].a, c[1].a, n1, n2, tj, tg, tb, gsum, sum_batches);
+    const unsigned n1 = (unsigned)sel.n[0], n2 = (unsigned)sel.n[1], n3 = (unsigned)sel.n3;
+    GemmArgs g3{};
+    if (n3) g3 = sel.c3.a;
+    dim3 grid(n1 + n2 + n3 + (unsigned)tj.n * tg);
+    const GemmArgs& g1 = sel.c[0].a;
+    const GemmArgs& g2 = sel.c[1].a;
+    if (sel.variant == 0)
+        hipLaunchKernelGGL((k_gemm_pair<true, false, false, false>), grid, dim3(256), 0, st, g1, g2, n1, n2, g3, n3, tj, tg);
+    else if (sel.variant == 1)
+        hipLaunchKernelGGL((k_gemm_pair<false, false, false, false>), grid, dim3(256), 0, st, g1, g2, n1, n2, g3, n3, tj, tg);
     else
-        return false;
+        hipLaunchKernelGGL((k_gemm_pair<true, false, true, false>), grid, dim3(256), 0, st, g1, g2, n1, n2, g3, n3, tj, tg);
     if (tj.n > 0) tail->n = 0;         // taken: nothing left for the caller to finish
-    if (sum_blocks > 0) run_sum->pending = false;
+    if (n3) third->taken = true;
     for (int i = 0; i < 2; ++i)
-        if (c[i].a.splits > 1) {
-            const long batch = sh[i]->batch(), nq = batch * (long)c[i].a.M * (c[i].a.N / 4);
-            if (defer_sum && !defer_sum->pending && c[i].a.partial == ws_base) {
-                memcpy(defer_sum->args, &c[i].a, sizeof(GemmArgs));
-                defer_sum->nb_total = batch;
-                defer_sum->floats = (size_t)batch * c[i].a.M * c[i].a.N * c[i].a.splits;
-                defer_sum->pending = true;
-                continue;
-            }
-            hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, c[i].a, batch);
+        if (sel.c[i].a.splits > 1) {
+            const long batch = sh[i]->batch(), nq = batch * (long)sel.c[i].a.M * (sel.c[i].a.N / 4);
+            hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, sel.c[i].a, batch);
         }
     check_launch("gemm pair");
     return true;
-}
-
-void launch_split_sum(SplitSum& s, hipStream_t st) {
-    if (!s.pending) return;
-    GemmArgs g;
-    memcpy(&g, s.args, sizeof(GemmArgs));
-    const long nq = s.nb_total * (long)g.M * (g.N / 4);
-    hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((nq + 255) / 256)), dim3(256), 0, st, g, s.nb_total);
-    check_launch("split-k sum");
-    s.pending = false;
 }
 
 void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C, float alpha,

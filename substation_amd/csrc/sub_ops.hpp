@@ -180,30 +180,33 @@ void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C
 // Can launch_gemm apply ep.relu_dropout to this product?  Only the asynchronous kernel with
 // 256x256 tiles does, on a single dense row-major output.
 bool gemm_relu_dropout_ok(const GemmShape& g, const void* A, const void* B, const void* C, const GemmEpilogue& ep);
-// A sum of split-k partials that has been put off: launch_gemm_pair fills it
-// instead of launching the sum, and a later launch_gemm_pair (or launch_split_sum)
-// runs it.  Until then the first `floats` elements of the scratch hold the partials.
-struct SplitSum {
-    alignas(8) unsigned char args[512];      // the product's kernel arguments
-    long nb_total = 0;
-    size_t floats = 0;
-    bool pending = false;
+// A third product offered to launch_gemm_pair: taken (and `taken` set) when its
+// whole 128x128 tiles fit into the places the pair leaves free on the CUs, it is
+// read the way the pair's second product is and its contraction is no longer
+// than theirs; the launch then takes about as long as without it.  Its
+// contraction is never split.
+struct PairThird {
+    const GemmShape* shape = nullptr;
+    const half_t* A = nullptr;
+    const half_t* B = nullptr;
+    half_t* C = nullptr;
+    float alpha = 1.f;
+    bool taken = false;
 };
-void launch_split_sum(SplitSum& s, hipStream_t st);
 // Two independent contractions in one launch, their workgroups interleaved so that
 // every CU works on both at once.  Returns false, having launched nothing, when
 // the pair does not qualify (then call launch_gemm for each).  `tail` (optional):
 // deferred column sums of EARLIER launches, finished by extra workgroups of this
 // launch; tail->n is set to 0 when they were taken, else it is left as it was.
-// `defer_sum` (optional): where to put off the sum of this launch's split-k partials
-// instead of launching it.  `run_sum` (optional): a sum put off earlier, run by
-// extra workgroups of this launch when it fits (pending is cleared then); this
-// launch's own partials go behind the pending ones in `ws`.
 bool launch_gemm_pair(const GemmShape& g1, const half_t* A1, const half_t* B1, half_t* C1, float alpha1,
                       const GemmEpilogue& ep1, const GemmShape& g2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws = nullptr,
-                      size_t ws_floats = 0, FinishJobs* tail = nullptr, SplitSum* defer_sum = nullptr,
-                      SplitSum* run_sum = nullptr);
+                      size_t ws_floats = 0, FinishJobs* tail = nullptr, PairThird* third = nullptr);
+// Would launch_gemm_pair with these two products take `third` along?
+bool gemm_pair_takes_third(const GemmShape& g1, const half_t* A1, const half_t* B1, half_t* C1,
+                           const GemmEpilogue& ep1, const GemmShape& g2, const half_t* A2, const half_t* B2,
+                           half_t* C2, const GemmEpilogue& ep2, float* ws, size_t ws_floats,
+                           const PairThird& third);
 // Scratch (in floats) that launch_gemm can make use of for this shape; 0 if none.
 size_t gemm_splitk_ws_floats(const GemmShape& g);
 // Which kernel launch_gemm would pick: 0 = scalar fallback, 1 = MFMA.

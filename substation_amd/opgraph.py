@@ -57,6 +57,7 @@ OPERATORS = [
     ('bs', 'bwd', ('ALPHA', 'ATTN_DROP_MASK', 'DATTN_DROP', 'DBETA')),
     ('dX1QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
     ('dX2QKT', 'bwd', ('KKQQVV', 'DBETA', 'DKKQQVV')),
+    ('dXQKV-fused+dWQKV-fused+dWout', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X', 'GAMMA', 'DATT', 'WO')),
     ('dXQKV-fused+dWQKV-fused', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X')),
     ('dXQKV-fused', 'bwd', ('WKQV', 'DKKQQVV', 'DXATT', 'DRESID1', 'X')),
     ('dWQKV-fused', 'bwd', ('X', 'DKKQQVV', 'WKQV')),
@@ -71,11 +72,12 @@ OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 #: which of them run depends on the layouts of the whole group's tensors.
 ALTERNATIVES = [
     ('QKV-fused', 'aib'),
-    ('dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei'),
+    # dWout runs inside the last launch of the pass when that has room for its tiles
+    ('dXQKV-fused+dWQKV-fused+dWout', 'dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei',
+     'dXout+dWout', 'dXout', 'dWout'),
     ('lin1+bad', 'lin1', 'bad'),
     ('dXlin2+bdrlb', 'dXlin2', 'bdrlb'),
     ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
-    ('dXout+dWout', 'dXout', 'dWout'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
     ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT',
      'baib'),

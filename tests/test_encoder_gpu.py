@@ -509,8 +509,9 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
 def test_column_sums_finished_inside_the_last_pair_launch_are_bit_identical(dims, activation):
     """The second stage of the column sums (bias and LayerNorm-parameter gradients)
     runs in extra workgroups of the last pair of products of the backward pass
-    (option 7) instead of in a launch of its own: every gradient must be equal bit
-    for bit, twice in a row (the deferred list is rebuilt per call).  The smallest
+    (option 7) instead of in a launch of its own, and so does dWout where that launch
+    has room for its tiles: every gradient must be equal bit for bit (DWO to rounding),
+    twice in a row (the deferred list is rebuilt per call).  The smallest
     case does not qualify for a pair launch and takes the separate launch either
     way."""
     from substation_amd import Encoder, layouts as L
@@ -541,7 +542,12 @@ def test_column_sums_finished_inside_the_last_pair_launch_are_bit_identical(dims
         outs.append(got)
     for (name, a), (_, b) in zip(*outs):
         assert torch.isfinite(a.float()).all()
-        assert torch.equal(a, b), name
+        if name == 'DWO':
+            # dWout runs inside that launch too, with its contraction in one piece instead
+            # of four: the same terms added in another order
+            assert_close(b.float().cpu().numpy(), a.float().cpu().numpy(), tol=2e-3, name=name)
+        else:
+            assert torch.equal(a, b), name
     assert all(float(a.abs().max()) > 0 for name, a in outs[1] if name in ('DBKQV', 'DBO', 'DS1', 'DB2', 'DLINB1'))
 
 
