@@ -203,8 +203,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
 /* SUB_OPT_FINISH_IN_PAIR (default 1): the second stage of the column sums of
  * encoder_backward (adding the per-chunk fp32 partials of the bias and
  * LayerNorm-parameter gradients) runs in extra workgroups of the last pair of
- * products of the pass, which its last, partly filled round of tiles leaves
- * room for, instead of in a launch of its own (same code, same order of
+ * products of the pass, in the places its tiles leave free on the CUs (two
+ * workgroups each), instead of in a launch of its own (same code, same order of
  * additions: bit-identical).  Where that launch also has room for the tiles of
  * the dWout product, dWout runs there with its contraction in one piece and
  * dXout runs alone (DWO then sums its terms in another order than with the
