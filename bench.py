@@ -1,13 +1,16 @@
 """Benchmark of the fused encoder layer on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3|4|5] [--layouts mi355x|ref]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 2|3|4|5] [--layouts mi355x|ref]
 
 A step is one forward + one backward pass of a single encoder layer over one
 batch of synthetic input (the protocol of pytorch_module/run_encoder.py:345-383).
 The default workload is BERT-large B=8 L=512 H=16 E=1024 fp16 with the four
-dropouts at p=0.1.  Prints ONE JSON line: ms per layer, the per-operator
+dropouts at p=0.1.  Prints ONE JSON line: ms per layer, the per-launch
 roofline measured live with HIP events on the launch stream, and the CPU
-baseline (the NumPy oracle on the reference's own CPU-sized case).
+baseline (the NumPy oracle on the bench workload and on the reference's own
+CPU-sized case).  --config 2 times the fused operators on their own (softmax
+and its backward at [H=16,B=8,J=512,K=512], and every other memory-bound
+operator at the default workload's shapes) and prints their line instead.
 """
 import argparse
 import json
@@ -34,15 +37,29 @@ CONFIGS = {
             name='configs[4]: wide encoder layer fwd+bwd B=4 L=2048 H=32 E=4096 P=128 FF=16384 GELU fp16'),
 }
 
-# HBM-side bytes per launch at the default workload and layouts: rocprofv3 FETCH_SIZE (x2.000) +
-# WRITE_SIZE (x1.000), scale factors from a 256 MiB device copy; see
-# profiles/encoder_layer_b8_l512_hbm_traffic.txt for the commands and the table.
-MEASURED_TRAFFIC_CFG3 = {
-    'QKV-fused': 91452057, 'attention': 38114912, 'out': 33775005, 'bdrln1': 59014043,
-    'lin1+bad': 87734212, 'lin2': 109264774, 'bdrln2': 59016749, 'bsb+blnrd1': 61022384,
-    'dXlin2+bdrlb': 118260844, 'dWlin2': 109269143, 'dXlin1+dWlin1': 298726901, 'ebsb+blnrd2+baob': 79940065,
-    'dXout': 33752717, 'attention-bwd-dQ': 55316836, 'attention-bwd-dKdV': 55518567, 'dXQKV-fused+dWQKV-fused+dWout': 373479999,
-}
+TRAFFIC_PROFILE = os.path.join(ROOT, 'profiles', 'encoder_layer_b8_l512_hbm_traffic.txt')
+
+
+def measured_traffic(path=TRAFFIC_PROFILE):
+    """launch name -> HBM-side bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by a
+    copy of known size) read from the tracked rocprofv3 summary of this workload; {} when the
+    file is not there.  Table rows are `name fetch-MiB write-MiB total-MiB algorithmic-MiB ratio`."""
+    out = {}
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return out
+    for line in lines:
+        f = line.split()
+        if len(f) != 6:
+            continue
+        try:
+            nums = [float(x) for x in f[1:]]
+        except ValueError:
+            continue
+        out[f[0]] = int(round(nums[2] * (1 << 20)))
+    return out
+
 
 GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1',
             'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
@@ -64,6 +81,9 @@ def algorithmic_work(B, L, H, E, relu_from_output=True):
         'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', (2 if relu_from_output else 4) * bju * 2),
         'bdrlb': ('hbm', (3 if relu_from_output else 4) * bju * 2),
         'baib': ('hbm', q * 2),
+        # second stage of the column sums when it runs as a launch of its own: fp32 partial rows
+        # in, a few vectors out (not one of the reference's operators: no algorithmic bytes)
+        'colfinish': ('hbm', 0),
         # single-launch forms: the scaled gradient is written but not read back
         # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
         'bsb+blnrd1': ('hbm', 7 * bji * 2), 'ebsb+blnrd2+baob': ('hbm', 9 * bji * 2),
@@ -191,7 +211,229 @@ def cpu_baseline(cfg, budget_s=20.0):
         'value': round(statistics.median(times) * 1e3 * scale_b, 1), 'unit': 'ms/layer', 'cores': threads,
         'kind': 'port',
         'sample': f'NumPy oracle on the bench workload shape {what}; host has {os.cpu_count()} logical CPUs',
+        'config1': cpu_baseline_config1(),
     }
+
+
+def cpu_baseline_config1(warmups=3, runs=10):
+    """BASELINE configs[0], the reference's own CPU-runnable case: B=2 L=128 H=12 E=768 P=64
+    FF=3072 post-LN ReLU fp32, X, dY ~ N(0,1), weights N(0,0.02), biases 0, gamma=1, beta=0,
+    p=0.1 masks from the seed; forward + backward, time.perf_counter, 3 warm-ups, median of 10.
+    Two implementations side by side: the NumPy oracle (per-sample np.matmul structure of
+    substation/transformer.py:176-285) and torch.nn.TransformerEncoderLayer on the CPU (what
+    test/test_transformer_torch.py:280-340 checks the NumPy path against)."""
+    import numpy as np
+    import torch
+    from oracle import encoder_ref as ref
+    B, L, H, E = 2, 128, 12, 768
+    U, P = 4 * E, E // H
+    rng = np.random.default_rng(1001)
+    f32 = np.float32
+    params = dict(
+        WKQV=(0.02 * rng.normal(size=(3, P, H, E))).astype(f32), BKQV=np.zeros((3, P, H), f32),
+        WO=(0.02 * rng.normal(size=(E, P, H))).astype(f32), BO=np.zeros(E, f32),
+        S1=np.ones(E, f32), B1=np.zeros(E, f32), LINB1=np.zeros(U, f32),
+        LINW1=(0.02 * rng.normal(size=(E, U))).astype(f32), S2=np.ones(E, f32), B2=np.zeros(E, f32),
+        LINB2=np.zeros(E, f32), LINW2=(0.02 * rng.normal(size=(U, E))).astype(f32))
+    X = rng.normal(size=(B, L, E)).astype(f32); DY = rng.normal(size=(B, L, E)).astype(f32)
+    a = ref.module_params_to_numpy(params)
+    scale = f32(1.0 / np.sqrt(P))
+    keep = lambda shape: (rng.random(shape, dtype=f32) >= f32(0.1)).astype(f32)
+    mk = dict(softmax_mask=keep((B, H, L, L)), attn_dropout_mask=keep((B, L, E)),
+              linear1_dropout_mask=keep((B, L, U)), ff_dropout_mask=keep((B, L, E)))
+
+    def numpy_step():
+        f = ref.encoder(X, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], a['attn_in_b'],
+                        a['attn_out_b'], scale, a['norm1_scale'], a['norm1_bias'], a['norm2_scale'],
+                        a['norm2_bias'], a['linear1_w'], a['linear1_b'], a['linear2_w'], a['linear2_b'],
+                        activation='relu', **mk)
+        ref.encoder_backward(X, DY, f, a['attn_wq'], a['attn_wk'], a['attn_wv'], a['attn_wo'], scale,
+                             a['norm1_scale'], a['norm2_scale'], a['linear1_w'], a['linear1_b'],
+                             a['linear2_w'], a['linear2_b'], activation='relu', **mk)
+
+    torch.manual_seed(1001)
+    layer = torch.nn.TransformerEncoderLayer(E, H, U, dropout=0.1, activation='relu')     # post-LN, [L, B, E]
+    layer.train()
+    xt = torch.from_numpy(X).transpose(0, 1).contiguous().requires_grad_(True)
+    dyt = torch.from_numpy(DY).transpose(0, 1).contiguous()
+
+    def torch_step():
+        xt.grad = None
+        layer.zero_grad(set_to_none=True)
+        layer(xt).backward(dyt)
+
+    def median_ms(fn):
+        for _ in range(warmups):
+            fn()
+        ts = []
+        for _ in range(runs):
+            t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+        return round(statistics.median(ts) * 1e3, 2)
+
+    try:
+        from threadpoolctl import threadpool_info
+        blas = sorted({f"{q.get('internal_api')} {q.get('num_threads')} threads" for q in threadpool_info()})
+    except Exception:
+        blas = []
+    return {'workload': 'configs[0]: B=2 L=128 H=12 E=768 P=64 FF=3072 post-LN ReLU fp32 fwd+bwd, p=0.1',
+            'numpy_oracle_ms': median_ms(numpy_step), 'torch_cpu_ms': median_ms(torch_step),
+            'protocol': f'time.perf_counter, {warmups} warm-ups, median of {runs}',
+            'logical_cpus': os.cpu_count(), 'torch_threads': torch.get_num_threads(),
+            'omp_num_threads': os.environ.get('OMP_NUM_THREADS'), 'blas': blas}
+
+
+def bench_fused_ops(args):
+    """BASELINE configs[1] and the other memory-bound operators on their own, through the
+    operator entry points of the C ABI (the units pytorch_module/benchmark.py times, whose
+    shipped results are perf_softmax.txt, perf_bad.txt, perf_bsb.txt, perf_bdrln.txt):
+    softmax forward (scale 1/8, p=0.1 seeded) and its backward on scores [H=16,B=8,J=512,K=512],
+    every other operator at the shapes of B=8 L=512 E=1024 FF=4096.  Each operator cycles over
+    enough buffer sets to exceed the 256 MiB memory-side cache; the launches of one round are
+    recorded in a HIP graph and replayed, so that the HIP events around the replays time the
+    GPU and not the Python caller.  GB/s = algorithmic bytes (each big tensor read once and
+    written once) / time."""
+    import torch
+    from substation_amd.ops import Ops
+    B, L, H, E = 8, 512, 16, 1024
+    U = 4 * E
+    o = Ops(B, L, H, E, activation='relu', seed=0x5EED + 2)
+    g = torch.Generator(device='cuda').manual_seed(1002)
+    bytes_of = {'HBJK': H * B * L * L * 2, 'BJI': B * L * E * 2, 'BJU': B * L * U * 2, 'QBJHP': 3 * B * L * E * 2}
+
+    def randn(layout, std=1.0):
+        t = o.empty(layout)
+        t.normal_(0.0, std, generator=g)
+        return t
+
+    def vec(n, std=0.02, mean=0.0):
+        return torch.empty(n, dtype=torch.float16, device='cuda').normal_(mean, std, generator=g)
+
+    def keepmask(layout):
+        return (torch.rand(o.empty(layout).shape, device='cuda', generator=g) >= 0.1).half()
+
+    # operator -> (algorithmic tensors moved, their layout, make(): one buffer set, run(set))
+    def softmax_set():
+        return dict(beta=randn('HBJK'), alpha=o.empty('HBJK'), mask=o.empty('HBJK'), drop=o.empty('HBJK'))
+
+    def bs_set():
+        d = softmax_set()
+        o.softmax(d['beta'], 'HBJK', d['alpha'], 'HBJK', d['mask'], 'HBJK', d['drop'], 'HBJK', scale=0.125, p=0.1)
+        return dict(alpha=d['alpha'], mask=d['mask'], ddrop=randn('HBJK'), dbeta=d['beta'])
+
+    def bdrln_set():
+        return dict(inp=randn('BJI'), resid=randn('BJI'), lb=vec(E), s=vec(E, 0.1, 1.0), b=vec(E), mask=o.empty('BJI'),
+                    diff=o.empty('BJI'), normed=o.empty('BJI'), out=o.empty('BJI'), istd=o.empty('BJ'))
+
+    def blnrd_set():
+        return dict(dout=randn('BJI'), istd=randn('BJ').abs_().add_(0.5), diff=randn('BJI'), mask=keepmask('BJI'),
+                    a=o.empty('BJI'), b=o.empty('BJI'))
+
+    def lnbwd_set(ext):
+        d = dict(inp=randn('BJI'), s=vec(E, 0.1, 1.0), d1=randn('BJI'), istd=randn('BJ').abs_().add_(0.5),
+                 diff=randn('BJI'), mask=keepmask('BJI'), g=o.empty('BJI'), a=o.empty('BJI'), b=o.empty('BJI'),
+                 ds=vec(E), db=vec(E))
+        if ext:
+            d.update(d2=randn('BJI'), dl=randn('BJI'), dlb=vec(E), dob=vec(E))
+        return d
+
+    def run_lnbwd(d):
+        if 'd2' in d:
+            o.ln_backward(d['inp'], 'BJI', d['s'], d['d1'], 'BJI', d['istd'], 'BJ', d['diff'], 'BJI', d['mask'], 'BJI',
+                          d['g'], 'BJI', d['a'], 'BJI', d['b'], 'BJI', d['ds'], d['db'], dout2=d['d2'], l_dout2='BJI',
+                          dlinear=d['dl'], l_dlinear='BJI', dlinear_bias=d['dlb'], dout_bias=d['dob'])
+        else:
+            o.ln_backward(d['inp'], 'BJI', d['s'], d['d1'], 'BJI', d['istd'], 'BJ', d['diff'], 'BJI', d['mask'], 'BJI',
+                          d['g'], 'BJI', d['a'], 'BJI', d['b'], 'BJI', d['ds'], d['db'])
+
+    specs = [
+        ('softmax', 4, 'HBJK', softmax_set,
+         lambda d: o.softmax(d['beta'], 'HBJK', d['alpha'], 'HBJK', d['mask'], 'HBJK', d['drop'], 'HBJK',
+                             scale=0.125, p=0.1)),
+        ('bs', 4, 'HBJK', bs_set,
+         lambda d: o.bs(d['alpha'], 'HBJK', d['mask'], 'HBJK', d['ddrop'], 'HBJK', d['dbeta'], 'HBJK', scale=0.125)),
+        ('bdrln', 7, 'BJI', bdrln_set,
+         lambda d: o.bdrln(d['inp'], 'BJI', d['resid'], 'BJI', d['lb'], d['s'], d['b'], d['inp'], 'BJI', d['mask'], 'BJI',
+                           d['diff'], 'BJI', d['normed'], 'BJI', d['out'], 'BJI', d['istd'], 'BJ', p=0.1, site=1)),
+        ('blnrd', 5, 'BJI', blnrd_set,
+         lambda d: o.blnrd(d['dout'], 'BJI', d['istd'], 'BJ', d['diff'], 'BJI', d['mask'], 'BJI', d['a'], 'BJI',
+                           d['b'], 'BJI')),
+        ('bad', 4, 'BJU', lambda: dict(inp=randn('BJU'), bias=vec(U), lin=o.empty('BJU'), mask=o.empty('BJU'),
+                                       out=o.empty('BJU')),
+         lambda d: o.bad(d['inp'], 'BJU', d['bias'], d['lin'], 'BJU', d['mask'], 'BJU', d['out'], 'BJU', p=0.1, site=2)),
+        ('bdrlb', 4, 'BJU', lambda: dict(dd=randn('BJU'), mask=keepmask('BJU'), lin=randn('BJU'), dl=o.empty('BJU'),
+                                         db=vec(U)),
+         lambda d: o.bdrlb(d['dd'], 'BJU', d['mask'], 'BJU', d['lin'], 'BJU', d['dl'], 'BJU', d['db'])),
+        ('bsb', 3, 'BJI', lambda: dict(inp=randn('BJI'), s=vec(E, 0.1, 1.0), dout=randn('BJI'), din=o.empty('BJI'),
+                                       ds=vec(E), db=vec(E)),
+         lambda d: o.bsb(d['inp'], 'BJI', d['s'], d['dout'], 'BJI', d['din'], 'BJI', d['ds'], d['db'])),
+        ('ebsb', 5, 'BJI', lambda: dict(inp=randn('BJI'), s=vec(E, 0.1, 1.0), d1=randn('BJI'), d2=randn('BJI'),
+                                        dl=randn('BJI'), din=o.empty('BJI'), ds=vec(E), db=vec(E), dlb=vec(E)),
+         lambda d: o.ebsb(d['inp'], 'BJI', d['s'], d['d1'], 'BJI', d['d2'], 'BJI', d['dl'], 'BJI', d['din'], 'BJI',
+                          d['ds'], d['db'], d['dlb'])),
+        ('bsb+blnrd', 7, 'BJI', lambda: lnbwd_set(False), run_lnbwd),
+        ('ebsb+blnrd+baob', 9, 'BJI', lambda: lnbwd_set(True), run_lnbwd),
+        ('baob', 1, 'BJI', lambda: dict(d=randn('BJI'), o=vec(E)), lambda d: o.baob(d['d'], 'BJI', d['o'])),
+        ('aib', 2, 'QBJHP', lambda: dict(i=randn('QBJHP'), b=o.empty('QHP').normal_(0, 0.02, generator=g),
+                                         o=o.empty('QBJHP')),
+         lambda d: o.aib(d['i'], 'QBJHP', d['b'], 'QHP', d['o'], 'QBJHP')),
+        ('baib', 1, 'QBJHP', lambda: dict(d=randn('QBJHP'), o=o.empty('QHP')),
+         lambda d: o.baib(d['d'], 'QBJHP', d['o'], 'QHP')),
+        ('bei', 3, 'BJI', lambda: dict(a=randn('BJI'), b=randn('BJI'), o=o.empty('BJI')),
+         lambda d: o.bei(d['a'], 'BJI', d['b'], 'BJI', d['o'], 'BJI')),
+    ]
+    rows = []
+    for name, ntens, layout, make, run in specs:
+        nbytes = ntens * bytes_of[layout]
+        nsets = max(2, -(-(640 << 20) // nbytes))            # > 2.5 x the memory-side cache in rotation
+        sets = [make() for _ in range(nsets)]
+        for d in sets:                                        # warm-up; also allocates the handle's scratch
+            run(d)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                for d in sets:
+                    run(d)
+        torch.cuda.synchronize()
+        for _ in range(max(1, args.warmup // 10)):
+            graph.replay()
+        reps = max(3, args.steps // 10)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / (reps * nsets)
+        rows.append(dict(op=name, bound='hbm', us=round(t * 1e6, 2), achieved=round(nbytes / t / 1e9, 1),
+                         unit='GB/s', frac=round(nbytes / t / HBM_PEAK, 4), bytes=nbytes, buffer_sets=nsets))
+        del sets, graph
+        torch.cuda.empty_cache()
+    if args.per_op:
+        for r in rows:
+            print(json.dumps(r), file=sys.stderr)
+    sm = [r for r in rows if r['op'] in ('softmax', 'bs')]
+    t_sm = sum(r['us'] for r in sm) * 1e-6
+    b_sm = sum(r['bytes'] for r in sm)
+    dom = max(sm, key=lambda r: r['us'])
+    out = {
+        'metric': 'fused-op HBM GB/s vs peak: softmax forward + backward alone, [H=16,B=8,J=512,K=512] fp16',
+        'value': round(b_sm / t_sm / 1e9, 1), 'unit': 'GB/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(t_sm * 1e3, 4), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'fp16', 'data': 'synthetic',
+        'config': {'workload': 'configs[1]: softmax (scale 1/8, dropout p=0.1 seeded) + softmax backward on scores '
+                               '[16,8,512,512]; the other fused operators at B=8 L=512 E=1024 FF=4096, each alone'},
+        'roofline': {'kernel': dom['op'], 'bound': 'hbm', 'achieved': dom['achieved'], 'peak': HBM_PEAK / 1e9,
+                     'unit': 'GB/s', 'frac': dom['frac'], 'traffic': None, 'launch_us': dom['us']},
+        'reference_published_us': {'softmax (1 read + 1 write, no dropout outputs)': 187.97, 'bad (p=0)': 91.45,
+                                   'bsb': 72.97, 'bdrln (p=0)': 51.53,
+                                   'source': 'pytorch_module/perf_softmax.txt, perf_bad.txt, perf_bsb.txt, '
+                                             'perf_bdrln.txt (GPU not stated)'},
+        'ops': [{k: r[k] for k in ('op', 'us', 'achieved', 'unit', 'frac', 'bytes', 'buffer_sets')} for r in rows],
+    }
+    print(json.dumps(out))
 
 
 def bench_decoder(cfg, args):
@@ -234,7 +476,7 @@ def main():
     ap.add_argument('--gpus', type=int, default=1)
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=30)
-    ap.add_argument('--config', type=int, default=3, choices=sorted(CONFIGS))
+    ap.add_argument('--config', type=int, default=3, choices=[2] + sorted(CONFIGS))
     ap.add_argument('--layouts', default='mi355x', choices=['mi355x', 'ref'])
     ap.add_argument('--profile-steps', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
@@ -259,6 +501,9 @@ def main():
         print('bench.py: no GPU visible', file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.config == 2:
+        bench_fused_ops(args)
+        return
     cfg = CONFIGS[args.config]
     if args.decoder:
         bench_decoder(cfg, args)
@@ -294,18 +539,15 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    # Per-operator durations: HIP events recorded by the library around every
-    # launch, on the stream the kernels run on.
+    # Per-launch durations: HIP events recorded by the library around every launch, on the
+    # stream the kernels run on; the launches are the timed region's.  Two steps are issued
+    # back to back and the events of the second are read after its backward pass, so that
+    # no start event sits on an idle stream (host time before a launch would land in it).
     enc._handle.profile_enable(True)
     per_op = {}
     for _ in range(args.profile_steps):
-        X.grad = None
-        for q in params:
-            q.grad = None
-        Y = enc(X)
-        for n, ms in enc.profile():
-            per_op.setdefault(n, []).append(ms)
-        Y.backward(DY)
+        step()
+        step()
         for n, ms in enc.profile():
             per_op.setdefault(n, []).append(ms)
     enc._handle.profile_enable(False)
@@ -350,8 +592,8 @@ def main():
         'roofline': {
             'kernel': dom['op'], 'bound': dom['bound'], 'achieved': dom['achieved'], 'peak': dom['peak'],
             'unit': dom['unit'], 'frac': dom['frac'],
-            'traffic': (MEASURED_TRAFFIC_CFG3.get(dom['op']) if args.config == 3 and args.layouts == 'mi355x'
-                        else None),
+            'traffic': (measured_traffic().get(dom['op']) if args.config == 3 and args.layouts == 'mi355x'
+                        and not args.option else None),
             'launch_us': dom['us'], 'launches_per_step': 1,
         },
         'op_time_us': round(total_us, 1),

@@ -227,9 +227,12 @@ int sub_encoder_forward(void* handle, void* const* ptrs, int n);
 int sub_encoder_backward(void* handle, void* const* ptrs, int n);
 
 /* Per-operator timing with HIP events on the handle's stream; the counterpart
- * of the NVTX ranges of encoder.cu:32-53.  sub_profile_read waits for the
- * stream and returns the number of operators of the last forward/backward call
- * (at most cap are written). */
+ * of the NVTX ranges of encoder.cu:32-53.  The launches are the same with timing
+ * on as with it off.  sub_profile_read waits for the stream and returns the number
+ * of launches of the last encoder_forward call followed, if one has been issued
+ * since, by those of the encoder_backward call after it (at most cap are
+ * written); reading only after the backward call leaves no host wait between
+ * the two passes. */
 int sub_profile_enable(void* handle, int on);
 int sub_profile_read(void* handle, int cap, const char** names, float* ms);
 

@@ -412,7 +412,7 @@ def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', rel
     alpha = np.einsum('BHJK->HBJK', np.stack(f['attn_scaled_scores']))
     out['ALPHA'] = alpha
     out['ATTN_DROP'] = np.einsum('BHJK->HBJK', np.stack(f['attn_drop']))
-    out['BETA'] = scale * np.einsum('BHJP,BHKP->HBJK', pq, pk)
+    out['BETA'] = scale * np.einsum('BHJK->HBJK', np.matmul(pq, np.swapaxes(pk, -1, -2)))
     out['GAMMA'] = np.einsum('BJHP->PHBJ', np.stack(f['attn_concat']).reshape(B, J, H, P))
     out['ATT'] = f['attn']                                   # biased, as stored in place
     out['LN1DIFF'] = f['attn_resid'] - f['norm1_mean']
@@ -445,9 +445,10 @@ def run_named(params, X, DY, masks=None, activation='relu', ln_mode='rsqrt', rel
     out['DGAMMA'] = np.einsum('BJHP->PHBJ', dgamma)
     # DKKQQVV from the bias-gradient-free definition: grads of the projections
     dbeta_b = np.stack(g['dbeta'])
-    dpq = scale * np.einsum('BHJK,BHKP->BHJP', dbeta_b, pk)
-    dpk = scale * np.einsum('BHJK,BHJP->BHKP', dbeta_b, pq)
-    dpv = np.einsum('BHJK,BHJP->BHKP', np.stack(f['attn_drop']), np.einsum('BJHP->BHJP', dgamma))
+    # (batched matmul: the same sums as 'BHJK,BHKP->BHJP', 'BHJK,BHJP->BHKP' twice)
+    dpq = scale * np.matmul(dbeta_b, pk)
+    dpk = scale * np.matmul(np.swapaxes(dbeta_b, -1, -2), pq)
+    dpv = np.matmul(np.swapaxes(np.stack(f['attn_drop']), -1, -2), np.einsum('BJHP->BHJP', dgamma))
     out['DKKQQVV'] = np.stack([np.einsum('BHJP->PHBJ', t) for t in (dpk, dpq, dpv)])
     # outputs and parameter gradients
     out['DX'] = g['dx']

@@ -192,6 +192,7 @@ struct Handle {
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
+    size_t prof_forward = 0;          // entries of the last forward call, kept by the backward call after it
 
     ~Handle() {
         // A handle may be destroyed (e.g. by a garbage collector) while some other
@@ -311,6 +312,13 @@ void configure(Handle& h, const sub_config* c) {
     const float ps[4] = {c->p_softmax, c->p_resid1, c->p_act, c->p_resid2};
     for (float p : ps) if (!(p >= 0.f && p <= 1.f)) fail("sub_configure: dropout probability outside [0,1]");
     h.configured = false;
+    // a handle that is configured again forgets the attention mask of its old sizes
+    // (the table of what the mask leaves to do was sized for them)
+    if (h.mask_plan) {
+        refuse_capture(h, "sub_configure");
+        hip_check(hipFree(h.mask_plan), "hipFree(mask plan)");
+    }
+    h.mask_plan = nullptr; h.mask_plan_bytes = 0; h.mask_plan_built = false; h.attn_mask = nullptr;
     Sizes sz;
     sz.n[dB] = c->batch; sz.n[dJ] = c->seq; sz.n[dK] = c->seq; sz.n[dH] = c->heads;
     sz.n[dP] = c->embed / c->heads; sz.n[dI] = c->embed;
@@ -808,6 +816,7 @@ __global__ void k_step_increment(uint32_t* step) {
 void forward(Handle& h, const FwdPtrs& t) {
     if (!h.configured) fail("encoder_forward: handle is not configured");
     h.prof_used = 0;
+    h.prof_forward = 0;
     void* const* W = t.W; void* const* F = t.F;
     if (h.fuse_epilogues && h.gemm[G_QKV_BIAS].ok && aligned16(W[BKQV]) && aligned16(F[KKQQVV])) {
         // projection + bias in one pass; WKKWQQWVV (the pre-bias copy) is not written
@@ -877,17 +886,21 @@ void forward(Handle& h, const FwdPtrs& t) {
     } else {
         h.step += 1;
     }
+    h.prof_forward = h.prof_used;
 }
 
 void backward(Handle& h, const BwdPtrs& t) {
     if (!h.configured) fail("encoder_backward: handle is not configured");
-    h.prof_used = 0;
+    // the first backward call after a forward call keeps that call's entries in front of its own
+    h.prof_used = h.prof_forward;
+    h.prof_forward = 0;
     // The five bias / scale gradients are only consumed by the caller: their
     // reductions leave fp32 partials in separate scratch regions and one launch
-    // at the end of the pass finishes them all.  (With per-operator timing on,
-    // each finishes on its own so that its time is attributed to it.)
+    // at the end of the pass finishes them all (or workgroups of the last pair of
+    // products do).  Per-operator timing times this same schedule: the finishing
+    // stage is part of the launch that carries it, or an entry of its own.
     ensure_ws(h, h.ws_need_bwd);
-    h.deferring = !h.profiling;
+    h.deferring = true;
     h.ws_cursor = 0;
     h.deferred.n = 0;
     struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
@@ -1071,7 +1084,10 @@ void backward(Handle& h, const BwdPtrs& t) {
         ProfScope ps(h, "bei");
         op_bei(h, D[DXATT], h.lb[DXATT], D[DRESID1], h.lb[DRESID1], t.DX, h.lX);
     }
-    if (h.deferring) launch_colfinish(h.deferred, h.stream);
+    if (h.deferred.n > 0) {
+        ProfScope ps(h, "colfinish");
+        launch_colfinish(h.deferred, h.stream);
+    }
 }
 
 void unpack_forward(const Handle& h, void* const* p, FwdPtrs& t) {

@@ -71,14 +71,6 @@ __global__ __launch_bounds__(256) void k_gemm_scalar(GemmArgs g, long total) {
 // ---------------------------------------------------------------------------
 constexpr int BK = 64;            // k per LDS tile
 
-#ifdef SUB_GEMM_ABLATE
-// Performance experiments only (results are wrong): bit 0 skips the global
-// loads and LDS writes after the first tile, bit 1 skips the fragment reads.
-__device__ int g_ablate = 0;
-#define SUB_ABLATE(bit) (g_ablate & (bit))
-#else
-#define SUB_ABLATE(bit) 0
-#endif
 constexpr int MC_PAD = 32;        // halves of padding per k-row of a free-dim-contiguous tile
 
 typedef short s4v __attribute__((ext_vector_type(4)));
@@ -282,7 +274,7 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id,
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
             fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
-            if (ks + 1 < BK / 16 && !SUB_ABLATE(2)) {                                             \
+            if (ks + 1 < BK / 16) {                                                               \
                 _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
                     fa[(ks + 1) & 1][i] = TA::frag(sA, (wm * TM + i) * 32, ks + 1, lane);         \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
@@ -310,15 +302,14 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id,
 
     // Step 2p: stage 0 holds tile 2p, set 1 holds tile 2p+1 in flight, set 0 is free.
     const int npairs = nkt >> 1;
-    const bool mem = !SUB_ABLATE(1);
     for (int p = 0; p < npairs; ++p) {
-        if (mem) SUB_GEMM_ISSUE(ra0, rb0);        // tile 2p+2
+        SUB_GEMM_ISSUE(ra0, rb0);                 // tile 2p+2
         SUB_GEMM_COMPUTE(0);
-        if (mem) SUB_GEMM_STORE(1, ra1, rb1);     // tile 2p+1
+        SUB_GEMM_STORE(1, ra1, rb1);              // tile 2p+1
         __syncthreads();
-        if (mem) SUB_GEMM_ISSUE(ra1, rb1);        // tile 2p+3
+        SUB_GEMM_ISSUE(ra1, rb1);                 // tile 2p+3
         SUB_GEMM_COMPUTE(1);
-        if (mem) SUB_GEMM_STORE(0, ra0, rb0);     // tile 2p+2 (a surplus copy when 2p+2 == nkt)
+        SUB_GEMM_STORE(0, ra0, rb0);              // tile 2p+2 (a surplus copy when 2p+2 == nkt)
         __syncthreads();
     }
     if (nkt & 1) {

@@ -293,9 +293,9 @@ class Encoder(torch.nn.Module):
         return counter
 
     def profile(self):
-        """Per-operator times in ms of the last forward or backward call
-        (``profiling=True`` only); the counterpart of the NVTX ranges of
-        pytorch_module/encoder.cu:32-53."""
+        """Per-launch times in ms of the last forward call and, once it has been
+        issued, of the backward call after it (``profiling=True`` only); the
+        counterpart of the NVTX ranges of pytorch_module/encoder.cu:32-53."""
         return self._handle.profile_read()
 
     def forward(self, X):

