@@ -327,6 +327,28 @@ int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l
                        const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
                        const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
                        const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias);
+/* sub_op_ln_backward for callers that cannot allocate device memory -- code under a
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments, same kernels and bit-identical
+ * results; the fp32 partial rows of the column sums (which sub_op_ln_backward keeps
+ * in a buffer the handle allocates on first use) live in a 4 MiB array that is part
+ * of the library's device image, one copy per GPU for the life of the process.
+ * Nothing is allocated or freed.  A call whose partial rows would need more than
+ * SUB_STATIC_SCRATCH_BYTES fails with a message, launching nothing; the way the
+ * rows are dealt out keeps every shape this operator takes within it (at most 256
+ * partial rows of up to 1024 features for each of four sums in the one-launch form,
+ * at most 3 MiB for the separate operators on longer rows).  All calls on one GPU, from
+ * whatever handle or stream, share the array: calls that may overlap on a GPU race.
+ * The first call on a GPU looks the array's address up (no allocation); make it
+ * outside a graph capture. */
+#define SUB_STATIC_SCRATCH_BYTES (4u << 20)
+int sub_op_ln_backward_static(void* handle, int extended, const void* in, const char* l_in, const void* scale,
+                              const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                              const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
+                              const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
+                              const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                              const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias,
+                              void* dout_bias);
 /* block_bei.cuh:58-106 */
 int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void* dresid1,
                const char* l_dresid1, void* dx, const char* l_dx);

@@ -86,6 +86,8 @@ SIGNATURES = {
     'sub_op_bei': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
     'sub_op_ln_backward': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP,
                                 _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
+    'sub_op_ln_backward_static': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP,
+                                       _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
     'sub_op_einsum': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_einsum_add': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_layout_strides': (_I, [_VP, _CP, ctypes.POINTER(ctypes.c_int64)]),

@@ -7,12 +7,23 @@
 
 #include <cmath>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
 #include "../../include/substation_amd.h"
 #include "sub_common.hpp"
 #include "sub_ops.hpp"
+
+// Scratch of the entry point that allocates nothing (sub_op_ln_backward_static):
+// the fp32 partial rows of its column sums live in this array instead of in a
+// buffer from hipMalloc.  Every GPU the library runs on holds its own copy, at
+// its own address, until the process ends.  In host code the array's name is
+// only a handle for hipGetSymbolAddress, never a device address: host code
+// hands the resolved pointer (static_scratch() below), and nothing else, to
+// kernels.
+constexpr size_t kStaticScratchFloats = SUB_STATIC_SCRATCH_BYTES / sizeof(float);     // 4 MiB
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
 
 namespace sub {
 
@@ -171,6 +182,7 @@ struct Handle {
     float* ws = nullptr;          // column-reduction partials
     size_t ws_floats = 0;
     size_t ws_need_bwd = 0;       // sum over the backward pass's column reductions
+    float* static_ws = nullptr;   // set for the duration of a call that must not allocate: take_ws hands it out
     bool deferring = false;       // backward pass: finish all column reductions in one launch
     size_t ws_cursor = 0;
     FinishJobs deferred;
@@ -210,6 +222,26 @@ struct Handle {
 
 void hip_check(hipError_t e, const char* what) {
     if (e != hipSuccess) fail(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// The address of `scratch` (top of this file) on the current device: resolved
+// once per device, with that device current, and kept.
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+float* static_scratch() {
+    int dev = -1;
+    hip_check(hipGetDevice(&dev), "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) fail("static scratch: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        hip_check(hipGetSymbolAddress(&p, HIP_SYMBOL(::scratch)), "hipGetSymbolAddress(scratch)");
+        if (!p) fail("static scratch: the symbol has no address on this device");
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    return g_scratch_ptr[dev];
 }
 
 PhiloxKey make_key(const Handle& h, uint32_t site, float p) {
@@ -259,6 +291,13 @@ void ensure_ws(Handle& h, size_t floats) {
 // Scratch for one column reduction.  While a backward pass defers the finishing
 // stage, every reduction gets its own region of the (pre-sized) buffer.
 float* take_ws(Handle& h, size_t floats) {
+    if (h.static_ws) {
+        if (floats > kStaticScratchFloats)
+            fail("the column sums of this call need " + std::to_string(floats * sizeof(float)) +
+                 " bytes of scratch, more than the " + std::to_string(kStaticScratchFloats * sizeof(float)) +
+                 " bytes of the static scratch array");
+        return h.static_ws;
+    }
     if (!h.deferring) {
         ensure_ws(h, floats);
         return h.ws;
@@ -1462,6 +1501,30 @@ int sub_op_ebsb(void* handle, const void* in, const char* l_in, const void* scal
     });
 }
 
+namespace {
+void ln_backward_body(Handle& h, int extended, const void* in, const char* l_in, const void* scale,
+                      const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                      const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
+                      const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
+                      const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                      const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias) {
+    const bool ext = extended != 0;
+    if (ext && (!dout2 || !dlinear || !dlinear_bias || !dout_bias))
+        fail("sub_op_ln_backward: the extended form needs dout2, dlinear, dlinear_bias and dout_bias");
+    const Layout li = L(h, l_in), l1 = L(h, l_dout1), lis = L(h, l_istd), ldf = L(h, l_diff), lm = L(h, l_mask),
+                 lg = L(h, l_g), lo1 = L(h, l_d_ln_in), lo2 = L(h, l_d_drop_in);
+    const Layout l2 = ext ? L(h, l_dout2) : l1, ldl = ext ? L(h, l_dlinear) : l1;
+    if (op_lnbwd(h, ext, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, istd, lis, diff, ldf, mask, lm, g, lg,
+                 d_ln_in, lo1, d_drop_in, lo2, dscale, dbias, dlinear_bias, dout_bias))
+        return;
+    // shapes or layouts the one-launch form does not take: the separate operators, same results
+    if (ext) op_ebsb(h, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, g, lg, dscale, dbias, dlinear_bias);
+    else op_bsb(h, in, li, scale, dout1, l1, g, lg, dscale, dbias);
+    op_blnrd(h, g, lg, istd, lis, diff, ldf, mask, lm, d_ln_in, lo1, d_drop_in, lo2);
+    if (ext) op_baob(h, d_drop_in, lo2, dout_bias);
+}
+}  // namespace
+
 int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l_in, const void* scale,
                        const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
                        const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
@@ -1470,20 +1533,32 @@ int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l
                        const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
-        const bool ext = extended != 0;
-        if (ext && (!dout2 || !dlinear || !dlinear_bias || !dout_bias))
-            fail("sub_op_ln_backward: the extended form needs dout2, dlinear, dlinear_bias and dout_bias");
-        const Layout li = L(h, l_in), l1 = L(h, l_dout1), lis = L(h, l_istd), ldf = L(h, l_diff), lm = L(h, l_mask),
-                     lg = L(h, l_g), lo1 = L(h, l_d_ln_in), lo2 = L(h, l_d_drop_in);
-        const Layout l2 = ext ? L(h, l_dout2) : l1, ldl = ext ? L(h, l_dlinear) : l1;
-        if (op_lnbwd(h, ext, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, istd, lis, diff, ldf, mask, lm, g, lg,
-                     d_ln_in, lo1, d_drop_in, lo2, dscale, dbias, dlinear_bias, dout_bias))
-            return;
-        // shapes or layouts the one-launch form does not take: the separate operators, same results
-        if (ext) op_ebsb(h, in, li, scale, dout1, l1, dout2, l2, dlinear, ldl, g, lg, dscale, dbias, dlinear_bias);
-        else op_bsb(h, in, li, scale, dout1, l1, g, lg, dscale, dbias);
-        op_blnrd(h, g, lg, istd, lis, diff, ldf, mask, lm, d_ln_in, lo1, d_drop_in, lo2);
-        if (ext) op_baob(h, d_drop_in, lo2, dout_bias);
+        ln_backward_body(h, extended, in, l_in, scale, dout1, l_dout1, dout2, l_dout2, dlinear, l_dlinear, istd, l_istd,
+                         diff, l_diff, mask, l_mask, g, l_g, d_ln_in, l_d_ln_in, d_drop_in, l_d_drop_in, dscale, dbias,
+                         dlinear_bias, dout_bias);
+    });
+}
+
+int sub_op_ln_backward_static(void* handle, int extended, const void* in, const char* l_in, const void* scale,
+                              const void* dout1, const char* l_dout1, const void* dout2, const char* l_dout2,
+                              const void* dlinear, const char* l_dlinear, const void* istd, const char* l_istd,
+                              const void* diff, const char* l_diff, const void* mask, const char* l_mask, void* g,
+                              const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
+                              const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias,
+                              void* dout_bias) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        // The partial rows go to the static array of the current device.  Each kernel of
+        // this call writes every partial it later reads, so nothing has to start at zero;
+        // the launches that share the array within the call are ordered by the stream.
+        struct Use {
+            Handle& h;
+            Use(Handle& h_, float* p) : h(h_) { h.static_ws = p; }
+            ~Use() { h.static_ws = nullptr; }
+        } use(h, static_scratch());
+        ln_backward_body(h, extended, in, l_in, scale, dout1, l_dout1, dout2, l_dout2, dlinear, l_dlinear, istd, l_istd,
+                         diff, l_diff, mask, l_mask, g, l_g, d_ln_in, l_d_ln_in, d_drop_in, l_d_drop_in, dscale, dbias,
+                         dlinear_bias, dout_bias);
     });
 }
 

@@ -117,11 +117,13 @@ class Ops:
 
     def ln_backward(self, inp, l_in, scale, dout1, l_dout1, istd, l_istd, diff, l_diff, mask, l_mask, g, l_g,
                     d_ln_in, l_d_ln_in, d_drop_in, l_d_drop_in, dscale, dbias, dout2=None, l_dout2=None,
-                    dlinear=None, l_dlinear=None, dlinear_bias=None, dout_bias=None):
+                    dlinear=None, l_dlinear=None, dlinear_bias=None, dout_bias=None, static_scratch=False):
         """bsb + blnrd, or with dout2 / dlinear / dlinear_bias / dout_bias given ebsb + blnrd + baob, in one
-        launch where the sizes and layouts allow."""
+        launch where the sizes and layouts allow.  ``static_scratch``: the entry point that allocates
+        nothing (partial sums in the library's static device array)."""
         ext = dout2 is not None
-        _lib.check(self.lib.sub_op_ln_backward(
+        fn = self.lib.sub_op_ln_backward_static if static_scratch else self.lib.sub_op_ln_backward
+        _lib.check(fn(
             self._pre(), int(ext), _p(inp), _s(l_in), _p(scale), _p(dout1), _s(l_dout1), _p(dout2),
             _s(l_dout2 or l_dout1), _p(dlinear), _s(l_dlinear or l_dout1), _p(istd), _s(l_istd), _p(diff), _s(l_diff),
             _p(mask), _s(l_mask), _p(g), _s(l_g), _p(d_ln_in), _s(l_d_ln_in), _p(d_drop_in), _s(l_d_drop_in),
