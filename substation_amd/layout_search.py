@@ -190,6 +190,7 @@ class LayoutSearch:
                 seen = []
                 for member in group:
                     seen += [n for n in _og.OP_TENSORS[member] if n not in seen]
+                    seen += [n for n in _og.GROUP_ALSO_DEPENDS.get(member, ()) if n not in seen]
                 return tuple(seen)
         return _og.OP_TENSORS[op]
 
@@ -361,6 +362,144 @@ class LayoutSearch:
                   f"Total: {tot['fwd'] + tot['bwd']:g}")
 
 
+# --------------------------------------------------------------------------- #
+# one operator under all its layouts
+# --------------------------------------------------------------------------- #
+
+class OperatorSweep:
+    """One fused operator timed on its own under every layout of its tensors: the
+    counterpart of the per-kernel sweep of pytorch_module/benchmark.py:178-302,
+    1362-1472, whose results the reference ships as perf_softmax.txt, perf_bsb.txt,
+    perf_bdrln.txt, perf_bad.txt.  The reference compiles one kernel per
+    combination; strides are run-time data here, so a combination is one call
+    through the operator entry points of the C ABI.  Tensors are grouped into
+    roles that change layout together (as the reference's files do: softmax
+    ``IN -> OUT``); every role runs through all permutations of its dims."""
+
+    #: operator -> (dims, [(role, [tensor arguments])]): arguments named as in substation_amd.ops.Ops
+    OPERATORS = {
+        'softmax': ('HBJK', [('IN', ['beta', 'drop']), ('OUT', ['alpha', 'mask'])]),
+        'bs': ('HBJK', [('IN', ['alpha', 'mask', 'ddrop']), ('OUT', ['dbeta'])]),
+        'bdrln': ('BJI', [('IN', ['inp', 'resid']), ('OUT', ['lin', 'mask', 'diff', 'normed', 'out'])]),
+        'blnrd': ('BJI', [('IN', ['dout', 'diff', 'mask']), ('OUT', ['d_ln_in', 'd_drop_in'])]),
+        'bad': ('BJU', [('IN', ['inp']), ('OUT', ['lin', 'mask', 'out'])]),
+        'bdrlb': ('BJU', [('IN', ['ddrop', 'mask', 'lin']), ('OUT', ['dlinear'])]),
+        'bsb': ('BJI', [('IN', ['inp', 'dout']), ('DIN', ['din'])]),
+        'ebsb': ('BJI', [('IN', ['inp', 'dout1', 'dout2', 'dlinear']), ('DIN', ['din'])]),
+        'baob': ('BJI', [('IN', ['datt'])]),
+        'bei': ('BJI', [('IN', ['dxatt', 'dresid1']), ('OUT', ['dx'])]),
+    }
+
+    def __init__(self, batch, seq, heads, embed, intermediate=None, iters=5, warmup=2, device='cuda'):
+        import torch
+        from . import ops as _ops
+        self.torch = torch
+        self.o = _ops.Ops(batch, seq, heads, embed, intermediate_size=intermediate, seed=0x5EED)
+        self.iters, self.warmup, self.device = iters, warmup, device
+        self.g = torch.Generator(device=device).manual_seed(7)
+
+    def _tensor(self, layout, kind='normal'):
+        t = self.o.empty(layout, self.device)
+        if kind == 'mask':
+            t.copy_((self.torch.rand(t.shape, device=self.device, generator=self.g) >= 0.1).half())
+        elif kind == 'positive':
+            t.normal_(0.0, 1.0, generator=self.g).abs_().add_(0.5)
+        else:
+            t.normal_(0.0, 1.0, generator=self.g)
+        return t
+
+    def _vector(self, dim):
+        n = self.o.sizes[dim]
+        return self.torch.empty(n, dtype=self.torch.float16, device=self.device).normal_(0.0, 0.1, generator=self.g)
+
+    def _call(self, op, lay):
+        """Allocates the operator's tensors under ``lay`` (argument -> layout) and returns a
+        function that launches it once."""
+        o, T = self.o, self._tensor
+        if op == 'softmax':
+            a = dict(beta=T(lay['beta']), alpha=T(lay['alpha']), mask=T(lay['mask']), drop=T(lay['drop']))
+            return lambda: o.softmax(a['beta'], lay['beta'], a['alpha'], lay['alpha'], a['mask'], lay['mask'],
+                                     a['drop'], lay['drop'], scale=0.125, p=0.1)
+        if op == 'bs':
+            a = dict(alpha=T(lay['alpha']), mask=T(lay['mask'], 'mask'), ddrop=T(lay['ddrop']), dbeta=T(lay['dbeta']))
+            return lambda: o.bs(a['alpha'], lay['alpha'], a['mask'], lay['mask'], a['ddrop'], lay['ddrop'],
+                                a['dbeta'], lay['dbeta'], scale=0.125)
+        if op == 'bdrln':
+            a = {k: T(lay[k]) for k in ('inp', 'resid', 'lin', 'mask', 'diff', 'normed', 'out')}
+            istd, v = T('BJ'), [self._vector('I') for _ in range(3)]
+            return lambda: o.bdrln(a['inp'], lay['inp'], a['resid'], lay['resid'], v[0], v[1], v[2], a['lin'], lay['lin'],
+                                   a['mask'], lay['mask'], a['diff'], lay['diff'], a['normed'], lay['normed'],
+                                   a['out'], lay['out'], istd, 'BJ', p=0.1, site=1)
+        if op == 'blnrd':
+            a = dict(dout=T(lay['dout']), diff=T(lay['diff']), mask=T(lay['mask'], 'mask'), d_ln_in=T(lay['d_ln_in']),
+                     d_drop_in=T(lay['d_drop_in']))
+            istd = T('BJ', 'positive')
+            return lambda: o.blnrd(a['dout'], lay['dout'], istd, 'BJ', a['diff'], lay['diff'], a['mask'], lay['mask'],
+                                   a['d_ln_in'], lay['d_ln_in'], a['d_drop_in'], lay['d_drop_in'])
+        if op == 'bad':
+            a = {k: T(lay[k]) for k in ('inp', 'lin', 'mask', 'out')}
+            b = self._vector('U')
+            return lambda: o.bad(a['inp'], lay['inp'], b, a['lin'], lay['lin'], a['mask'], lay['mask'], a['out'],
+                                 lay['out'], p=0.1, site=2)
+        if op == 'bdrlb':
+            a = dict(ddrop=T(lay['ddrop']), mask=T(lay['mask'], 'mask'), lin=T(lay['lin']), dlinear=T(lay['dlinear']))
+            db = self._vector('U')
+            return lambda: o.bdrlb(a['ddrop'], lay['ddrop'], a['mask'], lay['mask'], a['lin'], lay['lin'],
+                                   a['dlinear'], lay['dlinear'], db)
+        if op == 'bsb':
+            a = {k: T(lay[k]) for k in ('inp', 'dout', 'din')}
+            v = [self._vector('I') for _ in range(3)]
+            return lambda: o.bsb(a['inp'], lay['inp'], v[0], a['dout'], lay['dout'], a['din'], lay['din'], v[1], v[2])
+        if op == 'ebsb':
+            a = {k: T(lay[k]) for k in ('inp', 'dout1', 'dout2', 'dlinear', 'din')}
+            v = [self._vector('I') for _ in range(4)]
+            return lambda: o.ebsb(a['inp'], lay['inp'], v[0], a['dout1'], lay['dout1'], a['dout2'], lay['dout2'],
+                                  a['dlinear'], lay['dlinear'], a['din'], lay['din'], v[1], v[2], v[3])
+        if op == 'baob':
+            a, v = T(lay['datt']), self._vector('I')
+            return lambda: o.baob(a, lay['datt'], v)
+        if op == 'bei':
+            a = {k: T(lay[k]) for k in ('dxatt', 'dresid1', 'dx')}
+            return lambda: o.bei(a['dxatt'], lay['dxatt'], a['dresid1'], lay['dresid1'], a['dx'], lay['dx'])
+        raise KeyError(op)
+
+    def time(self, op, role_layouts):
+        """Seconds per launch with every tensor of a role in that role's layout."""
+        torch = self.torch
+        _, roles = self.OPERATORS[op]
+        lay = {arg: role_layouts[role] for role, args in roles for arg in args}
+        run = self._call(op, lay)
+        for _ in range(self.warmup):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(self.iters):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / self.iters
+
+    def sweep(self, op, out=sys.stdout, budget_s=None):
+        """Every combination of role layouts; one line per combination, `op ROLE layout ... time = X s`
+        (the key = value ... time = X s lines of pytorch_module/benchmark.py:1437-1447).  Returns the
+        list of (role_layouts, seconds), fastest first."""
+        dims, roles = self.OPERATORS[op]
+        perms = [''.join(p) for p in itertools.permutations(dims)]
+        results = []
+        t0 = time.monotonic()
+        for combo in itertools.product(perms, repeat=len(roles)):
+            if budget_s is not None and time.monotonic() - t0 > budget_s:
+                print(f'# time budget used up after {len(results)} combinations', file=out, flush=True)
+                break
+            rl = {role: l for (role, _), l in zip(roles, combo)}
+            sec = self.time(op, rl)
+            results.append((rl, sec))
+            print(f'op = {op} ' + ' '.join(f'{r} = {l}' for r, l in rl.items()) + f' time = {sec:g} s', file=out,
+                  flush=True)
+        results.sort(key=lambda x: x[1])
+        return results
+
+
 def _start_layouts(name):
     if name == 'mi355x':
         return _lay.mi355x_layouts()
@@ -388,7 +527,22 @@ def main(argv=None):
     ap.add_argument('--min-gain', type=float, default=0.002)
     ap.add_argument('--out', default=None, help='layouts pickle to write')
     ap.add_argument('--log', default=None, help="table entries as 'k = v ... time = X s' lines")
+    ap.add_argument('--sweep-op', default=None, choices=sorted(OperatorSweep.OPERATORS),
+                    help='time this one operator on its own under every layout of its tensors instead of '
+                         'searching (lines go to --log or stdout)')
     args = ap.parse_args(argv)
+
+    if args.sweep_op:
+        sweep = OperatorSweep(args.batch, args.seq, args.heads, args.embed, args.intermediate, iters=args.iters)
+        log = open(args.log, 'w') if args.log else sys.stdout
+        try:
+            res = sweep.sweep(args.sweep_op, out=log, budget_s=args.budget_s)
+        finally:
+            if args.log:
+                log.close()
+        show = lambda r: ' '.join(f'{k} {v}' for k, v in r[0].items()) + f' {r[1] * 1e6:.2f} us'
+        print(f'{args.sweep_op}: {len(res)} combinations; best {show(res[0])}; worst {show(res[-1])}', flush=True)
+        return res
 
     start = _start_layouts(args.start)
     timer = LayerTimer(args.batch, args.seq, args.heads, args.embed, args.intermediate,

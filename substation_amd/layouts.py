@@ -61,28 +61,25 @@ def _make(inp, out, params, fwd, bwd, special='', algos=''):
 
 def mi355x_layouts(name=None):
     """Configuration for MI355X (``name``: one of the two workloads the reference
-    ships configurations for, or None for the default).  The layout search
-    (substation_amd.layout_search) run on the device confirms the default for
-    'bert-b8-l512-h16-e1024' and finds one change for 'bert-b96-l128-h16-e1024'
-    (WKQV stored [Q,I,H,P], -1.5 % layer time).
+    ships configurations for, or None for the default), read from the files the
+    layout search (substation_amd.layout_search, the counterpart of
+    config_selection/optimize.py) wrote from timings on the device:
+    ``configs/layouts-mi355x-<name>.pickle``, same schema as the reference's
+    pickles, decoded as plain data.  None is the configuration of
+    'bert-b8-l512-h16-e1024'.
 
-    Default: token-major activations with the
-    feature dimension contiguous (every fused operator then moves 128-bit packs),
+    What the search settles on: token-major activations with the feature
+    dimension contiguous (every fused operator then moves 128-bit packs),
     projections stored [Q,B,J,H,P] and the attention output [B,J,H,P] so that
     QK^T, the output projection and both FFN products contract over a contiguous
-    dimension of both operands.  Weights are stored [out, in]."""
+    dimension of both operands, weights stored [out, in]; for B=96 L=128 the
+    projection weight is stored [Q,I,H,P]."""
     if name not in (None, 'bert-b8-l512-h16-e1024', 'bert-b96-l128-h16-e1024'):
         raise KeyError(name)
-    wkqv = 'QIHP' if name == 'bert-b96-l128-h16-e1024' else 'QHPI'
-    return _make(
-        'BJI', 'BJI',
-        f'WKQV:{wkqv} BKQV:QHP WO:IHP BO:I S1:I B1:I LINB1:U LINW1:UI S2:I B2:I LINB2:I LINW2:IU',
-        'KKQQVV:QBJHP WKKWQQWVV:QBJHP BETA:HBJK ALPHA:HBJK ATTN_DROP_MASK:HBJK ATTN_DROP:HBJK '
-        'GAMMA:BJHP ATT:BJI DROP1MASK:BJI SB1:BJI SB1_LINW1:BJU DROP2:BJU LIN1:BJU DROP2_LINW2:BJI '
-        'LIN2:BJI LN2:BJI LN2STD:BJ LN2DIFF:BJI DROP2MASK:BJU DROP3MASK:BJI LN1:BJI LN1STD:BJ '
-        'LN1DIFF:BJI',
-        'DLN2:BJI DRESID2:BJI DLIN2:BJI DDROP2:BJU DLIN1:BJU DLIN1_LINW1:BJI DLN1:BJI DRESID1:BJI '
-        'DATT:BJI DXATT:BJI DGAMMA:BJHP DATTN_DROP:HBJK DBETA:HBJK DKKQQVV:QBJHP')
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'configs',
+                        f'layouts-mi355x-{name or "bert-b8-l512-h16-e1024"}.pickle')
+    return load_layouts(path)
 
 
 def reference_layouts(name):

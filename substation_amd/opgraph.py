@@ -87,6 +87,18 @@ ALTERNATIVES = [
     ('ebsb+blnrd2+baob', 'ebsb', 'blnrd2', 'baob'),
 ]
 
+#: Tensors beyond its members' own that decide which members of a group run: the
+#: attention kernels with the scores in registers need feature-contiguous
+#: projections, outputs and gradients in both passes (one decision for both), and
+#: whether dWout and the column-sum finish ride in the last launch of the backward
+#: pass depends on that decision too.
+_ATTENTION_DECIDERS = ('KKQQVV', 'GAMMA', 'DGAMMA', 'DKKQQVV')
+GROUP_ALSO_DEPENDS = {
+    'attention': _ATTENTION_DECIDERS,
+    'attention-bwd-dQ': _ATTENTION_DECIDERS,
+    'dXQKV-fused+dWQKV-fused+dWout': _ATTENTION_DECIDERS + ('BKQV',),
+}
+
 #: the 18 contractions (pytorch_module/encoder.cu:90-276; canonical list
 #: tc_profiling/einsum_perms.py:367-394): name -> (A, B, C) operand names, where
 #: KK/QQ/VV and DKK/DQQ/DVV are the Q-slices of the stacked tensors
