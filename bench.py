@@ -411,8 +411,52 @@ def bench_fused_ops(args):
                          unit='GB/s', frac=round(nbytes / t / HBM_PEAK, 4), bytes=nbytes, buffer_sets=nsets))
         del sets, graph
         torch.cuda.empty_cache()
+    # What the same box gives vendor streaming kernels of the same shapes (torch elementwise kernels, timed the
+    # same way): a ceiling for 1 read + 1 write (copy), 2 reads + 1 write (add) and 1 write (fill) at the two
+    # sizes the operators above have, 8 MiB and 64 MiB per tensor.
+    stream = []
+    for mib in (8, 64):
+        n = mib << 19                                         # fp16 elements
+        for kind, ntens in (('copy', 2), ('add', 3), ('fill', 1)):
+            nbytes = ntens * n * 2
+            nsets = max(2, -(-(640 << 20) // nbytes))
+            sets = [[torch.empty(n, dtype=torch.float16, device='cuda').normal_() for _ in range(ntens)]
+                    for _ in range(nsets)]
+
+            def run(t, kind=kind):
+                if kind == 'copy':
+                    t[1].copy_(t[0])
+                elif kind == 'add':
+                    torch.add(t[0], t[1], out=t[2])
+                else:
+                    t[0].fill_(1.0)
+
+            for t in sets:
+                run(t)
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    for t in sets:
+                        run(t)
+            torch.cuda.synchronize()
+            graph.replay()
+            reps = max(3, args.steps // 10)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            t_one = e0.elapsed_time(e1) * 1e-3 / (reps * nsets)
+            stream.append(dict(kernel=f'torch {kind}, {mib} MiB per tensor', us=round(t_one * 1e6, 2),
+                               gbps=round(nbytes / t_one / 1e9, 1), frac=round(nbytes / t_one / HBM_PEAK, 4)))
+            del sets, graph
+            torch.cuda.empty_cache()
     if args.per_op:
-        for r in rows:
+        for r in rows + stream:
             print(json.dumps(r), file=sys.stderr)
     sm = [r for r in rows if r['op'] in ('softmax', 'bs')]
     t_sm = sum(r['us'] for r in sm) * 1e-6
@@ -432,6 +476,7 @@ def bench_fused_ops(args):
                                    'source': 'pytorch_module/perf_softmax.txt, perf_bad.txt, perf_bsb.txt, '
                                              'perf_bdrln.txt (GPU not stated)'},
         'ops': [{k: r[k] for k in ('op', 'us', 'achieved', 'unit', 'frac', 'bytes', 'buffer_sets')} for r in rows],
+        'stream_reference': stream,
     }
     print(json.dumps(out))
 
