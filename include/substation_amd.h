@@ -232,7 +232,8 @@ int sub_encoder_backward(void* handle, void* const* ptrs, int n);
  * of launches of the last encoder_forward call followed, if one has been issued
  * since, by those of the encoder_backward call after it (at most cap are
  * written); reading only after the backward call leaves no host wait between
- * the two passes. */
+ * the two passes.  One event is recorded in front of every launch and one at the
+ * end of each pass; a launch is timed from its event to the next one. */
 int sub_profile_enable(void* handle, int on);
 int sub_profile_read(void* handle, int cap, const char** names, float* ms);
 

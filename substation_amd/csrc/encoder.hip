@@ -164,7 +164,9 @@ struct GemmPlan {
 enum G { G_QKV_BIAS, G_DXQKV_RESID, G_LIN1_BAD, G_DXLIN2_BDRLB, G_QKV, G_QKT, G_GAMMA, G_OUT, G_LIN1, G_LIN2, G_DXLIN2, G_DWLIN2, G_DXLIN1, G_DWLIN1,
          G_DWOUT, G_DXOUT, G_DX1GAMMA, G_DX2GAMMA, G_DX1QKT, G_DX2QKT, G_DXQKV, G_DWQKV, G_COUNT };
 
-struct ProfEntry { const char* name; hipEvent_t a, b; };
+// One event in front of every launch: a launch lasts from its event to the next
+// one (the next launch's, or the marker that closes a pass: name == nullptr).
+struct ProfEntry { const char* name; hipEvent_t a; };
 
 struct Handle {
     bool configured = false;
@@ -215,7 +217,7 @@ struct Handle {
         if (ws) (void)hipFree(ws);
         if (gws) (void)hipFree(gws);
         if (mask_plan) (void)hipFree(mask_plan);
-        for (auto& e : prof) { (void)hipEventDestroy(e.a); (void)hipEventDestroy(e.b); }
+        for (auto& e : prof) (void)hipEventDestroy(e.a);
         if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
     }
 };
@@ -253,22 +255,24 @@ PhiloxKey make_key(const Handle& h, uint32_t site, float p) {
 }
 
 struct ProfScope {
-    Handle& h; ProfEntry* e = nullptr;
+    Handle& h; bool used = false;
     ProfScope(Handle& h_, const char* name) : h(h_) {
         if (!h.profiling) return;
         if (h.prof_used == h.prof.size()) {
-            ProfEntry n{name, nullptr, nullptr};
+            ProfEntry n{name, nullptr};
             hip_check(hipEventCreate(&n.a), "hipEventCreate");
-            hip_check(hipEventCreate(&n.b), "hipEventCreate");
             h.prof.push_back(n);
         }
-        e = &h.prof[h.prof_used++];
-        e->name = name;
-        hip_check(hipEventRecord(e->a, h.stream), "hipEventRecord");
+        ProfEntry& e = h.prof[h.prof_used++];
+        e.name = name;
+        hip_check(hipEventRecord(e.a, h.stream), "hipEventRecord");
+        used = true;
     }
-    ~ProfScope() { if (e) (void)hipEventRecord(e->b, h.stream); }
-    void cancel() { if (e) { --h.prof_used; e = nullptr; } }     // nothing was launched
+    // nothing was launched: the entry goes (its event stays in the stream, harmless)
+    void cancel() { if (used) { --h.prof_used; used = false; } }
 };
+// Closes the last launch of a pass.
+void prof_mark_end(Handle& h) { ProfScope end(h, nullptr); }
 
 // Allocations happen on the first call of a handle; that call cannot be part
 // of a graph capture.
@@ -919,6 +923,7 @@ void forward(Handle& h, const FwdPtrs& t) {
                  F[LIN2], h.lf[LIN2], F[DROP3MASK], h.lf[DROP3MASK], F[LN2DIFF], h.lf[LN2DIFF],
                  F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2);
     }
+    prof_mark_end(h);
     if (h.step_dev) {
         hipLaunchKernelGGL(k_step_increment, dim3(1), dim3(64), 0, h.stream, h.step_dev);
         check_launch("dropout step increment");
@@ -1127,6 +1132,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         ProfScope ps(h, "colfinish");
         launch_colfinish(h.deferred, h.stream);
     }
+    prof_mark_end(h);
 }
 
 void unpack_forward(const Handle& h, void* const* p, FwdPtrs& t) {
@@ -1327,12 +1333,15 @@ int sub_profile_read(void* handle, int cap, const char** names, float* ms) {
     int rc = guarded([&] {
         Handle& h = as_handle(handle);
         hip_check(hipStreamSynchronize(h.stream), "hipStreamSynchronize");
-        count = (int)h.prof_used;
-        for (int i = 0; i < count && i < cap; ++i) {
-            float t = 0.f;
-            hip_check(hipEventElapsedTime(&t, h.prof[i].a, h.prof[i].b), "hipEventElapsedTime");
-            if (names) names[i] = h.prof[i].name;
-            if (ms) ms[i] = t;
+        for (size_t i = 0; i + 1 < h.prof_used; ++i) {
+            if (!h.prof[i].name) continue;             // the marker between the two passes
+            if (count < cap) {
+                float t = 0.f;
+                hip_check(hipEventElapsedTime(&t, h.prof[i].a, h.prof[i + 1].a), "hipEventElapsedTime");
+                if (names) names[count] = h.prof[i].name;
+                if (ms) ms[count] = t;
+            }
+            ++count;
         }
     });
     return rc == 0 ? count : rc;

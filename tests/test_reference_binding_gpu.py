@@ -1,7 +1,7 @@
 """The reference's own way of calling the library, executed on the GPU: the ctypes
-binding that INTEGRATION.md (Option B) gives a maintainer of
-pytorch_module/encoder.py to put in place of `_compile_module` is taken from that
-file verbatim, and the four exports of pytorch_module/encoder.cu:304-318 are then
+binding that the integration notes at the repository root give a maintainer of
+pytorch_module/encoder.py to put in place of `_compile_module` is taken from
+there verbatim, and the four exports of pytorch_module/encoder.cu:304-318 are then
 driven as pytorch_module/encoder.py:71-139 drives them: `init()`, positional
 `encoder_forward` (1 + 37 pointers) and `encoder_backward` (1 + 64 pointers) in
 the order of the lists of the layouts dict, `destroy()`.  Results against the
