@@ -11,7 +11,6 @@
 // are always 8 consecutive k per lane.  The output is produced transposed in the
 // accumulators (4 consecutive n per lane), staged through LDS and written as
 // full 128-bit rows.
-#include <cstdlib>
 #include <cstring>
 
 #include "sub_ops.hpp"
@@ -831,7 +830,7 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
     return ok ? 1 : 0;
 }
 
-// Block tile for a problem: 22 = 128x128, 42 = 256x128, 44 = 256x256, 21 = 128x64.
+// Block tile for a problem: 22 = 128x128, 44 = 256x256, 21 = 128x64.
 int pick_tile(const GemmArgs& a, long batch, bool akc, bool bkc) {
     if (a.N <= 64) return 21;      // head-size wide outputs of the attention products
     // 256x256 tiles halve the L2->LDS traffic per flop; they pay once the output
@@ -839,13 +838,11 @@ int pick_tile(const GemmArgs& a, long batch, bool akc, bool bkc) {
     // tiles (asynchronous kernel only: whole tiles, no split contraction).  With
     // an operand that is read through the slower LDS transpose path the bar is
     // higher: three quarters of a round is not enough then (measured).
-    static const int min44 = [] { const char* e = getenv("SUB_GEMM_MIN44"); return e ? atoi(e) : 0; }();
     if (a.M % 256 == 0 && a.N % 256 == 0 && a.K1 % BK == 0 && a.splits == 1) {
         const long tiles = (long)(a.M / 256) * (a.N / 256) * batch;
         const long rounds = (tiles + 255) / 256;
         const double fill = (double)tiles / (double)(rounds * 256);
-        const bool ok = min44 > 0 ? tiles >= min44 : fill >= ((akc && bkc) ? 0.7 : 0.9);
-        if (ok) return 44;
+        if (fill >= ((akc && bkc) ? 0.7 : 0.9)) return 44;
     }
     return 22;
 }
@@ -883,10 +880,8 @@ void launch_dma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t s
 
 template <int TM, int TN>
 void launch_dma(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t st) {
-    static const bool eight = [] { const char* e = getenv("SUB_GEMM_W8"); return !e || atoi(e) != 0; }();
-    if constexpr (TM * TN >= 16) {                    // 256x256 tiles: two 64 KiB stages
-        if (eight) launch_dma2<TM, TN / 2, 2, 8>(a, akc, bkc, grid, st);
-        else launch_dma2<TM, TN, 2, 4>(a, akc, bkc, grid, st);
+    if constexpr (TM * TN >= 16) {                    // 256x256 tiles: two 64 KiB stages, eight waves
+        launch_dma2<TM, TN / 2, 2, 8>(a, akc, bkc, grid, st);
     } else {
         launch_dma2<TM, TN, 3, 4>(a, akc, bkc, grid, st);
     }
@@ -914,12 +909,10 @@ constexpr long kSplitTarget = 256;            // workgroups a split product aims
 // How many ways to split k so that a small output still fills the chip: the
 // weight-gradient products have few output tiles and a long contraction.
 int pick_splits(const GemmArgs& a, long batch, size_t ws_floats) {
-    static const int force = [] { const char* e = getenv("SUB_GEMM_SPLITK"); return e ? atoi(e) : 0; }();
     const long tiles = (long)((a.M + 127) / 128) * ((a.N + 127) / 128) * batch;
     const int nkt = a.K0 * ((a.K1 + BK - 1) / BK);
     // one workgroup per CU: a second, partly filled round costs more than it gains
-    int splits = force > 0 ? force : (int)(kSplitTarget / tiles);
-    if (force < 0) splits = 1;
+    int splits = (int)(kSplitTarget / tiles);
     if (splits > 8) splits = 8;
     while (splits > 1 && nkt / splits < 8) --splits;
     const size_t need = (size_t)batch * a.M * a.N;          // floats per split
@@ -1031,8 +1024,6 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
                       const GemmEpilogue& ep1, const GemmShape& s2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws,
                       size_t ws_floats, FinishJobs* tail, PairThird* third) {
-    static const int off = [] { const char* e = getenv("SUB_GEMM_PAIR"); return e ? atoi(e) == 0 : 0; }();
-    if (off) return false;
     const GemmShape* sh[2] = {&s1, &s2};
     const Canon cin[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
     PairSel sel;
@@ -1076,22 +1067,19 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
     bool akc = false, bkc = false;
     int kind = pick_kind(c, akc, bkc);
     if (kind == 1) {
-        static const int force = [] { const char* e = getenv("SUB_GEMM_TILE"); return e ? atoi(e) : 0; }();
-        // SUB_GEMM_DMA: -1 never / 1 always use the asynchronous kernel; default: when both
-        // operands are k-contiguous and there is at most about one tile per CU, where
-        // the register-staged kernel has no second workgroup to hide its waits behind.
-        static const int dma_env = [] { const char* e = getenv("SUB_GEMM_DMA"); return e ? atoi(e) : 0; }();
+        // The asynchronous 128x128 kernel is taken when both operands are k-contiguous and there
+        // is at most about one tile per CU, where the register-staged kernel has no second
+        // workgroup to hide its waits behind.
         const long tiles128 = (long)((c.a.M + 127) / 128) * ((c.a.N + 127) / 128) * batch;
         if (ws && (size_t)batch * c.a.M * c.a.N <= kSplitMaxOut) {
             c.a.splits = pick_splits(c.a, batch, ws_floats);
             c.a.partial = ws;
         }
-        const int tile = force ? force : pick_tile(c.a, batch, akc, bkc);
+        const int tile = pick_tile(c.a, batch, akc, bkc);
         if ((ep.relu_dropout || ep.gate) && (tile != 44 || batch != 1 || s.sCN != 1 || s.sCM != s.N))
             fail("gemm: the ReLU-dropout epilogue needs the 256x256 asynchronous kernel (see gemm_relu_dropout_ok)");
-        const bool dma = dma_env > 0 || (dma_env == 0 && akc && bkc && tiles128 <= 384);
+        const bool dma = akc && bkc && tiles128 <= 384;
         if (tile == 44) launch_mfma<4, 4, true>(c.a, akc, bkc, batch, true, st);
-        else if (tile == 42) launch_mfma<4, 2, true>(c.a, akc, bkc, batch, dma, st);
         else if (tile == 21) launch_mfma<2, 1, false>(c.a, akc, bkc, batch, false, st);
         else launch_mfma<2, 2, true>(c.a, akc, bkc, batch, dma, st);
     } else {
