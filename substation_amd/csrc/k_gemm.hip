@@ -532,6 +532,32 @@ struct DTile {
     }
 };
 
+// Issue order of half a step of the eight-wave kernel: NM matrix instructions with NR
+// fragment reads dealt out evenly between them (after FIRST reads in front).
+template <int m, int NM, int NR>
+__device__ __forceinline__ void sched_mfma_reads_from() {
+    if constexpr (m < NM) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        constexpr int r = (NR * (m + 1)) / NM - (NR * m) / NM;
+        if constexpr (r > 0) __builtin_amdgcn_sched_group_barrier(0x100, r, 0);
+        sched_mfma_reads_from<m + 1, NM, NR>();
+    }
+}
+// NM matrix instructions, each followed by NV vector instructions.
+template <int NM, int NV, int m = 0>
+__device__ __forceinline__ void sched_mfma_valu() {
+    if constexpr (m < NM) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
+        sched_mfma_valu<NM, NV, m + 1>();
+    }
+}
+template <int FIRST, int NM, int NR>
+__device__ __forceinline__ void sched_half_step() {
+    if constexpr (FIRST > 0) __builtin_amdgcn_sched_group_barrier(0x100, FIRST, 0);
+    sched_mfma_reads_from<0, NM, NR>();
+}
+
 // NW waves as 2 x (NW / 2); each wave owns TM x TN accumulator tiles of 32 x 32.
 // Eight waves (two per SIMD) on a 256 x 256 tile: a wave cannot issue past an
 // asynchronous load that the memory path has not accepted yet, and with all 256 CUs
@@ -619,6 +645,38 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         fetched += more_ ? 1 : 0;                                                                 \
     } while (0)
 
+    // ReLU-dropout epilogue: the keep bits of the 16 packs of 8 outputs this lane stores are
+    // drawn during the multiplication, one Philox call per step, where the vector unit is
+    // otherwise idle; the epilogue only picks its byte.  Pack c (0..15) covers output row
+    // (first row of the wave) + 8 c + lane / 8, so its group of 8 canonical elements is
+    // kb_group0 + c * sCM.  Every step shifts the 128 bits up by a byte and draws pack
+    // (kb_next & 15); the start is chosen so that the last 16 steps draw packs 0..15 in order.
+    constexpr int LPR = 4 * TN;                      // lanes per output row of the wave's slab
+    constexpr int RPI = 64 / LPR;                    // rows per store instruction
+    static_assert(EPI != EPI_RELU_DROPOUT || TM * (32 / RPI) == 16, "16 packs of keep bits per lane");
+    PhiloxKey rd_key = g.key;
+    uint32_t kb[4] = {0u, 0u, 0u, 0u};
+    uint64_t kb_group0 = 0;
+    int kb_next = 0;
+    if (EPI == EPI_RELU_DROPOUT) {
+        rd_key = resolved(g.key);
+        const uint64_t row = (uint64_t)(m0 + wm * 32 * TM + lane / LPR);
+        kb_group0 = (row * (uint64_t)g.sCM + (uint64_t)(n0 + wn * 32 * TN + (lane % LPR) * 8)) >> 3;
+        kb_next = nkt >= 16 ? (16 - (nkt & 15)) & 15 : 0;
+    }
+#define SUB_DMA_KEEP()                                                                            \
+    do {                                                                                          \
+        const U4 r_ = philox_group(rd_key, kb_group0 + (uint64_t)(kb_next & 15) * (uint64_t)g.sCM); \
+        uint32_t b_ = 0;                                                                          \
+        _Pragma("unroll") for (int e = 0; e < 8; ++e) b_ |= (field16(r_, e) >= rd_key.thr ? 1u : 0u) << e; \
+        kb[3] = (kb[3] << 8) | (kb[2] >> 24);                                                     \
+        kb[2] = (kb[2] << 8) | (kb[1] >> 24);                                                     \
+        kb[1] = (kb[1] << 8) | (kb[0] >> 24);                                                     \
+        kb[0] = (kb[0] << 8) | b_;                                                                \
+        ++kb_next;                                                                                \
+    } while (0)
+
+    constexpr int RA_ = AKC ? 1 : 2, RB_ = BKC ? 1 : 2;      // LDS reads per fragment
 #define SUB_DMA_COMPUTE(stage_, nx_)                                                              \
     do {                                                                                          \
         const half_t* sA = stage_;                                                                \
@@ -630,8 +688,17 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
             if (NW == 8 && ks == BK / 32) {                                                       \
+                /* first half: the reads of k-slices 1 and 2 between the products of 0 and 1 */   \
+                sched_half_step<TM * RA_ + TN * RB_, 2 * TM * TN, 2 * (TM * RA_ + TN * RB_)>();   \
                 if (late) SUB_DMA_ISSUE(nx_);                                                     \
                 __builtin_amdgcn_sched_barrier(0);                                                \
+            }                                                                                     \
+            if (NW == 8 && EPI == EPI_RELU_DROPOUT && ks == BK / 16 - 1) {                        \
+                /* the last k-slice shares its issue slots with the keep bits: the fragments of  \
+                   the slice before are dead by now, so the draw costs no registers */           \
+                sched_half_step<0, TM * TN, TM * RA_ + TN * RB_>();                               \
+                __builtin_amdgcn_sched_barrier(0);                                                \
+                SUB_DMA_KEEP();                                                                   \
             }                                                                                     \
             if (ks + 1 < BK / 16) {                                                               \
                 _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
@@ -644,6 +711,10 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][j], fa[ks & 1][i], \
                                                                        acc[i][j], 0, 0, 0);       \
         }                                                                                         \
+        /* second half: the reads of k-slice 3 between the products of k-slice 2 */               \
+        if constexpr (NW == 8 && EPI != EPI_RELU_DROPOUT)                                         \
+            sched_half_step<0, 2 * TM * TN, TM * RA_ + TN * RB_>();                               \
+        if constexpr (NW == 8 && EPI == EPI_RELU_DROPOUT) sched_mfma_valu<TM * TN, 12>();         \
     } while (0)
 
     // One step: tile kt is complete once at most the L loads of tile kt+1 are
@@ -688,23 +759,22 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         if (rem >= 1) SUB_DMA_STEP(st0, st2);
         if (rem >= 2) SUB_DMA_STEP(st1, st0);
     }
+    if (EPI == EPI_RELU_DROPOUT)
+        for (int c = nkt; c < 16; ++c) SUB_DMA_KEEP();        // a contraction shorter than 16 steps
 #undef SUB_DMA_STEP
 #undef SUB_DMA_COMPUTE
+#undef SUB_DMA_KEEP
 #undef SUB_DMA_ISSUE
     // surplus fetches may still be landing: drain them before LDS is reused
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
 
     half_t* stage = st0 + wave * STAGE_WAVE;
-    PhiloxKey rd_key = g.key;
-    if (EPI == EPI_RELU_DROPOUT) rd_key = resolved(g.key);
     float colsum[8];              // gate mode: this lane's 8 columns summed over its rows of the wave's slab
 #pragma unroll
     for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
     half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
     const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
-    constexpr int LPR = 4 * TN;
-    constexpr int RPI = 64 / LPR;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = m0 + wm * 32 * TM + i * 32;
@@ -739,8 +809,10 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             }
             if (EPI == EPI_RELU_DROPOUT) {
                 // what the bias-activation-dropout operator does to the rounded sum, with the
-                // same keep bits (the element index is the offset into the dense output)
-                const uint32_t bits = keep_bits8(rd_key, (uint64_t)mm * (uint64_t)g.sCM + (uint64_t)nn);
+                // same keep bits (the element index is the offset into the dense output):
+                // pack c sits in byte 15 - c of the bits drawn in the main loop
+                const int c = i * (32 / RPI) + it, byte = 15 - c;
+                const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     val[e] = ((bits >> e) & 1u) ? (half_t)fmaxf((float)val[e], 0.f) : (half_t)0.0f;

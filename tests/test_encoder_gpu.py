@@ -100,7 +100,7 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
 
 
 def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=None, compact=False,
-                      act='gelu', which='mi355x', inputs=None):
+                      act='gelu', which='mi355x', inputs=None, launches=None):
     """The module as a user gets it (no debug capture: every fusion on, attention
     with the scores in registers where the sizes allow) against the oracle, which
     draws the four dropout masks itself from the same seeded Philox streams.
@@ -110,13 +110,15 @@ def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=
     flips whole gradient elements (run_layer feeds LIN1 > 0 for the same reason).
     ``inputs`` = (params, X, DY) in canonical order replaces the drawn ones; the
     oracle is then not run (the caller has its results for these inputs) and None
-    is returned in its place.
+    is returned in its place.  ``launches``: a list that receives the names of the
+    launches of the step.
     Returns (oracle dict, device dict) with the output, DX and the 12 gradients."""
     from substation_amd import Encoder
     lay = _layouts(which)
     t = _all_layouts(lay)
     enc = Encoder('unused', B, L, H, E, lay, torch.float16, p, p, p, p, activation=act, seed=SEED,
-                  compact_attention=compact, persistent_workspace=(act == 'relu')).cuda()
+                  compact_attention=compact, persistent_workspace=(act == 'relu'),
+                  profiling=launches is not None).cuda()
     enc.set_rng(SEED, step)
     if attn_mask is not None:
         enc.set_attention_mask(torch.from_numpy(attn_mask).half().cuda())
@@ -148,6 +150,8 @@ def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=
     Y = enc(X)
     Y.backward(to_dev(DY_np, t['SB2']))
     torch.cuda.synchronize()
+    if launches is not None:
+        launches.extend(name for name, _ in enc.profile())
     got = {'SB2': from_layout(Y, 'BJI', t['SB2']), 'DX': from_layout(X.grad, 'BJI', t['X'])}
     for name, layout in lay['params']:
         canon = ref.CANONICAL[name]
@@ -203,6 +207,20 @@ def test_bench_path_matches_the_oracle(dims, which):
     BASELINE configs[2] (B=8 L=512) and configs[3] (B=96 L=128) with the layouts the
     benchmark uses.  Output, DX and the 12 gradients to 1e-2."""
     want, got = run_layer_default(*dims, 0.1, seed_data=17, w_std=0.02, act='relu', which=which)
+    _compare(want, got, names=OUTPUTS)
+
+
+@pytest.mark.parametrize('dims', [(96, 128, 4, 256),      # contraction of lin1: 4 steps of 64
+                                  (5, 512, 20, 1280),     # 20 steps
+                                  (3, 512, 36, 2304)])    # 36 steps
+def test_relu_dropout_epilogue_over_short_and_long_contractions(dims):
+    """lin1 with bias, ReLU and dropout in its epilogue draws the keep bits during the
+    contraction, one pack per step of 64 and 16 packs per lane: contractions of fewer
+    than 16 steps, of 16 (the benchmark's) and of more, not a multiple of 16.  The
+    helper also checks that DROP2 is zero exactly where the seeded mask drops."""
+    launches = []
+    want, got = run_layer_default(*dims, 0.1, seed_data=23, w_std=0.02, act='relu', launches=launches)
+    assert 'lin1+bad' in launches, launches
     _compare(want, got, names=OUTPUTS)
 
 

@@ -41,7 +41,8 @@ SIZES = [(2, 16, 2, 32), (3, 24, 2, 48), (2, 128, 4, 512)]
 
 # the last four: short rows, several side by side in a wave (needs >= 16384 rows)
 @pytest.mark.parametrize('B,L,H,E', SIZES + [(1, 520, 1, 8), (8, 128, 16, 64), (4, 256, 16, 64),
-                                            (9, 120, 16, 32), (6, 200, 16, 32)])
+                                            (9, 120, 16, 32), (6, 200, 16, 32),
+                                            (1, 2048, 2, 16)])     # rows of 2048 keys: four packs per lane
 @pytest.mark.parametrize('p', [0.0, 0.5])
 def test_softmax_and_backward(B, L, H, E, p):
     o = _ops(B, L, H, E)
@@ -97,7 +98,8 @@ def test_softmax_baseline_config_full_size():
     assert np.abs(alpha16.sum(axis=-1) - 1).max() < 4e-3
 
 
-@pytest.mark.parametrize('B,L,H,E', [(2, 16, 2, 32), (2, 128, 4, 512), (8, 128, 16, 64), (3, 40, 2, 16)])
+@pytest.mark.parametrize('B,L,H,E', [(2, 16, 2, 32), (2, 128, 4, 512), (8, 128, 16, 64), (3, 40, 2, 16),
+                                     (1, 2048, 2, 16)])
 def test_softmax_with_attention_mask(B, L, H, E):
     """alpha = softmax(scale * beta + mask_scale * attn_mask) with a causal mask
     plus finite entries, in both mask layouts; the backward operator needs no mask."""
@@ -187,7 +189,7 @@ def test_bad_and_bdrlb(B, L, H, E, act):
         assert_close(dbias.float().cpu().numpy(), w_dbias, name='DLINB1', tol=2e-2)
 
 
-@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 3, 1, 20), (4, 64, 1, 1024)])
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 3, 1, 20), (4, 64, 1, 1024), (2, 8, 1, 4096)])
 def test_bsb_ebsb_baob_bei(B, L, H, E):
     o = _ops(B, L, H, E)
     rng = np.random.default_rng(4)
