@@ -204,6 +204,10 @@ struct Handle {
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
     bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
+    // where the last forward call's lin1 epilogue left one bit per element of DROP2 (set = positive), or
+    // null: the unused SB1_LINW1 buffer of that call.  The backward call reads its gate from there when it
+    // is handed the same buffer, and from DROP2 itself otherwise.
+    const void* gate_bits_at = nullptr;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
     size_t prof_forward = 0;          // entries of the last forward call, kept by the backward call after it
@@ -907,8 +911,11 @@ void forward(Handle& h, const FwdPtrs& t) {
         GemmEpilogue ep;
         ep.bias = (const half_t*)W[LINB1]; ep.sbM = p.sM; ep.sbN = p.sN;
         ep.relu_dropout = true; ep.key = make_key(h, SUB_SITE_ACT, h.p_act);
+        if (F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0) ep.gate_bits_out = (uint32_t*)F[SB1_LINW1];
+        h.gate_bits_at = ep.gate_bits_out;
         launch_gemm(p.shape, (const half_t*)F[SB1], (const half_t*)W[LINW1], (half_t*)F[DROP2], p.alpha, ep, h.stream);
     } else {
+    h.gate_bits_at = nullptr;
     run_gemm(h, G_LIN1, F[SB1], W[LINW1], F[SB1_LINW1], "lin1");
     {
         ProfScope ps(h, "bad");
@@ -979,6 +986,9 @@ void backward(Handle& h, const BwdPtrs& t) {
         float* ws = take_ws(h, (size_t)ntc * U);
         GemmEpilogue ep;
         ep.gate = (const half_t*)F[DROP2]; ep.sbM = p.sM; ep.sbN = p.sN; ep.colsum = ws;
+        if (h.gate_bits_at && h.gate_bits_at == F[SB1_LINW1] && h.gemm[G_LIN1_BAD].shape.M == p.shape.M &&
+            h.gemm[G_LIN1_BAD].shape.N == p.shape.N)
+            ep.gate_bits = (const uint32_t*)F[SB1_LINW1];
         launch_gemm(p.shape, (const half_t*)D[DLIN2], (const half_t*)W[LINW2], (half_t*)D[DLIN1], p.alpha, ep, h.stream);
         FinishJob job{ws, FinishArgs{{(half_t*)DW[LINB1], nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};
         if (h.deferring) {

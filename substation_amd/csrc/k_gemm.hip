@@ -7,8 +7,11 @@
 //
 // Operands may be contiguous along the contraction (K) or along their free
 // dimension (M resp. N); an operand that is contiguous along its free dimension
-// is transposed in registers on the way into LDS, so the matrix-core fragments
-// are always 8 consecutive k per lane.  The output is produced transposed in the
+// lies in LDS as in memory and is gathered with the transposing LDS read, so the
+// matrix-core fragments are always 8 consecutive k per lane.  (Turning such tiles
+// around in registers on the way into LDS instead, to read them at the full rate of
+// ds_read_b128, was measured: 1 to 3 us slower per product of 34 GFLOP.)
+// The output is produced transposed in the
 // accumulators (4 consecutive n per lane), staged through LDS and written as
 // full 128-bit rows.
 #include <cstring>
@@ -38,6 +41,8 @@ struct GemmArgs {
     PhiloxKey key;
     const half_t* gate = nullptr; // or: zero where gate <= 0 (strides of `bias`), column sums per 128-row slab
     float* colsum = nullptr;
+    uint32_t* gate_bits_out = nullptr;     // relu_dropout: one bit per output, set where it is positive
+    const uint32_t* gate_bits = nullptr;   // gate: those bits instead of the values of `gate`
 };
 
 // ---------------------------------------------------------------------------
@@ -512,6 +517,21 @@ struct DTile {
                                              (lds_void_ptr)(stage + (wave * NV + i) * 512), 16, 0, 0);
     }
 
+    // KC fragments from one address register per wave and operand: with
+    // base = kc_off(row0 + lane % 32, lane / 32) (row0 a multiple of 32), the fragment of the
+    // idx-th 32-row block below row0 at k-step ks lies at
+    //   (base ^ ((2 ks ^ 4 (idx & 1)) * 8)) + idx * 32 * BK
+    // (32 rows further the swizzle flips bit 2 of the slot, a k-step further the slot moves
+    // by 2, and neither carries).  The eight-wave kernel computes that inside its loop from a
+    // value the compiler cannot see through: left to itself it keeps all 24 addresses of a
+    // wave in registers across the loop and spills other things.
+    static __device__ __forceinline__ int frag_base(int row0, int lane) {
+        return kc_off(row0 + (lane & 31), lane >> 5);
+    }
+    static __device__ __forceinline__ h8 frag_at(const half_t* lds, int base, int idx, int ks) {
+        return *reinterpret_cast<const h8*>(lds + ((base ^ (((2 * ks) ^ (4 * (idx & 1))) * 8)) + idx * 32 * BK));
+    }
+
     static __device__ __forceinline__ h8 frag(const half_t* lds, int row0, int ks, int lane) {
         if (KC) {
             return *reinterpret_cast<const h8*>(lds + kc_off(row0 + (lane & 31), ks * 2 + (lane >> 5)));
@@ -677,15 +697,20 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     } while (0)
 
     constexpr int RA_ = AKC ? 1 : 2, RB_ = BKC ? 1 : 2;      // LDS reads per fragment
+    const int fbase_a = TA::frag_base(wm * TM * 32, lane), fbase_b = TB::frag_base(wn * TN * 32, lane);
+#define SUB_DMA_FRAG_A(i_, ks_) (AKC ? TA::frag_at(sA, ba_, i_, ks_) : TA::frag(sA, (wm * TM + (i_)) * 32, ks_, lane))
+#define SUB_DMA_FRAG_B(j_, ks_) (BKC ? TB::frag_at(sB, bb_, j_, ks_) : TB::frag(sB, (wn * TN + (j_)) * 32, ks_, lane))
 #define SUB_DMA_COMPUTE(stage_, nx_)                                                              \
     do {                                                                                          \
         const half_t* sA = stage_;                                                                \
         const half_t* sB = stage_ + TA::HALVES;                                                   \
         h8 fa[2][TM], fb[2][TN];                                                                  \
+        int ba_ = fbase_a, bb_ = fbase_b;                                                         \
+        asm volatile("" : "+v"(ba_), "+v"(bb_));                                                  \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                                            \
-            fa[0][i] = TA::frag(sA, (wm * TM + i) * 32, 0, lane);                                 \
+            fa[0][i] = SUB_DMA_FRAG_A(i, 0);                                                      \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
-            fb[0][j] = TB::frag(sB, (wn * TN + j) * 32, 0, lane);                                 \
+            fb[0][j] = SUB_DMA_FRAG_B(j, 0);                                                      \
         _Pragma("unroll") for (int ks = 0; ks < BK / 16; ++ks) {                                  \
             if (NW == 8 && ks == BK / 32) {                                                       \
                 /* first half: the reads of k-slices 1 and 2 between the products of 0 and 1 */   \
@@ -702,9 +727,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             }                                                                                     \
             if (ks + 1 < BK / 16) {                                                               \
                 _Pragma("unroll") for (int i = 0; i < TM; ++i)                                    \
-                    fa[(ks + 1) & 1][i] = TA::frag(sA, (wm * TM + i) * 32, ks + 1, lane);         \
+                    fa[(ks + 1) & 1][i] = SUB_DMA_FRAG_A(i, ks + 1);                              \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
-                    fb[(ks + 1) & 1][j] = TB::frag(sB, (wn * TN + j) * 32, ks + 1, lane);         \
+                    fb[(ks + 1) & 1][j] = SUB_DMA_FRAG_B(j, ks + 1);                              \
             }                                                                                     \
             _Pragma("unroll") for (int i = 0; i < TM; ++i)                                        \
                 _Pragma("unroll") for (int j = 0; j < TN; ++j)                                    \
@@ -763,6 +788,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         for (int c = nkt; c < 16; ++c) SUB_DMA_KEEP();        // a contraction shorter than 16 steps
 #undef SUB_DMA_STEP
 #undef SUB_DMA_COMPUTE
+#undef SUB_DMA_FRAG_A
+#undef SUB_DMA_FRAG_B
 #undef SUB_DMA_KEEP
 #undef SUB_DMA_ISSUE
     // surplus fetches may still be landing: drain them before LDS is reused
@@ -775,9 +802,20 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
     half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
     const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
+    // One bit per output of the ReLU-dropout epilogue (set = positive), a dword per lane and 32-row
+    // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
+    // output shape reads 1/16 of what the outputs themselves would cost it.
+    static_assert(EPI == EPI_PLAIN || 32 / RPI == 4, "four packs of 8 outputs per lane and slab");
+    const long bits_at = (((long)tile_m * tiles_n + tile_n) * NW + wave) * (TM * 64) + lane;
+    uint32_t gbits[TM];
+    if (EPI == EPI_GATE_COLSUM && g.gate_bits) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) gbits[i] = g.gate_bits[bits_at + i * 64];
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = m0 + wm * 32 * TM + i * 32;
+        uint32_t positive = 0;
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -800,11 +838,20 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             }
             if (EPI == EPI_GATE_COLSUM) {
                 // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
-                const h8 gt = *reinterpret_cast<const h8*>(g.gate + (long)mm * g.sbM + nn);
+                if (g.gate_bits) {
+                    const uint32_t bits = gbits[i] >> (8 * it);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    val[e] = (float)gt[e] > 0.f ? val[e] : (half_t)0.0f;
-                    colsum[e] += (float)val[e];
+                    for (int e = 0; e < 8; ++e) {
+                        val[e] = ((bits >> e) & 1u) ? val[e] : (half_t)0.0f;
+                        colsum[e] += (float)val[e];
+                    }
+                } else {
+                    const h8 gt = *reinterpret_cast<const h8*>(g.gate + (long)mm * g.sbM + nn);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        val[e] = (float)gt[e] > 0.f ? val[e] : (half_t)0.0f;
+                        colsum[e] += (float)val[e];
+                    }
                 }
             }
             if (EPI == EPI_RELU_DROPOUT) {
@@ -814,11 +861,14 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                 const int c = i * (32 / RPI) + it, byte = 15 - c;
                 const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
+                for (int e = 0; e < 8; ++e) {
                     val[e] = ((bits >> e) & 1u) ? (half_t)fmaxf((float)val[e], 0.f) : (half_t)0.0f;
+                    positive |= ((float)val[e] > 0.f ? 1u : 0u) << (8 * it + e);
+                }
             }
             *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
         }
+        if (EPI == EPI_RELU_DROPOUT && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
     }
     if (EPI == EPI_GATE_COLSUM) {
         // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
@@ -903,7 +953,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     for (int i = 0; i < 3; ++i) { a.sCb[i] = s.sCb[i]; a.sbb[i] = ep.sbb[i]; }
     a.alpha = alpha; a.bias = ep.bias;
     a.relu_dropout = ep.relu_dropout ? 1 : 0; a.key = ep.key;
-    a.gate = ep.gate; a.colsum = ep.colsum;
+    a.gate = ep.gate; a.colsum = ep.colsum; a.gate_bits_out = ep.gate_bits_out; a.gate_bits = ep.gate_bits;
     a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;

@@ -172,6 +172,11 @@ struct GemmEpilogue {
     // same conditions as relu_dropout (gemm_relu_dropout_ok)
     const half_t* gate = nullptr;
     float* colsum = nullptr;
+    // relu_dropout: also writes one bit per output (set = positive), M * N / 8 bytes in the kernel's
+    // own order; gate: reads those bits, written by a product of the same output shape, instead of
+    // the values of `gate` (which must still be given)
+    uint32_t* gate_bits_out = nullptr;
+    const uint32_t* gate_bits = nullptr;
 };
 // `ws` (optional): fp32 scratch of ws_floats elements for splitting the
 // contraction of small-output products across workgroups.

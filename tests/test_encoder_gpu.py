@@ -771,6 +771,52 @@ def test_compact_activation_buffers_give_the_same_results_and_refuse_the_other_g
     assert ys[0][2] < ys[1][2] - 2 * 2 * (B * Ls * 4 * E * 2 - 16)
 
 
+def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to():
+    """With lin1's fused epilogue the forward call leaves one bit per element of DROP2
+    (positive or not) in the unused SB1_LINW1 buffer, and the backward call takes its
+    ReLU gate from there -- but only from the buffer the latest forward call wrote.
+    A backward pass that belongs to an earlier forward call (here: two forward calls,
+    then the backward pass of the first) must read the gate off its own DROP2 and
+    give what a forward-backward sequence without the second call gives, bit for bit."""
+    from substation_amd import Encoder, layouts as L
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = 128, 128, 4, 256          # 256 tiles of 256x256: both products take the kernel that carries the epilogues
+
+    def make():
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
+                      profiling=True).cuda()
+        with torch.no_grad():
+            for p in enc.parameters():
+                p.mul_(0.1)
+        enc.set_rng(SEED, 0)
+        return enc
+
+    g0 = torch.Generator().manual_seed(11)
+    X1 = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
+    X2 = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
+    DY = torch.randn(B, Ls, E, generator=g0).half().cuda()
+
+    def grads(enc, X):
+        return [X.grad.clone()] + [p.grad.clone() for p in enc.parameters()]
+
+    enc = make()
+    Y1 = enc(X1)
+    enc(X2)                                  # overwrites nothing of the first call, but owns the gate bits now
+    Y1.backward(DY)
+    torch.cuda.synchronize()
+    names = [n for n, _ in enc.profile()]
+    assert 'lin1+bad' in names and 'dXlin2+bdrlb' in names, names
+    got = grads(enc, X1)
+    X1.grad = None
+    ref_enc = make()
+    ref_enc(X1).backward(DY)
+    torch.cuda.synchronize()
+    want = grads(ref_enc, X1)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
     """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
     the library's one-time allocations) and replayed with eager work in between:
