@@ -114,8 +114,9 @@ def algorithmic_work(B, L, H, E, relu_from_output=True):
     # the last launch of the backward pass with dWout's tiles in the places it leaves free
     w['dXQKV-fused+dWQKV-fused+dWout'] = ('mfma', 2 * proj[0] + outp[0], 2 * proj[1] + outp[1])
     # lin1 with bias, ReLU and dropout in its epilogue: the product's flops, SB1 and LINW1 in, DROP2 out
-    w['lin1+bad'] = ('mfma',) + ffn
-    w['dXlin2+bdrlb'] = ('mfma', ffn[0], ffn[1] + 2 * tok * U)      # the product's bytes plus the gate (DROP2) read
+    # the ReLU gate travels as one bit per element of DROP2: written by lin1's epilogue, read by dXlin2's
+    w['lin1+bad'] = ('mfma', ffn[0], ffn[1] + tok * U // 8)
+    w['dXlin2+bdrlb'] = ('mfma', ffn[0], ffn[1] + tok * U // 8)
     for n in ('out', 'dWout', 'dXout'):
         w[n] = ('mfma',) + outp
     for n in ('lin1', 'lin2', 'dXlin2', 'dWlin2', 'dXlin1', 'dWlin1'):

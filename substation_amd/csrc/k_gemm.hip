@@ -524,7 +524,8 @@ struct DTile {
     // (32 rows further the swizzle flips bit 2 of the slot, a k-step further the slot moves
     // by 2, and neither carries).  The eight-wave kernel computes that inside its loop from a
     // value the compiler cannot see through: left to itself it keeps all 24 addresses of a
-    // wave in registers across the loop and spills other things.
+    // wave in registers across the loop and spills other things.  (The four-wave kernel has
+    // the registers and got slower with it: 40 -> 43 us at M = 4096, N = 1024, K = 4096.)
     static __device__ __forceinline__ int frag_base(int row0, int lane) {
         return kc_off(row0 + (lane & 31), lane >> 5);
     }
@@ -698,15 +699,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 
     constexpr int RA_ = AKC ? 1 : 2, RB_ = BKC ? 1 : 2;      // LDS reads per fragment
     const int fbase_a = TA::frag_base(wm * TM * 32, lane), fbase_b = TB::frag_base(wn * TN * 32, lane);
-#define SUB_DMA_FRAG_A(i_, ks_) (AKC ? TA::frag_at(sA, ba_, i_, ks_) : TA::frag(sA, (wm * TM + (i_)) * 32, ks_, lane))
-#define SUB_DMA_FRAG_B(j_, ks_) (BKC ? TB::frag_at(sB, bb_, j_, ks_) : TB::frag(sB, (wn * TN + (j_)) * 32, ks_, lane))
+#define SUB_DMA_FRAG_A(i_, ks_) (AKC && NW == 8 ? TA::frag_at(sA, ba_, i_, ks_) : TA::frag(sA, (wm * TM + (i_)) * 32, ks_, lane))
+#define SUB_DMA_FRAG_B(j_, ks_) (BKC && NW == 8 ? TB::frag_at(sB, bb_, j_, ks_) : TB::frag(sB, (wn * TN + (j_)) * 32, ks_, lane))
 #define SUB_DMA_COMPUTE(stage_, nx_)                                                              \
     do {                                                                                          \
         const half_t* sA = stage_;                                                                \
         const half_t* sB = stage_ + TA::HALVES;                                                   \
         h8 fa[2][TM], fb[2][TN];                                                                  \
         int ba_ = fbase_a, bb_ = fbase_b;                                                         \
-        asm volatile("" : "+v"(ba_), "+v"(bb_));                                                  \
+        if constexpr (NW == 8) asm volatile("" : "+v"(ba_), "+v"(bb_));                           \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                                            \
             fa[0][i] = SUB_DMA_FRAG_A(i, 0);                                                      \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                            \
