@@ -193,9 +193,13 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * traffic in each of the two launches at B=8, L=512, E=1024.  Outputs and gradients
  * are bit-identical to those with the option off.  With SUB_OPT_FUSE_EPILOGUES on
  * and DROP2 in BJU order, bias, ReLU and dropout then run in the epilogue of the
- * lin1 product (profiling name `lin1+bad`) and SB1_LINW1 is not written either;
- * in encoder_backward bdrlb runs in the epilogue of the dXlin2 product
- * (`dXlin2+bdrlb`), DDROP2 is not written and DLINB1 sums its terms in another
+ * lin1 product (profiling name `lin1+bad`) and SB1_LINW1 is not written either:
+ * the first B*J*U/8 bytes of that buffer then hold one bit per element of DROP2
+ * (set where it is positive), in the kernel's own order.  In encoder_backward
+ * bdrlb runs in the epilogue of the dXlin2 product (`dXlin2+bdrlb`), which takes
+ * its gate from those bits when it is handed the SB1_LINW1 buffer that the
+ * handle's latest encoder_forward call wrote and from DROP2 itself otherwise
+ * (same results); DDROP2 is not written and DLINB1 sums its terms in another
  * order.
  * Set it to 0 before the forward call when LIN1, DROP2MASK, SB1_LINW1 or
  * DDROP2 are wanted (debug capture). */
