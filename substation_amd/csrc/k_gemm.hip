@@ -93,11 +93,11 @@ typedef short s4v __attribute__((ext_vector_type(4)));
 // bytes addressed by lane 4e + i/4.  With lane l addressing
 // T[k0 + l/4][m0 + 4*(l%4) ..+3], lane i ends up with T[k0 + 0..3][m0 + i]:
 // four consecutive k of its own row, which is what the matrix core wants.
-template <int ROWS, bool KC>
+template <int ROWS, bool KC, int NT = 256>
 struct Tile {
     static constexpr int PITCH = KC ? BK : ROWS + MC_PAD;            // halves
     static constexpr int HALVES = KC ? ROWS * BK : BK * (ROWS + MC_PAD);
-    static constexpr int NV = ROWS / 32;                              // 16-byte loads per thread
+    static constexpr int NV = ROWS * 8 / NT;                          // 16-byte loads per thread (NT threads)
     static constexpr int VPR = ROWS / 8;                              // vectors per k-row (!KC)
 
     static __device__ __forceinline__ int kc_off(int row, int slot) {
@@ -113,7 +113,7 @@ struct Tile {
         okmask = 0;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            int id = tid + i * 256;
+            int id = tid + i * NT;
             if (KC) {
                 int row = id >> 3, slot = id & 7;
                 off[i] = (unsigned)((long)row * sF + slot * 8);
@@ -137,7 +137,7 @@ struct Tile {
             if (!CHECK) {
                 v[i] = *p;
             } else {
-                int id = tid + i * 256;
+                int id = tid + i * NT;
                 bool kok = KC ? ((id & 7) * 8 + 8 <= nk) : (id / VPR < nk);
                 v[i] = (h8)(half_t)0.0f;
                 if (kok && ((okmask >> i) & 1u)) v[i] = *p;
@@ -148,7 +148,7 @@ struct Tile {
     static __device__ __forceinline__ void store(const h8 (&v)[NV], half_t* lds, int tid) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            int id = tid + i * 256;
+            int id = tid + i * NT;
             if (KC) {
                 *reinterpret_cast<h8*>(lds + kc_off(id >> 3, id & 7)) = v[i];
             } else {
@@ -179,10 +179,10 @@ struct Tile {
 
 // LDS (in halves) of one workgroup of the register-staged kernel: two pipeline
 // stages, reused by the epilogue's per-wave staging slabs.
-template <int TM, int TN, bool AKC, bool BKC>
+template <int TM, int TN, bool AKC, bool BKC, int WM = 2>
 constexpr int mfma_lds_halves() {
-    constexpr int stage = Tile<64 * TM, AKC>::HALVES + Tile<64 * TN, BKC>::HALVES;
-    constexpr int slabs = 4 * 32 * (32 * TN + 8);
+    constexpr int stage = Tile<32 * WM * TM, AKC, 128 * WM>::HALVES + Tile<64 * TN, BKC, 128 * WM>::HALVES;
+    constexpr int slabs = 2 * WM * 32 * (32 * TN + 8);
     return 2 * stage > slabs ? 2 * stage : slabs;
 }
 
@@ -204,19 +204,21 @@ __device__ __forceinline__ void sched_k_tile() {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
     if constexpr ((m) < 12) __builtin_amdgcn_sched_group_barrier(0x100, (R1 * ((m) + 1)) / 4 - (R1 * (m)) / 4, 0); \
     if constexpr ((m) < NLOAD) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);                 \
-    if constexpr ((m) >= 12) __builtin_amdgcn_sched_group_barrier(0x200, NLOAD / 4, 0);
+    if constexpr ((m) >= 12) __builtin_amdgcn_sched_group_barrier(0x200, (NLOAD * ((m) - 11)) / 4 - (NLOAD * ((m) - 12)) / 4, 0);
     SUB_SCHED_ONE(0) SUB_SCHED_ONE(1) SUB_SCHED_ONE(2) SUB_SCHED_ONE(3) SUB_SCHED_ONE(4) SUB_SCHED_ONE(5)
     SUB_SCHED_ONE(6) SUB_SCHED_ONE(7) SUB_SCHED_ONE(8) SUB_SCHED_ONE(9) SUB_SCHED_ONE(10) SUB_SCHED_ONE(11)
     SUB_SCHED_ONE(12) SUB_SCHED_ONE(13) SUB_SCHED_ONE(14) SUB_SCHED_ONE(15)
 #undef SUB_SCHED_ONE
 }
 
-// One workgroup's share of a product: block `block_id` of `nblocks`.
-template <int TM, int TN, bool AKC, bool BKC, bool FULL>
+// One workgroup's share of a product: block `block_id` of `nblocks`.  WM x 2 waves
+// (WM = 2: 256 threads; WM = 4: 512 threads and a tile twice as tall, whose workgroup
+// draws a quarter less from L2 per flop than two workgroups with square tiles).
+template <int TM, int TN, bool AKC, bool BKC, bool FULL, int WM = 2>
 __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id, long nblocks, half_t* lds) {
-    constexpr int BM = 64 * TM, BN = 64 * TN;
-    using TA = Tile<BM, AKC>;
-    using TB = Tile<BN, BKC>;
+    constexpr int BM = 32 * WM * TM, BN = 64 * TN, NT = 128 * WM;
+    using TA = Tile<BM, AKC, NT>;
+    using TB = Tile<BN, BKC, NT>;
     constexpr int STAGE = TA::HALVES + TB::HALVES;                   // one pipeline stage
     constexpr int STAGE_PITCH = 32 * TN + 8;                          // halves
     constexpr int STAGE_WAVE = 32 * STAGE_PITCH;                      // one 32-row slab per wave
@@ -456,6 +458,39 @@ __global__ __launch_bounds__(256) void k_gemm_pair(GemmArgs g1, GemmArgs g2, uns
         const unsigned id = b - both / 2;
         if (n2 > n1) gemm_mfma_body<2, 2, A2, B2, true>(g2, id, n2, lds);
         else gemm_mfma_body<2, 2, A1, B1, true>(g1, id, n1, lds);
+    }
+}
+
+// The same with 256 x 128 tiles and one workgroup of eight waves (4 x 2, each 64 x 64 as
+// above) per CU, for pairs whose tiles are then about one per CU.  What bounds these
+// products is what the L2s deliver to the CUs; the two workgroups that shared a CU each
+// fetched their own 128 rows of the second operand, the tall tile fetches them once: a
+// quarter less from L2 per flop (dXlin1 + dWlin1 at 4096 x 1024 x 4096 each: 86.5 -> 79.8 us,
+// A/B on one device).
+template <bool A1, bool B1, bool A2, bool B2>
+__global__ __launch_bounds__(512) void k_gemm_pair8(GemmArgs g1, GemmArgs g2, unsigned n1, unsigned n2, GemmArgs g3,
+                                                    unsigned n3, FinishJobs tail, unsigned tail_groups) {
+    constexpr int L1 = mfma_lds_halves<2, 2, A1, B1, 4>(), L2 = mfma_lds_halves<2, 2, A2, B2, 4>();
+    __shared__ __attribute__((aligned(16))) half_t lds[L1 > L2 ? L1 : L2];
+    const unsigned b = blockIdx.x, both = 2 * (n1 < n2 ? n1 : n2);
+    if (b >= n1 + n2) {
+        const unsigned t = b - (n1 + n2);
+        if (t < n3) {
+            gemm_mfma_body<2, 2, A2, B2, true, 4>(g3, t, n3, lds);
+        } else {
+            if (threadIdx.x >= kFinishThreads) return;        // a finishing workgroup is four waves
+            finish_block(tail.j[(t - n3) / tail_groups], (t - n3) % tail_groups, reinterpret_cast<float (*)[33]>(lds));
+        }
+        return;
+    }
+    if (b < both) {
+        const unsigned id = ((b >> 4) << 3) | (b & 7);
+        if ((b >> 3) & 1) gemm_mfma_body<2, 2, A2, B2, true, 4>(g2, id, n2, lds);
+        else gemm_mfma_body<2, 2, A1, B1, true, 4>(g1, id, n1, lds);
+    } else {
+        const unsigned id = b - both / 2;
+        if (n2 > n1) gemm_mfma_body<2, 2, A2, B2, true, 4>(g2, id, n2, lds);
+        else gemm_mfma_body<2, 2, A1, B1, true, 4>(g1, id, n1, lds);
     }
 }
 
@@ -1181,6 +1216,44 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
     const Canon cin[2] = {canonicalise(s1, A1, B1, C1, alpha1, ep1), canonicalise(s2, A2, B2, C2, alpha2, ep2)};
     PairSel sel;
     if (!pair_select(sh, cin, ws, ws_floats, third, sel)) return false;
+    {
+        // 256 x 128 tiles when they are whole, unsplit and about one per CU
+        bool ok = true;
+        long n8[3] = {0, 0, 0};
+        for (int i = 0; i < 2; ++i) {
+            const GemmArgs& a = sel.c[i].a;
+            ok = ok && a.splits == 1 && a.M % 256 == 0;
+            n8[i] = sel.n[i] / 2;
+            ok = ok && n8[i] % 8 == 0;
+        }
+        if (sel.n3) { ok = ok && sel.c3.a.M % 256 == 0; n8[2] = sel.n3 / 2; ok = ok && n8[2] % 8 == 0; }
+        else if (third && third->shape) ok = false;            // a third product was offered and did not fit
+        ok = ok && n8[0] + n8[1] + n8[2] <= 256 && n8[0] + n8[1] + n8[2] >= 192;
+        if (ok) {
+            FinishJobs tj;
+            unsigned tg = 1;
+            if (tail && tail->n > 0) {
+                const long groups = finish_groups(*tail);
+                if (groups * tail->n <= 4096) { tj = *tail; tg = (unsigned)groups; }
+            }
+            GemmArgs g3{};
+            if (sel.n3) g3 = sel.c3.a;
+            dim3 grid((unsigned)(n8[0] + n8[1] + n8[2]) + (unsigned)tj.n * tg);
+            const GemmArgs& g1 = sel.c[0].a;
+            const GemmArgs& g2 = sel.c[1].a;
+            const unsigned m1 = (unsigned)n8[0], m2 = (unsigned)n8[1], m3 = (unsigned)n8[2];
+            if (sel.variant == 0)
+                hipLaunchKernelGGL((k_gemm_pair8<true, false, false, false>), grid, dim3(512), 0, st, g1, g2, m1, m2, g3, m3, tj, tg);
+            else if (sel.variant == 1)
+                hipLaunchKernelGGL((k_gemm_pair8<false, false, false, false>), grid, dim3(512), 0, st, g1, g2, m1, m2, g3, m3, tj, tg);
+            else
+                hipLaunchKernelGGL((k_gemm_pair8<true, false, true, false>), grid, dim3(512), 0, st, g1, g2, m1, m2, g3, m3, tj, tg);
+            if (tj.n > 0) tail->n = 0;
+            if (sel.n3) third->taken = true;
+            check_launch("gemm pair (256 x 128 tiles)");
+            return true;
+        }
+    }
     // column sums of earlier launches, finished by workgroups after the tiles (none of them
     // may be a sum that this launch itself contributes to)
     FinishJobs tj;
