@@ -198,7 +198,9 @@ def test_default_path_matches_the_oracle(dims, p, masked, compact):
 
 
 @pytest.mark.parametrize('dims,which', [((8, 512, 16, 1024), 'mi355x:bert-b8-l512-h16-e1024'),
-                                        ((96, 128, 16, 1024), 'mi355x:bert-b96-l128-h16-e1024')])
+                                        ((96, 128, 16, 1024), 'mi355x:bert-b96-l128-h16-e1024'),
+                                        # 96 + 96 and 96 + 96 + 32 tiles of 256 x 128 in the paired launches
+                                        ((6, 512, 16, 1024), 'mi355x:bert-b8-l512-h16-e1024')])
 def test_bench_path_matches_the_oracle(dims, which):
     """The configuration bench.py times, in one step against the oracle: ReLU, no debug
     capture, every option at its default (bias+ReLU+dropout in the epilogue of lin1,
