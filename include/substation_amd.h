@@ -216,6 +216,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * `dXQKV-fused+dWQKV-fused+dWout`.  Needs SUB_OPT_PAIR_PRODUCTS and the
  * in-register attention (whose kernels produce the DBKQV partials). */
 #define SUB_OPT_FINISH_IN_PAIR 7
+/* SUB_OPT_SIDE_JOBS (default 1): where the 256x256 tiles of the stacked
+ * projections leave CUs idle (192 tiles on 256 CUs at B=8, L=512, E=1024),
+ * workgroups behind the tiles of that launch draw the dropout keep bits of the
+ * first key tiles of every score row for the attention launch that follows
+ * (they depend on nothing but seed, step and position); the attention kernel
+ * draws the rest.  Same bits, same results.  Needs the in-register attention
+ * and SUB_OPT_FUSE_EPILOGUES. */
+#define SUB_OPT_SIDE_JOBS 8
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

@@ -21,6 +21,7 @@ OPT_FUSE_ATTENTION = 4
 OPT_PAIR_PRODUCTS = 5
 OPT_RELU_FROM_OUTPUT = 6
 OPT_FINISH_IN_PAIR = 7
+OPT_SIDE_JOBS = 8
 FUSE_REQUIRED = 2
 
 

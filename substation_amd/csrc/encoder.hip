@@ -204,6 +204,7 @@ struct Handle {
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
     bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
+    bool side_jobs = true;            // CUs that a product's tiles leave idle draw dropout bits for the launch after it
     // where the last forward call's lin1 epilogue left one bit per element of DROP2 (set = positive), or
     // null: the unused SB1_LINW1 buffer of that call.  The backward call reads its gate from there when it
     // is handed the same buffer, and from DROP2 itself otherwise.
@@ -493,7 +494,7 @@ void ensure_gws(Handle& h, size_t floats) {
 }
 
 void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const char* name,
-              const void* addend = nullptr) {
+              const void* addend = nullptr, GemmSideJob* side = nullptr) {
     ProfScope ps(h, name);
     const GemmPlan& p = h.gemm[id];
     GemmEpilogue ep;
@@ -503,7 +504,7 @@ void run_gemm(Handle& h, int id, const void* A, const void* B, void* C, const ch
     }
     ensure_gws(h, h.gws_need);
     launch_gemm(p.shape, (const half_t*)A, (const half_t*)B, (half_t*)C, p.alpha, ep, h.stream, h.gws,
-                h.gws_floats);
+                h.gws_floats, side);
 }
 
 // Two products that do not depend on one another (a data gradient and the weight
@@ -865,17 +866,24 @@ void forward(Handle& h, const FwdPtrs& t) {
     h.prof_used = 0;
     h.prof_forward = 0;
     void* const* W = t.W; void* const* F = t.F;
+    AttnArgs at;
+    const bool fused_attention = attention_fused(h, F, at);
     if (h.fuse_epilogues && h.gemm[G_QKV_BIAS].ok && aligned16(W[BKQV]) && aligned16(F[KKQQVV])) {
-        // projection + bias in one pass; WKKWQQWVV (the pre-bias copy) is not written
-        run_gemm(h, G_QKV_BIAS, t.X, W[WKQV], F[KKQQVV], "QKV-fused", W[BKQV]);
+        // projection + bias in one pass; WKKWQQWVV (the pre-bias copy) is not written.  The CUs its tiles
+        // leave idle draw part of the attention's dropout bits, which depend on nothing but the seed.
+        GemmSideJob side;
+        if (fused_attention && h.side_jobs) {
+            side.key = make_key(h, SUB_SITE_SOFTMAX, h.p_softmax);
+            side.keep = at.keep; side.rows = (uint32_t)((long)at.H * at.B * at.J); side.nk = (uint32_t)at.K;
+        }
+        run_gemm(h, G_QKV_BIAS, t.X, W[WKQV], F[KKQQVV], "QKV-fused", W[BKQV], &side);
+        at.keep_tiles_ready = side.tiles_done;
     } else {
         run_gemm(h, G_QKV, t.X, W[WKQV], F[WKKWQQWVV], "QKV-fused");
         ProfScope ps(h, "aib");
         op_aib(h, F[WKKWQQWVV], h.lf[WKKWQQWVV], W[BKQV], h.lp[BKQV], F[KKQQVV], h.lf[KKQQVV]);
     }
     half_t* KK = sub_q(F[KKQQVV], h, 0); half_t* QQ = sub_q(F[KKQQVV], h, 1); half_t* VV = sub_q(F[KKQQVV], h, 2);
-    AttnArgs at;
-    const bool fused_attention = attention_fused(h, F, at);
     if (fused_attention) {
         ProfScope ps(h, "attention");
         mask_plan(h, at, true);
@@ -1304,6 +1312,7 @@ int sub_get_option(void* handle, int option, int* value) {
         else if (option == SUB_OPT_PAIR_PRODUCTS) *value = h.pair_products;
         else if (option == SUB_OPT_RELU_FROM_OUTPUT) *value = h.relu_from_output;
         else if (option == SUB_OPT_FINISH_IN_PAIR) *value = h.finish_in_pair;
+        else if (option == SUB_OPT_SIDE_JOBS) *value = h.side_jobs;
         else fail("sub_get_option: unknown option");
     });
 }
@@ -1317,6 +1326,7 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_PAIR_PRODUCTS) h.pair_products = value != 0;
         else if (option == SUB_OPT_RELU_FROM_OUTPUT) h.relu_from_output = value != 0;
         else if (option == SUB_OPT_FINISH_IN_PAIR) h.finish_in_pair = value != 0;
+        else if (option == SUB_OPT_SIDE_JOBS) h.side_jobs = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;

@@ -43,7 +43,24 @@ struct GemmArgs {
     float* colsum = nullptr;
     uint32_t* gate_bits_out = nullptr;     // relu_dropout: one bit per output, set where it is positive
     const uint32_t* gate_bits = nullptr;   // gate: those bits instead of the values of `gate`
+    // GemmSideJob of the eight-wave asynchronous kernel: workgroups side_first .. gridDim.x - 1 draw
+    // the attention keep words of key tiles 0 .. side_tiles_done - 1 of side_rows score rows
+    unsigned side_first = 0, side_blocks = 0;
+    PhiloxKey side_key;
+    uint32_t* side_keep = nullptr;
+    uint32_t side_rows = 0, side_nk = 0, side_tiles_done = 0;
 };
+
+// A workgroup that multiplies nothing (see GemmSideJob): workgroup sb of nsb.
+__device__ __forceinline__ void side_block(const GemmArgs& g, unsigned sb, unsigned nsb) {
+    const PhiloxKey key = resolved(g.side_key);
+    const uint32_t nt = g.side_nk / 32, td = g.side_tiles_done;
+    const uint64_t total = (uint64_t)g.side_rows * td, stride = (uint64_t)nsb * blockDim.x;
+    for (uint64_t w = (uint64_t)sb * blockDim.x + threadIdx.x; w < total; w += stride) {
+        const uint32_t row = (uint32_t)(w / td), t = (uint32_t)(w - (uint64_t)row * td);
+        g.side_keep[(size_t)row * nt + t] = attention_keep_word(key, row, g.side_nk, t);
+    }
+}
 
 // ---------------------------------------------------------------------------
 // Scalar fallback: any strides, any sizes.  One thread per output element.
@@ -652,7 +669,13 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     const int tiles_m = g.M / BM, tiles_n = g.N / BN;
     long lid = blockIdx.x;
     {
-        const long nblocks = gridDim.x;
+        long nblocks = gridDim.x;
+        if constexpr (NW == 8 && EPI == EPI_PLAIN) {
+            if (g.side_blocks) {
+                if (blockIdx.x >= g.side_first) { side_block(g, blockIdx.x - g.side_first, g.side_blocks); return; }
+                nblocks = g.side_first;
+            }
+        }
         if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
     }
     const int per_batch = tiles_m * tiles_n;
@@ -1082,7 +1105,7 @@ void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, bool dma, hi
     long nblocks = (long)((a.N + 64 * TN - 1) / (64 * TN)) * ((a.M + 64 * TM - 1) / (64 * TM)) * batch *
                    a.splits;
     if (nblocks > 0x7fffffffL) fail("gemm: too many tiles");
-    dim3 grid((unsigned)nblocks);
+    dim3 grid((unsigned)nblocks + a.side_blocks);
     const bool full = a.M % (64 * TM) == 0 && a.N % (64 * TN) == 0 && a.K1 % BK == 0;
     if (DMA_OK && full && dma && a.splits == 1) { launch_dma<TM, TN>(a, akc, bkc, grid, st); return; }
     if (full) launch_mfma2<TM, TN, true>(a, akc, bkc, grid, st);
@@ -1288,7 +1311,7 @@ bool launch_gemm_pair(const GemmShape& s1, const half_t* A1, const half_t* B1, h
 }
 
 void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C, float alpha,
-                 const GemmEpilogue& ep, hipStream_t st, float* ws, size_t ws_floats) {
+                 const GemmEpilogue& ep, hipStream_t st, float* ws, size_t ws_floats, GemmSideJob* side) {
     long batch = s.batch();
     if (batch == 0 || s.M == 0 || s.N == 0) return;
     Canon c = canonicalise(s, A, B, C, alpha, ep);
@@ -1304,6 +1327,25 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             c.a.partial = ws;
         }
         const int tile = pick_tile(c.a, batch, akc, bkc);
+        if (side) side->tiles_done = 0;
+        if (side && side->keep && side->key.thr && tile == 44 && !ep.relu_dropout && !ep.gate && c.a.splits == 1) {
+            // CUs the tiles leave idle draw attention keep bits meanwhile: what fits into the time the
+            // product takes (about 9 us + 1.5 us per k-tile; a CU draws 1450 Philox groups per us, measured:
+            // with all 16 key tiles of the bench workload the launch takes 45 instead of 34 us)
+            const long tiles = (long)(c.a.M / 256) * (c.a.N / 256) * batch;
+            const long idle = 256 - tiles, nkt = (long)c.a.K0 * (c.a.K1 / BK);
+            if (tiles >= 128 && idle >= 32 && side->nk % 32 == 0) {
+                                const double groups = (double)idle * (9.0 + 1.5 * (double)nkt) * 1400.0;
+                long td = (long)(groups / (4.0 * (double)side->rows));
+                if (td > side->nk / 32) td = side->nk / 32;
+                if (td > 0) {
+                    c.a.side_first = (unsigned)tiles; c.a.side_blocks = (unsigned)idle;
+                    c.a.side_key = side->key; c.a.side_keep = side->keep;
+                    c.a.side_rows = side->rows; c.a.side_nk = side->nk; c.a.side_tiles_done = (uint32_t)td;
+                    side->tiles_done = (uint32_t)td;
+                }
+            }
+        }
         if ((ep.relu_dropout || ep.gate) && (tile != 44 || batch != 1 || s.sCN != 1 || s.sCM != s.N))
             fail("gemm: the ReLU-dropout epilogue needs the 256x256 asynchronous kernel (see gemm_relu_dropout_ok)");
         const bool dma = akc && bkc && tiles128 <= 384;

@@ -135,36 +135,6 @@ __device__ __forceinline__ void store_rows(const AttnSide& t, unsigned h, unsign
         }
 }
 
-// x ^ y ^ k in one instruction (k uniform).
-__device__ __forceinline__ uint32_t xor3(uint32_t x, uint32_t y, uint32_t k) {
-    uint32_t r;
-    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0x96" : "=v"(r) : "v"(x), "v"(y), "s"(k));
-    return r;
-}
-
-// philox_group() of sub_philox.hpp, bit for bit, with the two xors of each
-// half-round folded into one instruction.
-__device__ __forceinline__ U4 philox_group_dev(const PhiloxKey& k, uint64_t g) {
-    U4 c;
-    c.x = (uint32_t)g; c.y = (uint32_t)(g >> 32); c.z = k.site; c.w = k.step;
-    uint32_t k0 = k.k0, k1 = k.k1;
-#pragma unroll
-    for (int r = 0; r < 10; ++r) {
-        uint32_t hi0, lo0, hi1, lo1;
-        mulhilo(0xD2511F53u, c.x, hi0, lo0);
-        mulhilo(0xCD9E8D57u, c.z, hi1, lo1);
-        U4 n;
-        n.x = xor3(hi1, c.y, k0);
-        n.y = lo1;
-        n.z = xor3(hi0, c.w, k1);
-        n.w = lo0;
-        c = n;
-        k0 += 0x9E3779B9u;
-        k1 += 0xBB67AE85u;
-    }
-    return c;
-}
-
 // x where bit `pos` of `bits` is set, else +0.0
 __device__ __forceinline__ float keep_if(float x, uint32_t bits, int pos) {
     return __int_as_float(__float_as_int(x) & __builtin_amdgcn_sbfe((int)bits, pos, 1));
@@ -186,13 +156,6 @@ __device__ __forceinline__ void column_sums(const f16v (&acc)[P / 32], float sca
         }
     __syncthreads();
     if (tid < P) out[tid] = (red[tid] + red[P + tid]) + (red[2 * P + tid] + red[3 * P + tid]);
-}
-
-__device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
-    uint32_t b = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) b |= (field16(r, i) >= thr ? 1u : 0u) << i;
-    return b;
 }
 
 // Additive attention mask (substation/attention.py:65-68: added to the raw scores,
@@ -407,14 +370,16 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         // keep bits of the 32 scores (this query, keys of tile t): each half of the
         // wave draws two of the four groups of 8 and the halves trade them
         uint32_t word = 0xffffffffu;
-        if (key.thr) {
+        if (key.thr && t < a.keep_tiles_ready) {
+            word = a.keep[(size_t)row * nt + t];                     // drawn ahead of this launch
+        } else if (key.thr) {
             const uint64_t g0 = (uint64_t)row * (a.K / 8) + 4 * t + 2 * hi;
             const uint32_t mine = keep8(philox_group_dev(key, g0), key.thr) |
                                   (keep8(philox_group_dev(key, g0 + 1), key.thr) << 8);
             const uint32_t other = (uint32_t)__shfl_xor((int)mine, 32);
             word = hi ? (other | (mine << 16)) : (mine | (other << 16));
         }
-        if (hi == 0) a.keep[(size_t)row * nt + t] = word;
+        if (hi == 0 && t >= a.keep_tiles_ready) a.keep[(size_t)row * nt + t] = word;
         const uint32_t nib = word >> (hi * 4);                       // bit reg_pos(v, 0) of nib = keep of register v
 
         // Running softmax with a reference value per query that trails the running

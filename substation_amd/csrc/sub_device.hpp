@@ -154,6 +154,52 @@ __device__ __forceinline__ PhiloxKey resolved(PhiloxKey k) {
     return k;
 }
 
+// x ^ y ^ k in one instruction (k uniform).
+__device__ __forceinline__ uint32_t xor3(uint32_t x, uint32_t y, uint32_t k) {
+    uint32_t r;
+    asm("v_bitop3_b32 %0, %1, %2, %3 bitop3:0x96" : "=v"(r) : "v"(x), "v"(y), "s"(k));
+    return r;
+}
+
+// philox_group() of sub_philox.hpp, bit for bit, with the two xors of each
+// half-round folded into one instruction.
+__device__ __forceinline__ U4 philox_group_dev(const PhiloxKey& k, uint64_t g) {
+    U4 c;
+    c.x = (uint32_t)g; c.y = (uint32_t)(g >> 32); c.z = k.site; c.w = k.step;
+    uint32_t k0 = k.k0, k1 = k.k1;
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        uint32_t hi0, lo0, hi1, lo1;
+        mulhilo(0xD2511F53u, c.x, hi0, lo0);
+        mulhilo(0xCD9E8D57u, c.z, hi1, lo1);
+        U4 n;
+        n.x = xor3(hi1, c.y, k0);
+        n.y = lo1;
+        n.z = xor3(hi0, c.w, k1);
+        n.w = lo0;
+        c = n;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+    return c;
+}
+
+// Keep bits of the 8 elements of one Philox group: bit i set = 16-bit field i >= thr.
+__device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
+    uint32_t b = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) b |= (field16(r, i) >= thr ? 1u : 0u) << i;
+    return b;
+}
+
+// The 32 keep bits of key tile t of score row `row` in the attention kernels' format (bit k =
+// key 32 t + k of a row of nk keys): four Philox groups.
+__device__ __forceinline__ uint32_t attention_keep_word(const PhiloxKey& key, uint64_t row, uint32_t nk, uint32_t t) {
+    const uint64_t g0 = row * (nk / 8) + 4 * t;
+    return keep8(philox_group_dev(key, g0), key.thr) | (keep8(philox_group_dev(key, g0 + 1), key.thr) << 8) |
+           (keep8(philox_group_dev(key, g0 + 2), key.thr) << 16) | (keep8(philox_group_dev(key, g0 + 3), key.thr) << 24);
+}
+
 // d(LN input) of one element: g * istd - c1 - diff * c2, with the contraction
 // into FMAs spelled out so that every kernel that evaluates it rounds alike.
 __device__ __forceinline__ float ln_bwd_value(float g, float diff, float istd, float c1, float c2) {

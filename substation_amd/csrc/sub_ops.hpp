@@ -125,6 +125,9 @@ struct AttnArgs {
     float* lse = nullptr;      // [H*B*J]  log2-domain log-sum-exp of each score row
     float* dsum = nullptr;     // [H*B*J]  row sums of dO o O (written by the dQ launch, read by the dK/dV one)
     uint32_t* keep = nullptr;  // [H*B*J][K/32]  keep bits of the softmax dropout, bit k%32 of word k/32
+    // forward: the words of key tiles 0 .. keep_tiles_ready-1 of every row are in `keep` already
+    // (GemmSideJob); the kernel draws and stores the others
+    uint32_t keep_tiles_ready = 0;
     int H = 0, B = 0, J = 0, K = 0;
     float alpha = 1.f;         // score scale
     // optional (backward): per-workgroup sums over positions of the rounded dq resp.
@@ -178,10 +181,22 @@ struct GemmEpilogue {
     uint32_t* gate_bits_out = nullptr;
     const uint32_t* gate_bits = nullptr;
 };
+// Work that needs no memory path, offered to a product whose 256x256 tiles leave CUs idle: the
+// keep bits of the attention dropout (attention_keep_word) for the first `tiles_done` key tiles of
+// every score row, drawn by workgroups behind the product's tiles on the CUs these leave free.
+// launch_gemm sets tiles_done (0: not taken) from the number of idle CUs and the length of the
+// product; the attention kernel then draws only the other tiles' bits itself.
+struct GemmSideJob {
+    PhiloxKey key;
+    uint32_t* keep = nullptr;       // [rows][nk / 32]
+    uint32_t rows = 0, nk = 0;
+    uint32_t tiles_done = 0;        // out
+};
 // `ws` (optional): fp32 scratch of ws_floats elements for splitting the
 // contraction of small-output products across workgroups.
 void launch_gemm(const GemmShape& g, const half_t* A, const half_t* B, half_t* C, float alpha,
-                 const GemmEpilogue& ep, hipStream_t st, float* ws = nullptr, size_t ws_floats = 0);
+                 const GemmEpilogue& ep, hipStream_t st, float* ws = nullptr, size_t ws_floats = 0,
+                 GemmSideJob* side = nullptr);
 // Can launch_gemm apply ep.relu_dropout to this product?  Only the asynchronous kernel with
 // 256x256 tiles does, on a single dense row-major output.
 bool gemm_relu_dropout_ok(const GemmShape& g, const void* A, const void* B, const void* C, const GemmEpilogue& ep);
