@@ -1335,7 +1335,7 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
             const long tiles = (long)(c.a.M / 256) * (c.a.N / 256) * batch;
             const long idle = 256 - tiles, nkt = (long)c.a.K0 * (c.a.K1 / BK);
             if (tiles >= 128 && idle >= 32 && side->nk % 32 == 0) {
-                                const double groups = (double)idle * (9.0 + 1.5 * (double)nkt) * 1400.0;
+                                const double groups = (double)idle * (9.0 + 1.5 * (double)nkt) * 1300.0;   // a tenth of margin
                 long td = (long)(groups / (4.0 * (double)side->rows));
                 if (td > side->nk / 32) td = side->nk / 32;
                 if (td > 0) {
