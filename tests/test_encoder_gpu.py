@@ -819,6 +819,35 @@ def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to():
         assert torch.equal(a, b)
 
 
+def test_keep_bits_drawn_beside_the_projections_are_the_same_bits():
+    """At B=8 L=512 E=1024 the stacked projections have 192 tiles for 256 CUs and the
+    launch draws the attention's dropout keep bits for the first key tiles of every
+    score row on the idle ones (option 8); the attention kernel draws the rest.  With
+    the option off it draws them all: outputs and gradients must be bit-identical."""
+    from substation_amd import Encoder, layouts as L, _lib
+    lay = L.mi355x_layouts()
+    B, Ls, H, E = 8, 512, 16, 1024
+
+    def run(side_jobs):
+        torch.manual_seed(0)
+        enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED).cuda()
+        with torch.no_grad():
+            for p in enc.parameters():
+                p.mul_(0.05)
+        enc.set_rng(SEED, 3)
+        enc._handle.set_option(_lib.OPT_SIDE_JOBS, int(side_jobs))
+        g0 = torch.Generator().manual_seed(5)
+        X = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
+        DY = torch.randn(B, Ls, E, generator=g0).half().cuda()
+        Y = enc(X)
+        Y.backward(DY)
+        torch.cuda.synchronize()
+        return [Y.detach().clone(), X.grad.clone()] + [p.grad.clone() for p in enc.parameters()]
+
+    for a, b in zip(run(True), run(False)):
+        assert torch.equal(a, b)
+
+
 def test_hip_graph_replays_match_eager_and_draw_new_masks():
     """Forward + backward recorded in a HIP graph (after an eager warm-up that makes
     the library's one-time allocations) and replayed with eager work in between:
