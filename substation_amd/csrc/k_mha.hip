@@ -386,6 +386,16 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         // maximum by up to RESCALE_SLACK (in log2 units): the accumulators are only
         // rescaled when some query of the wave outgrows its reference by more, which
         // after the first tiles is rare.  Scores and reference are in raw units.
+        // The exponentials are taken against the reference as it stands, beside the search
+        // for the tile's maximum rather than behind it (the chain maximum -> exchange between
+        // the wave's halves -> vote -> exponentials left the wave with nothing to issue), and
+        // again in the rare case that the reference moves.
+        float ex[16];
+        {
+            const float mc0 = m_ref == -INFINITY ? 0.f : -m_ref * c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ex[v] = __builtin_amdgcn_exp2f(fmaf(s[v], c, mc0));
+        }
         float mt = s[0];
 #pragma unroll
         for (int v = 1; v < 16; ++v) mt = fmaxf(mt, s[v]);
@@ -401,14 +411,14 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
             for (int pt = 0; pt < G::NPT; ++pt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[pt][v] *= corr;
+            // (masked: a query whose keys so far are all masked out has no reference yet)
+            const float mc = m_ref == -INFINITY ? 0.f : -m_ref * c;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) ex[v] = __builtin_amdgcn_exp2f(fmaf(s[v], c, mc));
         }
-        // (masked: a query whose keys so far are all masked out has no reference yet)
-        const float mc = (MASKED && m_ref == -INFINITY) ? 0.f : -m_ref * c;
         h8 pb[2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = fmaf(s[v], c, mc);
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = __builtin_amdgcn_exp2f(s[v]);
+        for (int v = 0; v < 16; ++v) s[v] = ex[v];
         {   // four partial sums: a single one would be a chain of 16 dependent additions
             float l4[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
