@@ -376,8 +376,10 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
             const uint64_t g0 = (uint64_t)row * (a.K / 8) + 4 * t + 2 * hi;
             const uint32_t mine = keep8(philox_group_dev(key, g0), key.thr) |
                                   (keep8(philox_group_dev(key, g0 + 1), key.thr) << 8);
-            const uint32_t other = (uint32_t)__shfl_xor((int)mine, 32);
-            word = hi ? (other | (mine << 16)) : (mine | (other << 16));
+            // v_permlane32_swap on two copies: [0] holds the lower half's value in both halves
+            // of the wave, [1] the upper half's
+            const auto both = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
+            word = both[0] | (both[1] << 16);
         }
         if (hi == 0 && t >= a.keep_tiles_ready) a.keep[(size_t)row * nt + t] = word;
         const uint32_t nib = word >> (hi * 4);                       // bit reg_pos(v, 0) of nib = keep of register v
@@ -399,7 +401,10 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         float mt = s[0];
 #pragma unroll
         for (int v = 1; v < 16; ++v) mt = fmaxf(mt, s[v]);
-        mt = fmaxf(mt, __shfl_xor(mt, 32));
+        {
+            const auto both = __builtin_amdgcn_permlane32_swap(__float_as_uint(mt), __float_as_uint(mt), false, false);
+            mt = fmaxf(__uint_as_float(both[0]), __uint_as_float(both[1]));
+        }
         if (__builtin_amdgcn_ballot_w64(mt > m_ref + slack) != 0) {
             const float m_new = fmaxf(m_ref, mt);
             // (masked: a query that has seen no key yet has nothing to rescale; the
