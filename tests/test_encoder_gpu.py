@@ -184,6 +184,9 @@ OUTPUTS = ['SB2', 'DX', 'DWKQV', 'DBKQV', 'DWO', 'DBO', 'DS1', 'DB1', 'DLINB1', 
     ((2, 256, 4, 256), 0.1, False, True),
     ((1, 256, 2, 256), 0.2, True, False),         # head size 128, causal mask
     ((4, 512, 4, 256), 0.1, False, False),
+    # causal mask at a size where idle CUs of the projections' launch draw part of the keep bits,
+    # also for tiles the mask then leaves out
+    ((8, 512, 16, 1024), 0.1, True, True),
 ])
 def test_default_path_matches_the_oracle(dims, p, masked, compact):
     """Output, DX and the 12 gradients of the layer as shipped -- attention with the
