@@ -224,6 +224,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * draws the rest.  Same bits, same results.  Needs the in-register attention
  * and SUB_OPT_FUSE_EPILOGUES. */
 #define SUB_OPT_SIDE_JOBS 8
+/* SUB_OPT_PACKED_MASKS (default 1; embedding size a multiple of 8): the masks of
+ * the two residual dropouts travel from encoder_forward to encoder_backward as one
+ * bit per element (byte (b*J + j)*I/8 + i/8, bit i%8, canonical order whatever
+ * the tensor's layout) in the first B*J*I/8 bytes of the DROP1MASK and DROP3MASK
+ * buffers, instead of as 0/1 tensors: 7.5 MiB less to write and to read per mask at
+ * B=8, L=512, E=1024.  Same results.  Set it to 0 before the forward call when the
+ * mask tensors are wanted (debug capture); both calls must see the same value. */
+#define SUB_OPT_PACKED_MASKS 9
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

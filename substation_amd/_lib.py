@@ -22,6 +22,7 @@ OPT_PAIR_PRODUCTS = 5
 OPT_RELU_FROM_OUTPUT = 6
 OPT_FINISH_IN_PAIR = 7
 OPT_SIDE_JOBS = 8
+OPT_PACKED_MASKS = 9
 FUSE_REQUIRED = 2
 
 

@@ -26,11 +26,12 @@ constexpr int LN_WPB = LN_BLOCK / WAVE;
 template <int VPL>
 struct LnRow {
     h8 in[VPL], d1[VPL], d2[VPL], dl[VPL], df[VPL], mk[VPL];
+    uint32_t mkb[VPL];          // PACKED: the mask of the pack as 8 bits, in place of mk
     float is;
     RowIdx ix;
 };
 
-template <int VPL, bool EXT>
+template <int VPL, bool EXT, bool PACKED>
 __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs& a, unsigned row, int lane,
                                             const int (&nv)[VPL], LnRow<VPL>& r) {
     r.ix = row_index(rs, row);
@@ -42,6 +43,7 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
     for (int c = 0; c < VPL; ++c) {
         const int e0 = (c * WAVE + lane) * 8;
         r.in[c] = r.d1[c] = r.d2[c] = r.dl[c] = r.df[c] = r.mk[c] = (h8)(half_t)0.0f;
+        r.mkb[c] = 0;
         if (nv[c]) {
             r.in[c] = ldg8<true>(a.in.p + oin + e0);          // saved by the forward pass
             // the incoming gradient of the plain form is the caller's tensor;
@@ -52,14 +54,15 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
                 r.dl[c] = ldg8<true>(a.dlinear.p + odl + e0);
             }
             r.df[c] = ldg8<true>(a.diff.p + odf + e0);
-            r.mk[c] = ldg8<true>(a.mask.p + omk + e0);
+            if (PACKED) r.mkb[c] = a.mask_bits[(size_t)row * (rs.R >> 3) + (c * WAVE + lane)];
+            else r.mk[c] = ldg8<true>(a.mask.p + omk + e0);
         }
     }
 }
 
 // VPL: 128-bit packs per lane and row (row length <= VPL * 512).  EXT: the
 // extended form (two incoming gradients, linear-bias and output-bias sums).
-template <int VPL, bool EXT>
+template <int VPL, bool EXT, bool PACKED>
 __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, float* ws, unsigned nrows) {
     constexpr int NS = EXT ? 4 : 2;
     __shared__ float red[LN_WPB][VPL * WAVE * 8];
@@ -83,11 +86,11 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
     const unsigned stride = gridDim.x * LN_WPB;
     unsigned row = blockIdx.x * LN_WPB + wave;
     LnRow<VPL> cur, nxt;
-    if (row < nrows) ln_load_row<VPL, EXT>(rs, a, row, lane, nv, cur);
+    if (row < nrows) ln_load_row<VPL, EXT, PACKED>(rs, a, row, lane, nv, cur);
     for (; row < nrows; row += stride) {
         // the next row's loads are in flight while this one is worked on
         const bool more = row + stride < nrows;
-        if (more) ln_load_row<VPL, EXT>(rs, a, row + stride, lane, nv, nxt);
+        if (more) ln_load_row<VPL, EXT, PACKED>(rs, a, row + stride, lane, nv, nxt);
         float g[VPL][8], df[VPL][8];
         float s1 = 0.f, s2 = 0.f;
         const long og = view_offset(a.g, cur.ix);
@@ -129,7 +132,8 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
             x = pin(x);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                y[i] = cur.mk[c][i] != (half_t)0.0f ? x[i] : (half_t)0.0f;
+                const bool kept = PACKED ? ((cur.mkb[c] >> i) & 1u) != 0 : cur.mk[c][i] != (half_t)0.0f;
+                y[i] = kept ? x[i] : (half_t)0.0f;
                 if (EXT) acc[3][c][i] += (float)y[i];
             }
             stg8<false>(a.d_ln_in.p + oa + e0, x);
@@ -170,7 +174,7 @@ inline int lnbwd_blocks(long nrows) {
 bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext) {
     if (rs.R <= 0 || rs.R > 1024 || rs.R % 8 != 0) return false;
     if (rs.rows() <= 0 || rs.rows() >= (1L << 31)) return false;
-    bool ok = a.in.vec && a.d1.vec && a.diff.vec && a.mask.vec && a.g.vec && a.d_ln_in.vec && a.d_drop_in.vec &&
+    bool ok = a.in.vec && a.d1.vec && a.diff.vec && (a.mask.vec || a.mask_bits) && a.g.vec && a.d_ln_in.vec && a.d_drop_in.vec &&
               a.scale.vec;
     if (ext) ok = ok && a.d2.vec && a.dlinear.vec;
     return ok;
@@ -187,13 +191,19 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     const unsigned nrows = (unsigned)rs.rows();
     const int blocks = lnbwd_blocks(nrows);
     const int vpl = rs.R <= 512 ? 1 : 2;
+#define SUB_LNBWD(VPL_, EXT_)                                                                                     \
+    do {                                                                                                          \
+        if (a.mask_bits) hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+        else hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);            \
+    } while (0)
     if (ext) {
-        if (vpl == 1) hipLaunchKernelGGL((k_lnbwd<1, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
-        else hipLaunchKernelGGL((k_lnbwd<2, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+        if (vpl == 1) SUB_LNBWD(1, true);
+        else SUB_LNBWD(2, true);
     } else {
-        if (vpl == 1) hipLaunchKernelGGL((k_lnbwd<1, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
-        else hipLaunchKernelGGL((k_lnbwd<2, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);
+        if (vpl == 1) SUB_LNBWD(1, false);
+        else SUB_LNBWD(2, false);
     }
+#undef SUB_LNBWD
     check_launch("fused LayerNorm backward");
     FinishArgs fo{{sums[0], sums[1], sums[2], sums[3]}, 0, 0, 1, 1};
     FinishJob job{ws, fo, ext ? 4 : 2, 1, blocks, rs.R};

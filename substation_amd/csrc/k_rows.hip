@@ -165,7 +165,7 @@ template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resid, View lin_bias,
                                                  View scale, View bias, View lin, View mask,
                                                  View diff, View normed, View out, View istd,
-                                                 PhiloxKey key_, float eps, unsigned nrows) {
+                                                 PhiloxKey key_, float eps, unsigned nrows, uint8_t* mask_bits) {
     const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63;
     const unsigned step = gridDim.x * WPB * RPW;
@@ -202,7 +202,8 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                 }
                 if (nv > 0) {
                     st8h<FAST, true>(lin, ol, e0, nv, lh);
-                    st8h<FAST, true>(mask, om, e0, nv, mask_h8(bits[r][c]));
+                    if (mask_bits) mask_bits[(size_t)(row0 + r) * (rs.R >> 3) + (c * WAVE + lane)] = (uint8_t)bits[r][c];
+                    else st8h<FAST, true>(mask, om, e0, nv, mask_h8(bits[r][c]));
                 }
             }
         }
@@ -255,7 +256,8 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
 
 template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View istd, View diff,
-                                                 View mask, View d_ln_in, View d_drop_in, unsigned nrows) {
+                                                 View mask, View d_ln_in, View d_drop_in, unsigned nrows,
+                                                 const uint8_t* mask_bits) {
     const int lane = threadIdx.x & 63;
     const unsigned step = gridDim.x * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;
@@ -276,7 +278,14 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
                 F8 fg = ld8<FAST, true>(dout, oo, e0, nv), fd = ld8<FAST, true>(diff, od, e0, nv);
-                F8 fm = ld8<FAST, true>(mask, om, e0, nv);
+                F8 fm;
+                if (mask_bits) {
+                    const uint32_t b = nv > 0 ? mask_bits[(size_t)(row0 + r) * (rs.R >> 3) + (c * WAVE + lane)] : 0u;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) fm.v[i] = (float)((b >> i) & 1u);
+                } else {
+                    fm = ld8<FAST, true>(mask, om, e0, nv);
+                }
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     g[r][c][i] = fg.v[i];
@@ -423,24 +432,26 @@ void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta
 
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st) {
+                  float eps, hipStream_t st, uint8_t* mask_bits) {
+    if (mask_bits && rs.R % 8) fail("bias-dropout-residual-layernorm: a bit mask needs rows of whole 8-packs");
     unsigned nrows = check_rows(rs, "bias-dropout-residual-layernorm");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "bias-dropout-residual-layernorm");
-    bool fast = in.vec && resid.vec && lin_bias.vec && scale.vec && bias.vec && lin.vec && mask.vec &&
+    bool fast = in.vec && resid.vec && lin_bias.vec && scale.vec && bias.vec && lin.vec && (mask.vec || mask_bits) &&
                 diff.vec && normed.vec && out.vec;
     SUB_ROW_DISPATCH(k_bdrln, vpl, fast, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
-                     out, istd, key, eps, nrows);
+                     out, istd, key, eps, nrows, mask_bits);
     check_launch("bias-dropout-residual-layernorm");
 }
 
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
-                  View d_drop_in, hipStream_t st) {
+                  View d_drop_in, hipStream_t st, const uint8_t* mask_bits) {
+    if (mask_bits && rs.R % 8) fail("layernorm backward: a bit mask needs rows of whole 8-packs");
     unsigned nrows = check_rows(rs, "layernorm backward");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "layernorm backward");
-    bool fast = dout.vec && diff.vec && mask.vec && d_ln_in.vec && d_drop_in.vec;
-    SUB_ROW_DISPATCH(k_blnrd, vpl, fast, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows);
+    bool fast = dout.vec && diff.vec && (mask.vec || mask_bits) && d_ln_in.vec && d_drop_in.vec;
+    SUB_ROW_DISPATCH(k_blnrd, vpl, fast, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows, mask_bits);
     check_launch("layernorm backward");
 }
 

@@ -21,11 +21,14 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
                     float scale, float mscale, PhiloxKey key, hipStream_t st);
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st);
+// mask_bits (optional; rows of whole 8-packs): the dropout mask as one bit per element in canonical
+// order -- byte row * R / 8 + e / 8, bit e % 8 -- instead of the 0/1 tensor `mask`, which is then
+// neither written (bdrln) nor read (blnrd, the fused LayerNorm backward): 1/16 of the bytes.
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st);
+                  float eps, hipStream_t st, uint8_t* mask_bits = nullptr);
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
-                  View d_drop_in, hipStream_t st);
+                  View d_drop_in, hipStream_t st, const uint8_t* mask_bits = nullptr);
 
 // --- elementwise operators ---------------------------------------------------
 // out_only: neither LIN (input + bias) nor the mask is written, only the output
@@ -84,6 +87,7 @@ void launch_colsum(const RowSpace& rs, View d, half_t* out, long ob0, long ob1, 
 struct LnBwdArgs {
     View in, d1, d2, dlinear, diff, mask, istd, scale;     // inputs (d2, dlinear: extended form)
     View g, d_ln_in, d_drop_in;                            // outputs
+    const uint8_t* mask_bits = nullptr;                    // see launch_bdrln; replaces `mask`
 };
 bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext);
 size_t lnbwd_ws_floats(const RowSpace& rs, bool ext);

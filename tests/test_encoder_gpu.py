@@ -365,7 +365,7 @@ def test_config5_full_size_properties_on_the_device():
     X0 = torch.randn(B, L, E, generator=g).half().cuda()
     DY = torch.randn(B, L, E, generator=g).half().cuda()
     outs = {}
-    for label, options in (('separate', ((1, 0), (3, 0), (4, 0))), ('shipped', ())):
+    for label, options in (('separate', ((1, 0), (3, 0), (4, 0), (9, 0))), ('shipped', ())):      # 9: masks as tensors
         torch.manual_seed(0)
         enc = Encoder('unused', B, L, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, activation='gelu',
                       seed=SEED, persistent_workspace=True).cuda()

@@ -93,8 +93,12 @@ def test_positional_exports_through_the_reference_binding(which):
     layouts_f = dict(lay['forward_interm'])
     drop2 = from_layout(fwd[names.index('DROP2')], 'BJU', layouts_f['DROP2'])
     assert (drop2[masks['DROP2MASK'] == 0] == 0).all()
-    d1 = from_layout(fwd[names.index('DROP1MASK')], 'BJI', layouts_f['DROP1MASK'])
-    assert (d1 == masks['DROP1MASK']).all()
+    # by default the residual dropout masks travel as one bit per element, canonical order, in
+    # the first B*J*I/8 bytes of their buffers (SUB_OPT_PACKED_MASKS)
+    for name in ('DROP1MASK', 'DROP3MASK'):
+        raw = fwd[names.index(name)].contiguous().view(torch.uint8).reshape(-1)[:B * S * E // 8].cpu().numpy()
+        bits = np.unpackbits(raw, bitorder='little').reshape(B, S, E)
+        assert (bits == masks[name]).all(), name
     # ReLU layer (the reference's only activation): the gate the backward pass read, as in the other layer tests
     want = ref.run_named(params_np, X_np, DY_np, masks, 'relu', relu_gate=(drop2 > 0).astype(np.float64))
     for name in ('SB2', 'DX') + tuple('D' + n for n, _ in lay['params']):
