@@ -65,20 +65,23 @@ GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin
             'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
 
 
-def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True):
+def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_unread=True):
     """Per operator: ('hbm', bytes) or ('mfma', flops, bytes).  Bytes = each big
     tensor read once + written once in fp16; flops = 2*batch*M*N*K.
     relu_from_output: the ReLU layer as it runs by default -- bad writes only its
     output (one [B,J,U] tensor in, one out) and bdrlb reads the gate off that output
     (two in, one out); otherwise both move four.
     packed_masks: the two residual dropout masks as one bit per element (the default):
-    1/16 of a [B,J,I] tensor where bdrln writes and the LayerNorm backward reads them."""
+    1/16 of a [B,J,I] tensor where bdrln writes and the LayerNorm backward reads them.
+    skip_unread: the [B,J,I] output that nothing reads afterwards is not written by
+    bdrln (input + bias) and by the one-launch LayerNorm backward (the scaled gradient)."""
     U, P = 4 * E, E // H
     bji, bju, hbjk, q = B * L * E, B * L * U, H * B * L * L, 3 * B * L * E
     mk = bji // 8 if packed_masks else bji * 2           # bytes of one residual dropout mask
+    un = 0 if skip_unread else bji * 2                   # bytes of an output nothing reads
     w = {
         'aib': ('hbm', 2 * q * 2), 'softmax': ('hbm', 4 * hbjk * 2), 'bs': ('hbm', 4 * hbjk * 2),
-        'bdrln1': ('hbm', 6 * bji * 2 + mk), 'bdrln2': ('hbm', 6 * bji * 2 + mk),
+        'bdrln1': ('hbm', 5 * bji * 2 + mk + un), 'bdrln2': ('hbm', 5 * bji * 2 + mk + un),
         'blnrd1': ('hbm', 4 * bji * 2 + mk), 'blnrd2': ('hbm', 4 * bji * 2 + mk),
         'bsb': ('hbm', 3 * bji * 2), 'ebsb': ('hbm', 5 * bji * 2), 'baob': ('hbm', bji * 2),
         'bei': ('hbm', 3 * bji * 2), 'bad': ('hbm', (2 if relu_from_output else 4) * bju * 2),
@@ -89,7 +92,7 @@ def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True):
         'colfinish': ('hbm', 0),
         # single-launch forms: the scaled gradient is written but not read back
         # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
-        'bsb+blnrd1': ('hbm', 6 * bji * 2 + mk), 'ebsb+blnrd2+baob': ('hbm', 8 * bji * 2 + mk),
+        'bsb+blnrd1': ('hbm', 5 * bji * 2 + mk + un), 'ebsb+blnrd2+baob': ('hbm', 7 * bji * 2 + mk + un),
         # scores formed in place: the score tensor itself is neither written nor read
         # (QKT + softmax: Q, K in, three score-sized tensors out; dX1gamma + bs: dO, V
         # and two score-sized tensors in, one out)
@@ -602,7 +605,8 @@ def main():
     enc._handle.profile_enable(False)
     work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
                             relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
-                            packed_masks='9=0' not in args.option and cfg['E'] % 8 == 0)
+                            packed_masks='9=0' not in args.option and cfg['E'] % 8 == 0,
+                            skip_unread='10=0' not in args.option)
     # The events themselves cost time: a step with an event in front of every launch takes longer
     # than the timed steps without them.  That difference, spread evenly over the launches, is taken
     # off every entry, so that the entries add up to the timed step.

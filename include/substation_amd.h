@@ -232,6 +232,14 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * B=8, L=512, E=1024.  Same results.  Set it to 0 before the forward call when the
  * mask tensors are wanted (debug capture); both calls must see the same value. */
 #define SUB_OPT_PACKED_MASKS 9
+/* SUB_OPT_SKIP_UNREAD (default 1): intermediates that neither call reads
+ * afterwards are not written: ATT keeps the product without its bias (the bias
+ * is added in registers, encoder.cu:134-135 writes it back in place), LIN2 is
+ * left alone, and where the LayerNorm backward runs as one launch DLN2 and DLN1
+ * are left alone.  8 MiB less to write in each of four launches at B=8, L=512,
+ * E=1024; outputs and gradients are bit-identical.  Set it to 0 (debug capture
+ * does) when those tensors are wanted. */
+#define SUB_OPT_SKIP_UNREAD 10
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */

@@ -23,6 +23,7 @@ OPT_RELU_FROM_OUTPUT = 6
 OPT_FINISH_IN_PAIR = 7
 OPT_SIDE_JOBS = 8
 OPT_PACKED_MASKS = 9
+OPT_SKIP_UNREAD = 10
 FUSE_REQUIRED = 2
 
 

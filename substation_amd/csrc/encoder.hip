@@ -206,6 +206,7 @@ struct Handle {
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
     bool side_jobs = true;            // CUs that a product's tiles leave idle draw dropout bits for the launch after it
     bool packed_masks = true;         // DROP1MASK / DROP3MASK travel as one bit per element inside their buffers
+    bool skip_unread = true;          // intermediates that neither pass reads are not written (ATT after its bias, LIN2, DLN2, DLN1)
     // where the last forward call's lin1 epilogue left one bit per element of DROP2 (set = positive), or
     // null: the unused SB1_LINW1 buffer of that call.  The backward call reads its gate from there when it
     // is handed the same buffer, and from DROP2 itself otherwise.
@@ -586,7 +587,7 @@ void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, 
               const void* linear_bias, const void* scale, const void* bias, void* lin,
               const Layout& llin, void* mask, const Layout& lmask, void* diff, const Layout& ldiff,
               void* normed, const Layout& lnorm, void* out, const Layout& lout, void* istd,
-              const Layout& listd, float p, uint32_t site, bool packed_mask = false) {
+              const Layout& listd, float p, uint32_t site, bool packed_mask = false, bool write_lin = true) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     int R = sp.rs.R;
     View vi = make_view(in, lin_, sp), vr = make_view(resid, lres, sp), vl = make_view(lin, llin, sp),
@@ -594,7 +595,8 @@ void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, 
          vo = make_view(out, lout, sp), vs = make_view(istd, listd, sp);
     flatten(sp.rs, {&vi, &vr, &vl, &vm, &vd, &vn, &vo, &vs});
     launch_bdrln(sp.rs, vi, vr, vector_view(linear_bias, R), vector_view(scale, R), vector_view(bias, R),
-                 vl, vm, vd, vn, vo, vs, make_key(h, site, p), h.eps, h.stream, packed_mask ? (uint8_t*)mask : nullptr);
+                 vl, vm, vd, vn, vo, vs, make_key(h, site, p), h.eps, h.stream, packed_mask ? (uint8_t*)mask : nullptr,
+                 write_lin);
 }
 
 void op_blnrd(Handle& h, const void* dout, const Layout& ldout, const void* istd, const Layout& listd,
@@ -776,10 +778,11 @@ bool op_lnbwd(Handle& h, bool ext, const void* in, const Layout& lin_, const voi
               const void* istd, const Layout& listd, const void* diff, const Layout& ldiff,
               const void* mask, const Layout& lmask, void* g, const Layout& lg, void* d_ln_in,
               const Layout& lo1, void* d_drop_in, const Layout& lo2, void* dscale, void* dbias,
-              void* dlinear_bias, void* dout_bias, bool packed_mask = false) {
+              void* dlinear_bias, void* dout_bias, bool packed_mask = false, bool write_g = true) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     LnBwdArgs a;
     if (packed_mask) a.mask_bits = (const uint8_t*)mask;
+    a.write_g = write_g;
     a.in = make_view(in, lin_, sp); a.d1 = make_view(d1, l1, sp);
     a.d2 = ext ? make_view(d2, l2, sp) : a.d1;
     a.dlinear = ext ? make_view(dlinear, ldl, sp) : a.d1;
@@ -914,7 +917,7 @@ void forward(Handle& h, const FwdPtrs& t) {
         ProfScope ps(h, "bdrln1");   // adds BO to ATT in place (encoder.cu:134-135)
         op_bdrln(h, F[ATT], h.lf[ATT], t.X, h.lX, W[BO], W[S1], W[B1], F[ATT], h.lf[ATT],
                  F[DROP1MASK], h.lf[DROP1MASK], F[LN1DIFF], h.lf[LN1DIFF], F[LN1], h.lf[LN1],
-                 F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1, packed_masks(h));
+                 F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1, packed_masks(h), !h.skip_unread);
     }
     if (relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok && aligned16(W[LINB1]) && aligned16(F[DROP2]) &&
         aligned16(F[SB1]) && aligned16(W[LINW1])) {
@@ -941,7 +944,7 @@ void forward(Handle& h, const FwdPtrs& t) {
         ProfScope ps(h, "bdrln2");
         op_bdrln(h, F[DROP2_LINW2], h.lf[DROP2_LINW2], F[SB1], h.lf[SB1], W[LINB2], W[S2], W[B2],
                  F[LIN2], h.lf[LIN2], F[DROP3MASK], h.lf[DROP3MASK], F[LN2DIFF], h.lf[LN2DIFF],
-                 F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2, packed_masks(h));
+                 F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2, packed_masks(h), !h.skip_unread);
     }
     prof_mark_end(h);
     if (h.step_dev) {
@@ -975,7 +978,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         fused = op_lnbwd(h, false, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, nullptr, h.lY, nullptr, h.lY,
                          F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF], F[DROP3MASK], h.lf[DROP3MASK],
                          D[DLN2], h.lb[DLN2], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2],
-                         DW[S2], DW[B2], nullptr, nullptr, packed_masks(h));
+                         DW[S2], DW[B2], nullptr, nullptr, packed_masks(h), !h.skip_unread);
         if (!fused) ps.cancel();
     }
     if (!fused) {
@@ -1031,7 +1034,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         fused = op_lnbwd(h, true, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
                          h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], F[LN1STD], h.lf[LN1STD], F[LN1DIFF],
                          h.lf[LN1DIFF], F[DROP1MASK], h.lf[DROP1MASK], D[DLN1], h.lb[DLN1], D[DRESID1],
-                         h.lb[DRESID1], D[DATT], h.lb[DATT], DW[S1], DW[B1], DW[LINB2], DW[BO], packed_masks(h));
+                         h.lb[DRESID1], D[DATT], h.lb[DATT], DW[S1], DW[B1], DW[LINB2], DW[BO], packed_masks(h), !h.skip_unread);
         if (!fused) ps.cancel();
     }
     if (!fused) {
@@ -1319,6 +1322,7 @@ int sub_get_option(void* handle, int option, int* value) {
         else if (option == SUB_OPT_FINISH_IN_PAIR) *value = h.finish_in_pair;
         else if (option == SUB_OPT_SIDE_JOBS) *value = h.side_jobs;
         else if (option == SUB_OPT_PACKED_MASKS) *value = h.packed_masks;
+        else if (option == SUB_OPT_SKIP_UNREAD) *value = h.skip_unread;
         else fail("sub_get_option: unknown option");
     });
 }
@@ -1334,6 +1338,7 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_FINISH_IN_PAIR) h.finish_in_pair = value != 0;
         else if (option == SUB_OPT_SIDE_JOBS) h.side_jobs = value != 0;
         else if (option == SUB_OPT_PACKED_MASKS) h.packed_masks = value != 0;
+        else if (option == SUB_OPT_SKIP_UNREAD) h.skip_unread = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
                 if (EXT) acc[2][c][i] += (float)cur.dl[c][i];
             }
             o = pin(o);
-            if (nv[c]) stg8<true>(a.g.p + og + e0, o);           // nothing reads G again
+            if (nv[c] && a.write_g) stg8<true>(a.g.p + og + e0, o);     // nothing reads G again
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 g[c][i] = (float)o[i];

@@ -165,7 +165,8 @@ template <int VPL, int RPW, bool FAST>
 __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resid, View lin_bias,
                                                  View scale, View bias, View lin, View mask,
                                                  View diff, View normed, View out, View istd,
-                                                 PhiloxKey key_, float eps, unsigned nrows, uint8_t* mask_bits) {
+                                                 PhiloxKey key_, float eps, unsigned nrows, uint8_t* mask_bits,
+                                                 bool write_lin) {
     const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63;
     const unsigned step = gridDim.x * WPB * RPW;
@@ -201,7 +202,7 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                     s[r] += x[r][c][i];
                 }
                 if (nv > 0) {
-                    st8h<FAST, true>(lin, ol, e0, nv, lh);
+                    if (write_lin) st8h<FAST, true>(lin, ol, e0, nv, lh);
                     if (mask_bits) mask_bits[(size_t)(row0 + r) * (rs.R >> 3) + (c * WAVE + lane)] = (uint8_t)bits[r][c];
                     else st8h<FAST, true>(mask, om, e0, nv, mask_h8(bits[r][c]));
                 }
@@ -432,7 +433,7 @@ void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta
 
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st, uint8_t* mask_bits) {
+                  float eps, hipStream_t st, uint8_t* mask_bits, bool write_lin) {
     if (mask_bits && rs.R % 8) fail("bias-dropout-residual-layernorm: a bit mask needs rows of whole 8-packs");
     unsigned nrows = check_rows(rs, "bias-dropout-residual-layernorm");
     if (nrows == 0) return;
@@ -440,7 +441,7 @@ void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View s
     bool fast = in.vec && resid.vec && lin_bias.vec && scale.vec && bias.vec && lin.vec && (mask.vec || mask_bits) &&
                 diff.vec && normed.vec && out.vec;
     SUB_ROW_DISPATCH(k_bdrln, vpl, fast, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
-                     out, istd, key, eps, nrows, mask_bits);
+                     out, istd, key, eps, nrows, mask_bits, write_lin);
     check_launch("bias-dropout-residual-layernorm");
 }
 

@@ -21,12 +21,13 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
                     float scale, float mscale, PhiloxKey key, hipStream_t st);
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st);
+// write_lin = false: `lin` (input + bias, which the backward pass does not read) is not stored.
 // mask_bits (optional; rows of whole 8-packs): the dropout mask as one bit per element in canonical
 // order -- byte row * R / 8 + e / 8, bit e % 8 -- instead of the 0/1 tensor `mask`, which is then
 // neither written (bdrln) nor read (blnrd, the fused LayerNorm backward): 1/16 of the bytes.
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st, uint8_t* mask_bits = nullptr);
+                  float eps, hipStream_t st, uint8_t* mask_bits = nullptr, bool write_lin = true);
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
                   View d_drop_in, hipStream_t st, const uint8_t* mask_bits = nullptr);
 
@@ -88,6 +89,7 @@ struct LnBwdArgs {
     View in, d1, d2, dlinear, diff, mask, istd, scale;     // inputs (d2, dlinear: extended form)
     View g, d_ln_in, d_drop_in;                            // outputs
     const uint8_t* mask_bits = nullptr;                    // see launch_bdrln; replaces `mask`
+    bool write_g = true;                                   // false: g (which nothing reads afterwards) is not stored
 };
 bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext);
 size_t lnbwd_ws_floats(const RowSpace& rs, bool ext);
