@@ -607,6 +607,12 @@ def main():
                             relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
                             packed_masks='9=0' not in args.option and cfg['E'] % 8 == 0,
                             skip_unread='10=0' not in args.option)
+    # Memory-bound launches are priced on the bytes of the reference's operators (each distinct big
+    # tensor read once and written once, masks as fp16 tensors, every named output written); what
+    # this build's launches still have to move after options 9 and 10 is reported beside it.
+    work_ref = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
+                                relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
+                                packed_masks=False, skip_unread=False)
     # The events themselves cost time: a step with an event in front of every launch takes longer
     # than the timed steps without them.  That difference, spread evenly over the launches, is taken
     # off every entry, so that the entries add up to the timed step.
@@ -617,9 +623,10 @@ def main():
         t = max(raw_us[n] - event_us, 0.5) * 1e-6
         kind = work[n]
         if kind[0] == 'hbm':
-            ops.append(dict(op=n, bound='hbm', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e9, 1),
-                            peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(kind[1] / t / HBM_PEAK, 4),
-                            bytes=kind[1]))
+            ref_bytes = work_ref[n][1]
+            ops.append(dict(op=n, bound='hbm', us=round(t * 1e6, 2), achieved=round(ref_bytes / t / 1e9, 1),
+                            peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(ref_bytes / t / HBM_PEAK, 4),
+                            bytes=ref_bytes, moved_bytes=kind[1], moved_gbps=round(kind[1] / t / 1e9, 1)))
         else:
             ops.append(dict(op=n, bound='mfma', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e12, 1),
                             peak=MFMA_PEAK_F16 / 1e12, unit='TFLOP/s', frac=round(kind[1] / t / MFMA_PEAK_F16, 4),
@@ -658,11 +665,14 @@ def main():
         'op_time_us': round(total_us, 1), 'event_us_per_launch': round(event_us, 2),
         'fused_ops': {'us': round(sum(o['us'] for o in fused), 1),
                       'gbps': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / 1e9, 1),
-                      'frac_of_hbm_peak': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4)},
+                      'frac_of_hbm_peak': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4),
+                      'bytes': "the reference operators' tensors, each read once and written once",
+                      'moved_gbps': round(sum(o['moved_bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / 1e9, 1),
+                      'moved_frac_of_hbm_peak': round(sum(o['moved_bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4)},
         'contractions': {'us': round(sum(o['us'] for o in gemms), 1),
                          'tflops': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / 1e12, 1),
                          'frac_of_mfma_peak': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / MFMA_PEAK_F16, 4)},
-        'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac')} for o in ops],
+        'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac', 'moved_gbps') if k in o} for o in ops],
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
