@@ -92,7 +92,9 @@ def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_
         'colfinish': ('hbm', 0),
         # single-launch forms: the scaled gradient is written but not read back
         # (bsb + blnrd1 - one [B,J,I] read; ebsb + blnrd2 + baob - two reads)
-        'bsb+blnrd1': ('hbm', 5 * bji * 2 + mk + un), 'ebsb+blnrd2+baob': ('hbm', 7 * bji * 2 + mk + un),
+        # (moved: the extended launch does not read DLIN2, whose column sum the plain launch took along)
+        'bsb+blnrd1': ('hbm', 5 * bji * 2 + mk + un),
+        'ebsb+blnrd2+baob': ('hbm', (6 if packed_masks or skip_unread else 7) * bji * 2 + mk + un),
         # scores formed in place: the score tensor itself is neither written nor read
         # (QKT + softmax: Q, K in, three score-sized tensors out; dX1gamma + bs: dO, V
         # and two score-sized tensors in, one out)

@@ -773,16 +773,20 @@ void mask_plan(Handle& h, AttnArgs& a, bool forward) {
 // bsb + blnrd (plain) or ebsb + blnrd + baob (extended) in one launch.  Returns
 // false, having done nothing, when the shape or the layouts rule the fused
 // kernel out; the caller then runs the separate operators.
+// How op_lnbwd runs: see LnBwdArgs for the first three; dry = only say whether the launch is possible.
+struct LnBwdMode { bool packed_mask = false, write_g = true, move_sum = false, dry = false; };
+
 bool op_lnbwd(Handle& h, bool ext, const void* in, const Layout& lin_, const void* scale, const void* d1,
               const Layout& l1, const void* d2, const Layout& l2, const void* dlinear, const Layout& ldl,
               const void* istd, const Layout& listd, const void* diff, const Layout& ldiff,
               const void* mask, const Layout& lmask, void* g, const Layout& lg, void* d_ln_in,
               const Layout& lo1, void* d_drop_in, const Layout& lo2, void* dscale, void* dbias,
-              void* dlinear_bias, void* dout_bias, bool packed_mask = false, bool write_g = true) {
+              void* dlinear_bias, void* dout_bias, LnBwdMode mode = {}) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     LnBwdArgs a;
-    if (packed_mask) a.mask_bits = (const uint8_t*)mask;
-    a.write_g = write_g;
+    if (mode.packed_mask) a.mask_bits = (const uint8_t*)mask;
+    a.write_g = mode.write_g;
+    a.move_sum = mode.move_sum;
     a.in = make_view(in, lin_, sp); a.d1 = make_view(d1, l1, sp);
     a.d2 = ext ? make_view(d2, l2, sp) : a.d1;
     a.dlinear = ext ? make_view(dlinear, ldl, sp) : a.d1;
@@ -794,6 +798,7 @@ bool op_lnbwd(Handle& h, bool ext, const void* in, const Layout& lin_, const voi
                     &a.d_drop_in});
     a.scale = vector_view(scale, sp.rs.R);
     if (!lnbwd_supported(sp.rs, a, ext)) return false;
+    if (mode.dry) return true;
     float* ws = take_ws(h, lnbwd_ws_floats(sp.rs, ext));
     half_t* sums[4] = {(half_t*)dscale, (half_t*)dbias, (half_t*)dlinear_bias, (half_t*)dout_bias};
     launch_lnbwd(sp.rs, a, ext, sums, ws, h.stream, defer_of(h));
@@ -973,12 +978,31 @@ void backward(Handle& h, const BwdPtrs& t) {
     struct Reset { Handle& h; ~Reset() { h.deferring = false; } } reset{h};
     void* const* W = t.W; void* const* F = t.F; void* const* D = t.Bk; void* const* DW = t.DW;
     bool fused = false;
+    // the backward passes around the two LayerNorms, each as one launch where possible
+    auto ln2_backward = [&](LnBwdMode m) {
+        return op_lnbwd(h, false, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, nullptr, h.lY, nullptr, h.lY,
+                        F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF], F[DROP3MASK], h.lf[DROP3MASK],
+                        D[DLN2], h.lb[DLN2], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2],
+                        DW[S2], DW[B2], DW[LINB2], nullptr, m);
+    };
+    auto ln1_backward = [&](LnBwdMode m) {
+        return op_lnbwd(h, true, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
+                        h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], F[LN1STD], h.lf[LN1STD], F[LN1DIFF],
+                        h.lf[LN1DIFF], F[DROP1MASK], h.lf[DROP1MASK], D[DLN1], h.lb[DLN1], D[DRESID1],
+                        h.lb[DRESID1], D[DATT], h.lb[DATT], DW[S1], DW[B1], DW[LINB2], DW[BO], m);
+    };
+    LnBwdMode ln_mode;
+    ln_mode.packed_mask = packed_masks(h); ln_mode.write_g = !h.skip_unread;
+    if (h.fuse_ln_backward) {
+        // DLINB2 is the column sum of DLIN2, which the first of the two launches writes and the second
+        // would only read for that sum: when both run, the first one sums it
+        LnBwdMode probe = ln_mode;
+        probe.dry = true;
+        ln_mode.move_sum = ln2_backward(probe) && ln1_backward(probe);
+    }
     if (h.fuse_ln_backward) {
         ProfScope ps(h, "bsb+blnrd1");
-        fused = op_lnbwd(h, false, F[LN2], h.lf[LN2], W[S2], t.DY, h.lY, nullptr, h.lY, nullptr, h.lY,
-                         F[LN2STD], h.lf[LN2STD], F[LN2DIFF], h.lf[LN2DIFF], F[DROP3MASK], h.lf[DROP3MASK],
-                         D[DLN2], h.lb[DLN2], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2],
-                         DW[S2], DW[B2], nullptr, nullptr, packed_masks(h), !h.skip_unread);
+        fused = ln2_backward(ln_mode);
         if (!fused) ps.cancel();
     }
     if (!fused) {
@@ -1031,10 +1055,7 @@ void backward(Handle& h, const BwdPtrs& t) {
     fused = false;
     if (h.fuse_ln_backward) {
         ProfScope ps(h, "ebsb+blnrd2+baob");
-        fused = op_lnbwd(h, true, F[LN1], h.lf[LN1], W[S1], D[DRESID2], h.lb[DRESID2], D[DLIN1_LINW1],
-                         h.lb[DLIN1_LINW1], D[DLIN2], h.lb[DLIN2], F[LN1STD], h.lf[LN1STD], F[LN1DIFF],
-                         h.lf[LN1DIFF], F[DROP1MASK], h.lf[DROP1MASK], D[DLN1], h.lb[DLN1], D[DRESID1],
-                         h.lb[DRESID1], D[DATT], h.lb[DATT], DW[S1], DW[B1], DW[LINB2], DW[BO], packed_masks(h), !h.skip_unread);
+        fused = ln1_backward(ln_mode);
         if (!fused) ps.cancel();
     }
     if (!fused) {

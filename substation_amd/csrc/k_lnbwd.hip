@@ -31,7 +31,7 @@ struct LnRow {
     RowIdx ix;
 };
 
-template <int VPL, bool EXT, bool PACKED>
+template <int VPL, bool EXT, bool PACKED, bool MOVE>
 __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs& a, unsigned row, int lane,
                                             const int (&nv)[VPL], LnRow<VPL>& r) {
     r.ix = row_index(rs, row);
@@ -51,7 +51,7 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
             r.d1[c] = ldg8<EXT>(a.d1.p + o1 + e0);
             if (EXT) {
                 r.d2[c] = ldg8<true>(a.d2.p + o2 + e0);
-                r.dl[c] = ldg8<true>(a.dlinear.p + odl + e0);
+                if (!MOVE) r.dl[c] = ldg8<true>(a.dlinear.p + odl + e0);
             }
             r.df[c] = ldg8<true>(a.diff.p + odf + e0);
             if (PACKED) r.mkb[c] = a.mask_bits[(size_t)row * (rs.R >> 3) + (c * WAVE + lane)];
@@ -62,9 +62,12 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
 
 // VPL: 128-bit packs per lane and row (row length <= VPL * 512).  EXT: the
 // extended form (two incoming gradients, linear-bias and output-bias sums).
-template <int VPL, bool EXT, bool PACKED>
+// MOVE: see LnBwdArgs::move_sum (sums of the plain form: d scale, d bias, column sum of d_drop_in; of
+// the extended form: d scale, d bias, column sum of d_drop_in = d output-bias).
+template <int VPL, bool EXT, bool PACKED, bool MOVE>
 __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, float* ws, unsigned nrows) {
-    constexpr int NS = EXT ? 4 : 2;
+    constexpr int NS = MOVE ? 3 : (EXT ? 4 : 2);
+    constexpr int S_DROP = MOVE ? 2 : 3;          // which sum takes d_drop_in
     __shared__ float red[LN_WPB][VPL * WAVE * 8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float invn = 1.0f / (float)rs.R;
@@ -86,11 +89,11 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
     const unsigned stride = gridDim.x * LN_WPB;
     unsigned row = blockIdx.x * LN_WPB + wave;
     LnRow<VPL> cur, nxt;
-    if (row < nrows) ln_load_row<VPL, EXT, PACKED>(rs, a, row, lane, nv, cur);
+    if (row < nrows) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row, lane, nv, cur);
     for (; row < nrows; row += stride) {
         // the next row's loads are in flight while this one is worked on
         const bool more = row + stride < nrows;
-        if (more) ln_load_row<VPL, EXT, PACKED>(rs, a, row + stride, lane, nv, nxt);
+        if (more) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row + stride, lane, nv, nxt);
         float g[VPL][8], df[VPL][8];
         float s1 = 0.f, s2 = 0.f;
         const long og = view_offset(a.g, cur.ix);
@@ -105,7 +108,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
                 o[i] = (half_t)(d * fsc[c].v[i]);
                 acc[0][c][i] += d * (float)cur.in[c][i];
                 acc[1][c][i] += d;
-                if (EXT) acc[2][c][i] += (float)cur.dl[c][i];
+                if (EXT && !MOVE) acc[2][c][i] += (float)cur.dl[c][i];
             }
             o = pin(o);
             if (nv[c] && a.write_g) stg8<true>(a.g.p + og + e0, o);     // nothing reads G again
@@ -134,7 +137,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
             for (int i = 0; i < 8; ++i) {
                 const bool kept = PACKED ? ((cur.mkb[c] >> i) & 1u) != 0 : cur.mk[c][i] != (half_t)0.0f;
                 y[i] = kept ? x[i] : (half_t)0.0f;
-                if (EXT) acc[3][c][i] += (float)y[i];
+                if (EXT || MOVE) acc[S_DROP][c][i] += (float)y[i];
             }
             stg8<false>(a.d_ln_in.p + oa + e0, x);
             stg8<false>(a.d_drop_in.p + ob + e0, y);
@@ -181,7 +184,7 @@ bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext) {
 }
 
 size_t lnbwd_ws_floats(const RowSpace& rs, bool ext) {
-    return (size_t)(ext ? 4 : 2) * lnbwd_blocks(rs.rows()) * rs.R;
+    return (size_t)(ext ? 4 : 3) * lnbwd_blocks(rs.rows()) * rs.R;      // (3: the plain form with move_sum)
 }
 
 void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* const sums[4], float* ws,
@@ -193,8 +196,14 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     const int vpl = rs.R <= 512 ? 1 : 2;
 #define SUB_LNBWD(VPL_, EXT_)                                                                                     \
     do {                                                                                                          \
-        if (a.mask_bits) hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
-        else hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);            \
+        if (a.mask_bits && a.move_sum)                                                                            \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);  \
+        else if (a.mask_bits)                                                                                     \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+        else if (a.move_sum)                                                                                      \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+        else                                                                                                      \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
     } while (0)
     if (ext) {
         if (vpl == 1) SUB_LNBWD(1, true);
@@ -205,8 +214,9 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     }
 #undef SUB_LNBWD
     check_launch("fused LayerNorm backward");
-    FinishArgs fo{{sums[0], sums[1], sums[2], sums[3]}, 0, 0, 1, 1};
-    FinishJob job{ws, fo, ext ? 4 : 2, 1, blocks, rs.R};
+    // with move_sum both forms have three sums; the extended form's third is the output-bias gradient
+    FinishArgs fo{{sums[0], sums[1], a.move_sum && ext ? sums[3] : sums[2], sums[3]}, 0, 0, 1, 1};
+    FinishJob job{ws, fo, a.move_sum ? 3 : (ext ? 4 : 2), 1, blocks, rs.R};
     if (defer) {
         if (defer->n >= kMaxFinishJobs) fail("fused LayerNorm backward: too many deferred reductions");
         defer->j[defer->n++] = job;

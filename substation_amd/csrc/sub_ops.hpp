@@ -90,6 +90,11 @@ struct LnBwdArgs {
     View g, d_ln_in, d_drop_in;                            // outputs
     const uint8_t* mask_bits = nullptr;                    // see launch_bdrln; replaces `mask`
     bool write_g = true;                                   // false: g (which nothing reads afterwards) is not stored
+    // The column sum of `dlinear` that the extended form owes (the gradient of the second linear
+    // bias) is the column sum of what the plain form writes as d_drop_in one LayerNorm earlier in
+    // the backward pass: with move_sum the plain form adds that third sum (sums[2]) and the extended
+    // form neither reads `dlinear` nor sums it (its sums are then d scale, d bias, d output-bias).
+    bool move_sum = false;
 };
 bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext);
 size_t lnbwd_ws_floats(const RowSpace& rs, bool ext);
