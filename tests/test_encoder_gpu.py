@@ -822,11 +822,15 @@ def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to():
         assert torch.equal(a, b)
 
 
-def test_keep_bits_drawn_beside_the_projections_are_the_same_bits():
-    """At B=8 L=512 E=1024 the stacked projections have 192 tiles for 256 CUs and the
-    launch draws the attention's dropout keep bits for the first key tiles of every
-    score row on the idle ones (option 8); the attention kernel draws the rest.  With
-    the option off it draws them all: outputs and gradients must be bit-identical."""
+@pytest.mark.parametrize('option', [8, 9, 10])
+def test_options_that_only_change_where_bytes_go_give_the_same_bits(option):
+    """Options that must not change a single bit of the output or of any gradient, at
+    B=8 L=512 E=1024, each switched off against the default:
+    8 -- the launch of the stacked projections (192 tiles for 256 CUs) draws the
+         attention's dropout keep bits for the first key tiles of every score row on
+         the idle CUs, the attention kernel the rest (off: it draws them all);
+    9 -- the residual dropout masks travel as one bit per element (off: 0/1 tensors);
+    10 -- intermediates that nothing reads are not written (off: they are)."""
     from substation_amd import Encoder, layouts as L, _lib
     lay = L.mi355x_layouts()
     B, Ls, H, E = 8, 512, 16, 1024
@@ -838,7 +842,7 @@ def test_keep_bits_drawn_beside_the_projections_are_the_same_bits():
             for p in enc.parameters():
                 p.mul_(0.05)
         enc.set_rng(SEED, 3)
-        enc._handle.set_option(_lib.OPT_SIDE_JOBS, int(side_jobs))
+        enc._handle.set_option(option, int(side_jobs))
         g0 = torch.Generator().manual_seed(5)
         X = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
         DY = torch.randn(B, Ls, E, generator=g0).half().cuda()
