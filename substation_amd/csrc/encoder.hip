@@ -587,7 +587,8 @@ void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, 
               const void* linear_bias, const void* scale, const void* bias, void* lin,
               const Layout& llin, void* mask, const Layout& lmask, void* diff, const Layout& ldiff,
               void* normed, const Layout& lnorm, void* out, const Layout& lout, void* istd,
-              const Layout& listd, float p, uint32_t site, bool packed_mask = false, bool write_lin = true) {
+              const Layout& listd, float p, uint32_t site, bool packed_mask = false, bool write_lin = true,
+              KeepWordsJob* side = nullptr) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
     int R = sp.rs.R;
     View vi = make_view(in, lin_, sp), vr = make_view(resid, lres, sp), vl = make_view(lin, llin, sp),
@@ -596,7 +597,7 @@ void op_bdrln(Handle& h, const void* in, const Layout& lin_, const void* resid, 
     flatten(sp.rs, {&vi, &vr, &vl, &vm, &vd, &vn, &vo, &vs});
     launch_bdrln(sp.rs, vi, vr, vector_view(linear_bias, R), vector_view(scale, R), vector_view(bias, R),
                  vl, vm, vd, vn, vo, vs, make_key(h, site, p), h.eps, h.stream, packed_mask ? (uint8_t*)mask : nullptr,
-                 write_lin);
+                 write_lin, side);
 }
 
 void op_blnrd(Handle& h, const void* dout, const Layout& ldout, const void* istd, const Layout& listd,
@@ -918,20 +919,34 @@ void forward(Handle& h, const FwdPtrs& t) {
     }
     if (!fused_attention) run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
     run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
+    const bool lin1_bad = relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok && aligned16(W[LINB1]) &&
+                          aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]);
+    // The keep bits of lin1's ReLU-dropout epilogue depend on nothing but seed, step and position:
+    // workgroups behind those of bdrln1, a launch that waits for memory with its vector units idle,
+    // draw them, into the SB1_LINW1 buffer (unused with that epilogue) behind its B*J*U/8 bytes of gate bits.
+    KeepWordsJob keep_job;
+    if (lin1_bad && h.side_jobs && aligned16(F[SB1_LINW1])) {
+        const GemmPlan& p = h.gemm[G_LIN1_BAD];
+        keep_job.key = make_key(h, SUB_SITE_ACT, h.p_act);
+        keep_job.M = (uint32_t)p.shape.M; keep_job.N = (uint32_t)p.shape.N;
+        if ((size_t)keep_job.M * keep_job.N / 8 % 16 == 0)
+            keep_job.out = (uint32_t*)((char*)F[SB1_LINW1] + (size_t)keep_job.M * keep_job.N / 8);
+    }
     {
         ProfScope ps(h, "bdrln1");   // adds BO to ATT in place (encoder.cu:134-135)
         op_bdrln(h, F[ATT], h.lf[ATT], t.X, h.lX, W[BO], W[S1], W[B1], F[ATT], h.lf[ATT],
                  F[DROP1MASK], h.lf[DROP1MASK], F[LN1DIFF], h.lf[LN1DIFF], F[LN1], h.lf[LN1],
-                 F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1, packed_masks(h), !h.skip_unread);
+                 F[SB1], h.lf[SB1], F[LN1STD], h.lf[LN1STD], h.p_resid1, SUB_SITE_RESID1, packed_masks(h), !h.skip_unread,
+                 &keep_job);
     }
-    if (relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok && aligned16(W[LINB1]) && aligned16(F[DROP2]) &&
-        aligned16(F[SB1]) && aligned16(W[LINW1])) {
+    if (lin1_bad) {
         // product, bias, ReLU and dropout in one launch: SB1_LINW1 (and LIN1, DROP2MASK) are not produced
         ProfScope ps(h, "lin1+bad");
         const GemmPlan& p = h.gemm[G_LIN1_BAD];
         GemmEpilogue ep;
         ep.bias = (const half_t*)W[LINB1]; ep.sbM = p.sM; ep.sbN = p.sN;
         ep.relu_dropout = true; ep.key = make_key(h, SUB_SITE_ACT, h.p_act);
+        if (keep_job.blocks) ep.keep_words = keep_job.out;
         if (F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0) ep.gate_bits_out = (uint32_t*)F[SB1_LINW1];
         h.gate_bits_at = ep.gate_bits_out;
         launch_gemm(p.shape, (const half_t*)F[SB1], (const half_t*)W[LINW1], (half_t*)F[DROP2], p.alpha, ep, h.stream);

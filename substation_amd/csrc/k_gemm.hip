@@ -41,6 +41,7 @@ struct GemmArgs {
     PhiloxKey key;
     const half_t* gate = nullptr; // or: zero where gate <= 0 (strides of `bias`), column sums per 128-row slab
     float* colsum = nullptr;
+    const uint32_t* keep_words = nullptr;  // relu_dropout: the keep bits, drawn ahead (relu_dropout_keep_words)
     uint32_t* gate_bits_out = nullptr;     // relu_dropout: one bit per output, set where it is positive
     const uint32_t* gate_bits = nullptr;   // gate: those bits instead of the values of `gate`
     // GemmSideJob of the eight-wave asynchronous kernel: workgroups side_first .. gridDim.x - 1 draw
@@ -425,8 +426,9 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id,
                 if (biasb) {
                     // the addend (a bias row or a whole tensor) is N-contiguous like C
                     h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
+                    // the sum of two halves is exact in fp32: the packed half add rounds as the
+                    // conversion of that sum would
+                    val = val + ad;
                 }
                 *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
             }
@@ -641,7 +643,8 @@ __device__ __forceinline__ void sched_half_step() {
 // while one wave of a SIMD sits in the issue of its loads the other multiplies.
 // EPI: what the epilogue does after the scaling and the optional addend.  A template
 // parameter so that the plain kernel does not carry the registers of the others.
-enum { EPI_PLAIN = 0, EPI_RELU_DROPOUT = 1, EPI_GATE_COLSUM = 2 };
+// EPI_RELU_DROPOUT_PRE: EPI_RELU_DROPOUT with the keep bits drawn ahead of the launch (GemmEpilogue::keep_words)
+enum { EPI_PLAIN = 0, EPI_RELU_DROPOUT = 1, EPI_GATE_COLSUM = 2, EPI_RELU_DROPOUT_PRE = 3 };
 
 template <int TM, int TN, bool AKC, bool BKC, int S, int NW, int EPI = EPI_PLAIN>
 __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
@@ -866,8 +869,13 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     // One bit per output of the ReLU-dropout epilogue (set = positive), a dword per lane and 32-row
     // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
     // output shape reads 1/16 of what the outputs themselves would cost it.
+    constexpr bool RELU_DROP = EPI == EPI_RELU_DROPOUT || EPI == EPI_RELU_DROPOUT_PRE;
     static_assert(EPI == EPI_PLAIN || 32 / RPI == 4, "four packs of 8 outputs per lane and slab");
     const long bits_at = (((long)tile_m * tiles_n + tile_n) * NW + wave) * (TM * 64) + lane;
+    if (EPI == EPI_RELU_DROPOUT_PRE) {
+        const uint4 w = reinterpret_cast<const uint4*>(g.keep_words)[(((long)tile_m * tiles_n + tile_n) * NW + wave) * 64 + lane];
+        kb[0] = w.x; kb[1] = w.y; kb[2] = w.z; kb[3] = w.w;
+    }
     uint32_t gbits[TM];
     if (EPI == EPI_GATE_COLSUM && g.gate_bits) {
 #pragma unroll
@@ -894,8 +902,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             int mm = mrow + rr2, nn = n0 + wn * 32 * TN + c8;
             if (biasb) {
                 h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) val[e] = (half_t)((float)val[e] + (float)ad[e]);
+                val = val + ad;          // packed half add: the same single rounding as through fp32
             }
             if (EPI == EPI_GATE_COLSUM) {
                 // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
@@ -915,21 +922,22 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                     }
                 }
             }
-            if (EPI == EPI_RELU_DROPOUT) {
+            if (RELU_DROP) {
                 // what the bias-activation-dropout operator does to the rounded sum, with the
                 // same keep bits (the element index is the offset into the dense output):
                 // pack c sits in byte 15 - c of the bits drawn in the main loop
                 const int c = i * (32 / RPI) + it, byte = 15 - c;
                 const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
+                val = __builtin_elementwise_max(val, (h8)(half_t)0.0f);       // ReLU, packed
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
-                    val[e] = ((bits >> e) & 1u) ? (half_t)fmaxf((float)val[e], 0.f) : (half_t)0.0f;
-                    positive |= ((float)val[e] > 0.f ? 1u : 0u) << (8 * it + e);
+                    val[e] = ((bits >> e) & 1u) ? val[e] : (half_t)0.0f;
+                    positive |= (val[e] > (half_t)0.0f ? 1u : 0u) << (8 * it + e);
                 }
             }
             *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
         }
-        if (EPI == EPI_RELU_DROPOUT && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
+        if (RELU_DROP && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
     }
     if (EPI == EPI_GATE_COLSUM) {
         // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
@@ -1015,6 +1023,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     a.alpha = alpha; a.bias = ep.bias;
     a.relu_dropout = ep.relu_dropout ? 1 : 0; a.key = ep.key;
     a.gate = ep.gate; a.colsum = ep.colsum; a.gate_bits_out = ep.gate_bits_out; a.gate_bits = ep.gate_bits;
+    a.keep_words = ep.keep_words;
     a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;
@@ -1082,6 +1091,7 @@ void launch_dma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t s
         // only the eight-wave 256x256 kernel carries these epilogues
         if constexpr (NW == 8) {
             if (a.gate) launch_dma3<TM, TN, S, NW, EPI_GATE_COLSUM>(a, akc, bkc, grid, st);
+            else if (a.keep_words) launch_dma3<TM, TN, S, NW, EPI_RELU_DROPOUT_PRE>(a, akc, bkc, grid, st);
             else launch_dma3<TM, TN, S, NW, EPI_RELU_DROPOUT>(a, akc, bkc, grid, st);
             return;
         } else {

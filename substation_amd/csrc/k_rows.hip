@@ -166,10 +166,23 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                                                  View scale, View bias, View lin, View mask,
                                                  View diff, View normed, View out, View istd,
                                                  PhiloxKey key_, float eps, unsigned nrows, uint8_t* mask_bits,
-                                                 bool write_lin) {
+                                                 bool write_lin, KeepWordsJob side) {
+    // side.blocks workgroups behind those of the rows only draw keep words: the rows wait for memory
+    // with the vector units idle
+    const unsigned row_blocks = gridDim.x - side.blocks;
+    if (blockIdx.x >= row_blocks) {
+        const PhiloxKey skey = resolved(side.key);
+        const uint32_t tiles_n = side.N / 256, items = (side.M / 256) * tiles_n * 512;
+        for (uint32_t id = (blockIdx.x - row_blocks) * BLOCK + threadIdx.x; id < items; id += side.blocks * BLOCK) {
+            const uint32_t tile = id >> 9, tm = tile / tiles_n;
+            const KeepWords k = relu_dropout_keep_words(skey, side.N, tm, tile - tm * tiles_n, (id >> 6) & 7, id & 63);
+            reinterpret_cast<uint4*>(side.out)[id] = make_uint4(k.w[0], k.w[1], k.w[2], k.w[3]);
+        }
+        return;
+    }
     const PhiloxKey key = resolved(key_);
     const int lane = threadIdx.x & 63;
-    const unsigned step = gridDim.x * WPB * RPW;
+    const unsigned step = row_blocks * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;
     for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
         float x[RPW][VPL][8];
@@ -349,8 +362,10 @@ inline unsigned check_rows(const RowSpace& rs, const char* what) {
 
 // Dispatch on (VPL, rows per wave, FAST).  Rows per wave: 4 for rows of up to 512
 // elements, 2 up to 1024, else 1; the generic (strided) path always takes 1.
+// (extra_blocks: workgroups behind those of the rows, for a kernel that has a side job; a
+// variable of the calling function.)
 #define SUB_ROW_LAUNCH(KERNEL, V, RP, F, ...) \
-    hipLaunchKernelGGL((KERNEL<V, RP, F>), dim3(row_grid(nrows, RP)), dim3(BLOCK), 0, st, __VA_ARGS__)
+    hipLaunchKernelGGL((KERNEL<V, RP, F>), dim3(row_grid(nrows, RP) + extra_blocks), dim3(BLOCK), 0, st, __VA_ARGS__)
 #define SUB_ROW_DISPATCH(KERNEL, vpl, fast, ...)                                   \
     do {                                                                           \
         if (fast) {                                                                \
@@ -376,6 +391,7 @@ inline unsigned check_rows(const RowSpace& rs, const char* what) {
 
 void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View drop, View amask,
                     float scale, float mscale, PhiloxKey key, hipStream_t st) {
+    const unsigned extra_blocks = 0;
     unsigned nrows = check_rows(rs, "softmax");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax");
@@ -413,6 +429,7 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
 
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st) {
+    const unsigned extra_blocks = 0;
     unsigned nrows = check_rows(rs, "softmax backward");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "softmax backward");
@@ -433,20 +450,33 @@ void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta
 
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st, uint8_t* mask_bits, bool write_lin) {
+                  float eps, hipStream_t st, uint8_t* mask_bits, bool write_lin, KeepWordsJob* side) {
     if (mask_bits && rs.R % 8) fail("bias-dropout-residual-layernorm: a bit mask needs rows of whole 8-packs");
     unsigned nrows = check_rows(rs, "bias-dropout-residual-layernorm");
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "bias-dropout-residual-layernorm");
     bool fast = in.vec && resid.vec && lin_bias.vec && scale.vec && bias.vec && lin.vec && (mask.vec || mask_bits) &&
                 diff.vec && normed.vec && out.vec;
+    // the side job: as many workgroups as draw one lane's words per thread, at most four per CU
+    KeepWordsJob job;
+    if (side && side->out && side->key.thr && side->M % 256 == 0 && side->N % 256 == 0 && side->M > 0 && side->N > 0 &&
+        (uint64_t)side->M * side->N / 8 / 16 <= 0x7fffffffu) {
+        job = *side;
+        const uint64_t items = (uint64_t)side->M / 256 * (side->N / 256) * 512;
+        job.blocks = (uint32_t)((items + BLOCK - 1) / BLOCK < 1024 ? (items + BLOCK - 1) / BLOCK : 1024);
+        side->blocks = job.blocks;
+    } else if (side) {
+        side->blocks = 0;
+    }
+    const unsigned extra_blocks = job.blocks;
     SUB_ROW_DISPATCH(k_bdrln, vpl, fast, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
-                     out, istd, key, eps, nrows, mask_bits, write_lin);
+                     out, istd, key, eps, nrows, mask_bits, write_lin, job);
     check_launch("bias-dropout-residual-layernorm");
 }
 
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
                   View d_drop_in, hipStream_t st, const uint8_t* mask_bits) {
+    const unsigned extra_blocks = 0;
     if (mask_bits && rs.R % 8) fail("layernorm backward: a bit mask needs rows of whole 8-packs");
     unsigned nrows = check_rows(rs, "layernorm backward");
     if (nrows == 0) return;

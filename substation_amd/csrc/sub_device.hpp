@@ -200,6 +200,30 @@ __device__ __forceinline__ uint32_t attention_keep_word(const PhiloxKey& key, ui
            (keep8(philox_group_dev(key, g0 + 2), key.thr) << 16) | (keep8(philox_group_dev(key, g0 + 3), key.thr) << 24);
 }
 
+// The ReLU-dropout epilogue of the eight-wave 256x256 contraction kernel walks its tile so that lane
+// `lane` of wave `wave` (of 8: 2 rows x 4 columns of waves) stores 16 packs of 8 outputs, pack c at
+//   row = 256 tile_m + 128 (wave / 4) + 8 c + lane / 8,   column = 256 tile_n + 64 (wave % 4) + 8 (lane % 8)
+// of the dense [M][N] output.  Its keep bits are 128 bits per lane, pack c in byte 15 - c: four words,
+// word j = bytes of packs 15 - 4 j (lowest byte) .. 12 - 4 j.  This draws them for one lane.
+struct KeepWords { uint32_t w[4]; };
+__device__ __forceinline__ KeepWords relu_dropout_keep_words(const PhiloxKey& key, uint32_t N, uint32_t tile_m,
+                                                             uint32_t tile_n, uint32_t wave, uint32_t lane) {
+    const uint64_t row0 = (uint64_t)tile_m * 256 + (wave >> 2) * 128 + (lane >> 3);
+    const uint64_t g0 = (row0 * N + (uint64_t)tile_n * 256 + (wave & 3) * 64 + (lane & 7) * 8) >> 3;
+    KeepWords k;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int c = 15 - 4 * j - b;
+            w |= keep8(philox_group_dev(key, g0 + (uint64_t)c * N), key.thr) << (8 * b);
+        }
+        k.w[j] = w;
+    }
+    return k;
+}
+
 // d(LN input) of one element: g * istd - c1 - diff * c2, with the contraction
 // into FMAs spelled out so that every kernel that evaluates it rounds alike.
 __device__ __forceinline__ float ln_bwd_value(float g, float diff, float istd, float c1, float c2) {

@@ -21,13 +21,24 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
                     float scale, float mscale, PhiloxKey key, hipStream_t st);
 void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta, float scale,
                hipStream_t st);
+// Side job of launch_bdrln (a launch that waits for memory with its vector units idle): `blocks`
+// workgroups behind those of the rows draw the keep words of the ReLU-dropout epilogue
+// (relu_dropout_keep_words) of a later product with a dense [M][N] output in 256x256 tiles, word
+// quadruple ((tile_m * N/256 + tile_n) * 8 + wave) * 64 + lane of `out` (M * N / 8 bytes).
+struct KeepWordsJob {
+    PhiloxKey key;
+    uint32_t* out = nullptr;
+    uint32_t M = 0, N = 0;
+    uint32_t blocks = 0;         // set by launch_bdrln; 0 = not taken
+};
 // write_lin = false: `lin` (input + bias, which the backward pass does not read) is not stored.
 // mask_bits (optional; rows of whole 8-packs): the dropout mask as one bit per element in canonical
 // order -- byte row * R / 8 + e / 8, bit e % 8 -- instead of the 0/1 tensor `mask`, which is then
 // neither written (bdrln) nor read (blnrd, the fused LayerNorm backward): 1/16 of the bytes.
 void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View scale, View bias,
                   View lin, View mask, View diff, View normed, View out, View istd, PhiloxKey key,
-                  float eps, hipStream_t st, uint8_t* mask_bits = nullptr, bool write_lin = true);
+                  float eps, hipStream_t st, uint8_t* mask_bits = nullptr, bool write_lin = true,
+                  KeepWordsJob* side = nullptr);
 void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask, View d_ln_in,
                   View d_drop_in, hipStream_t st, const uint8_t* mask_bits = nullptr);
 
@@ -191,6 +202,9 @@ struct GemmEpilogue {
     // the values of `gate` (which must still be given)
     uint32_t* gate_bits_out = nullptr;
     const uint32_t* gate_bits = nullptr;
+    // relu_dropout: the keep bits drawn ahead by a KeepWordsJob with the same key, M and N; without
+    // them the kernel draws them itself during the contraction
+    const uint32_t* keep_words = nullptr;
 };
 // Work that needs no memory path, offered to a product whose 256x256 tiles leave CUs idle: the
 // keep bits of the attention dropout (attention_keep_word) for the first `tiles_done` key tiles of
