@@ -866,6 +866,11 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
     half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
     const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
+    // a bias row (the same for every row of the output): a lane's 8 columns are the same in all of its
+    // packs, so it loads them once instead of before every store
+    const bool bias_row = biasb && g.sbM == 0;
+    h8 bias8 = (h8)(half_t)0.0f;
+    if (bias_row) bias8 = *reinterpret_cast<const h8*>(biasb + n0 + wn * 32 * TN + (lane % LPR) * 8);
     // One bit per output of the ReLU-dropout epilogue (set = positive), a dword per lane and 32-row
     // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
     // output shape reads 1/16 of what the outputs themselves would cost it.
@@ -901,7 +906,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
             h8 val = *reinterpret_cast<const h8*>(stage + rr2 * STAGE_PITCH + c8);
             int mm = mrow + rr2, nn = n0 + wn * 32 * TN + c8;
             if (biasb) {
-                h8 ad = *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
+                const h8 ad = bias_row ? bias8 : *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
                 val = val + ad;          // packed half add: the same single rounding as through fp32
             }
             if (EPI == EPI_GATE_COLSUM) {
