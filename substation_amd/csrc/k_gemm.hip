@@ -751,8 +751,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 #define SUB_DMA_KEEP()                                                                            \
     do {                                                                                          \
         const U4 r_ = philox_group(rd_key, kb_group0 + (uint64_t)(kb_next & 15) * (uint64_t)g.sCM); \
-        uint32_t b_ = 0;                                                                          \
-        _Pragma("unroll") for (int e = 0; e < 8; ++e) b_ |= (field16(r_, e) >= rd_key.thr ? 1u : 0u) << e; \
+        const uint32_t b_ = keep8(r_, rd_key.thr);                                                \
         kb[3] = (kb[3] << 8) | (kb[2] >> 24);                                                     \
         kb[2] = (kb[2] << 8) | (kb[1] >> 24);                                                     \
         kb[1] = (kb[1] << 8) | (kb[0] >> 24);                                                     \
@@ -1345,12 +1344,12 @@ void launch_gemm(const GemmShape& s, const half_t* A, const half_t* B, half_t* C
         if (side) side->tiles_done = 0;
         if (side && side->keep && side->key.thr && tile == 44 && !ep.relu_dropout && !ep.gate && c.a.splits == 1) {
             // CUs the tiles leave idle draw attention keep bits meanwhile: what fits into the time the
-            // product takes (about 9 us + 1.5 us per k-tile; a CU draws 1450 Philox groups per us, measured:
-            // with all 16 key tiles of the bench workload the launch takes 45 instead of 34 us)
+            // product takes (about 9 us + 1.5 us per k-tile; the rate per CU and us is the measured break-even:
+            // 12 of the 16 key tiles of the bench workload cost the launch 0.3 us, 14 cost it 2.5, all 16 6 us)
             const long tiles = (long)(c.a.M / 256) * (c.a.N / 256) * batch;
             const long idle = 256 - tiles, nkt = (long)c.a.K0 * (c.a.K1 / BK);
             if (tiles >= 128 && idle >= 32 && side->nk % 32 == 0) {
-                                const double groups = (double)idle * (9.0 + 1.5 * (double)nkt) * 1300.0;   // a tenth of margin
+                const double groups = (double)idle * (9.0 + 1.5 * (double)nkt) * 1600.0;
                 long td = (long)(groups / (4.0 * (double)side->rows));
                 if (td > side->nk / 32) td = side->nk / 32;
                 if (td > 0) {

@@ -341,6 +341,10 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
     int cur = 0, nxt = 1, nn = 2;
     MaskRegs mk = {};
     if (MASKED && n > 0 && entry_class(e0, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e0) * 32, hi, mk);
+    // keep words drawn ahead of this launch are fetched a tile early: at the place of their
+    // use the load would stand between the scores and their exponentials
+    uint32_t word_ahead = 0;
+    if (key.thr && n > 0 && entry_tile(e0) < a.keep_tiles_ready) word_ahead = a.keep[(size_t)row * nt + entry_tile(e0)];
     wait_loads();
 
     for (unsigned i = 0; i < n; ++i) {
@@ -348,6 +352,9 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         const unsigned t = entry_tile(e0);
         const bool from_mask = MASKED && entry_class(e0, wave) != BLOCK_CLEAR;
         const bool fetch = i + 2 < n;
+        const uint32_t word_ready = word_ahead;
+        if (key.thr && i + 1 < n && entry_tile(e1) < a.keep_tiles_ready)
+            word_ahead = a.keep[(size_t)row * nt + entry_tile(e1)];
         if (fetch) {
             tile_fetch<P>(a.k, h, b, entry_tile(e2) * 32, tid, kr);
             tile_fetch<P>(a.v, h, b, entry_tile(e2) * 32, tid, vr);
@@ -371,7 +378,7 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
         // wave draws two of the four groups of 8 and the halves trade them
         uint32_t word = 0xffffffffu;
         if (key.thr && t < a.keep_tiles_ready) {
-            word = a.keep[(size_t)row * nt + t];                     // drawn ahead of this launch
+            word = word_ready;                                       // drawn ahead of this launch
         } else if (key.thr) {
             const uint64_t g0 = (uint64_t)row * (a.K / 8) + 4 * t + 2 * hi;
             const uint32_t mine = keep8(philox_group_dev(key, g0), key.thr) |

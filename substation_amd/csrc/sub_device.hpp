@@ -184,14 +184,6 @@ __device__ __forceinline__ U4 philox_group_dev(const PhiloxKey& k, uint64_t g) {
     return c;
 }
 
-// Keep bits of the 8 elements of one Philox group: bit i set = 16-bit field i >= thr.
-__device__ __forceinline__ uint32_t keep8(const U4& r, uint32_t thr) {
-    uint32_t b = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) b |= (field16(r, i) >= thr ? 1u : 0u) << i;
-    return b;
-}
-
 // The 32 keep bits of key tile t of score row `row` in the attention kernels' format (bit k =
 // key 32 t + k of a row of nk keys): four Philox groups.
 __device__ __forceinline__ uint32_t attention_keep_word(const PhiloxKey& key, uint64_t row, uint32_t nk, uint32_t t) {

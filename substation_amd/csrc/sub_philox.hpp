@@ -67,6 +67,32 @@ SUB_HD uint32_t field16(const U4& r, int i) {
     return (i & 1) ? (w >> 16) : (w & 0xFFFFu);
 }
 
+// Keep bits of the 8 elements of one Philox group: bit i set = 16-bit field i >= thr.
+// On the device both fields of a word are compared at once: thr - field, saturating at 0,
+// is non-zero exactly where the element is dropped (v_pk_sub_u16 clamp, v_pk_min_u16
+// against 1: the word's two drop bits at positions 0 and 16); the four words are shifted
+// together and the upper fields' bits folded down beside the lower ones'.  About 15
+// instructions where a compare and a select per field take 30.
+SUB_HD uint32_t keep8(const U4& r, uint32_t thr) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    // (spelled as instructions: written as min(sub_sat(thr, field), 1) the compiler turns the
+    // pair back into a compare and a select per field)
+    const uint32_t thr2 = (thr & 0xffffu) * 0x10001u, one2 = 0x10001u;
+    auto drop2 = [&](uint32_t w) {
+        uint32_t d;
+        asm("v_pk_sub_u16 %0, %1, %2 clamp\n\tv_pk_min_u16 %0, %0, %3" : "=&v"(d) : "v"(thr2), "v"(w), "v"(one2));
+        return d;
+    };
+    const uint32_t d = drop2(r.x) | (drop2(r.y) << 2) | (drop2(r.z) << 4) | (drop2(r.w) << 6);
+    const uint32_t all = 0u - (thr >> 16);                         // thr = 2^16: every element dropped
+    return ~(d | (d >> 15) | all) & 0xffu;
+#else
+    uint32_t b = 0;
+    for (int i = 0; i < 8; ++i) b |= (field16(r, i) >= thr ? 1u : 0u) << i;
+    return b;
+#endif
+}
+
 // Keep-bits (bit i set = element e0+i kept) for 8 consecutive canonical elements
 // starting at e0.  One Philox call when e0 is a multiple of 8, two otherwise.
 SUB_HD uint32_t keep_bits8(const PhiloxKey& k, uint64_t e0) {
@@ -75,8 +101,7 @@ SUB_HD uint32_t keep_bits8(const PhiloxKey& k, uint64_t e0) {
     U4 r0 = philox_group(k, g);
     uint32_t bits = 0;
     if (off == 0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) bits |= (field16(r0, i) >= k.thr ? 1u : 0u) << i;
+        bits = keep8(r0, k.thr);
     } else {
         U4 r1 = philox_group(k, g + 1);
         for (int i = 0; i < 8; ++i) {
