@@ -216,16 +216,17 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * `dXQKV-fused+dWQKV-fused+dWout`.  Needs SUB_OPT_PAIR_PRODUCTS and the
  * in-register attention (whose kernels produce the DBKQV partials). */
 #define SUB_OPT_FINISH_IN_PAIR 7
-/* SUB_OPT_SIDE_JOBS (default 1): where the 256x256 tiles of the stacked
- * projections leave CUs idle (192 tiles on 256 CUs at B=8, L=512, E=1024),
- * workgroups behind the tiles of that launch draw the dropout keep bits of the
- * first key tiles of every score row for the attention launch that follows
+/* SUB_OPT_SIDE_JOBS (bit mask, default 1).  Bit 0: where the 256x256 tiles of
+ * the stacked projections leave CUs idle (192 tiles on 256 CUs at B=8, L=512,
+ * E=1024), workgroups behind the tiles of that launch draw the dropout keep bits
+ * of the first key tiles of every score row for the attention launch that follows
  * (they depend on nothing but seed, step and position); the attention kernel
- * draws the rest.  Likewise workgroups behind the rows of the first
- * bias-dropout-residual-LayerNorm launch, which waits for memory with its vector
- * units idle, draw the keep bits of lin1's ReLU-dropout epilogue (into the
- * SB1_LINW1 buffer, behind its gate bits).  Same bits, same results.  Needs the
- * in-register attention resp. the `lin1+bad` launch (SUB_OPT_FUSE_EPILOGUES). */
+ * draws the rest.  Bit 1 (off by default: since that launch stopped being bound
+ * by its own vector work the drawing costs it more than it saves the next one):
+ * workgroups behind the rows of the first bias-dropout-residual-LayerNorm launch
+ * draw the keep bits of lin1's ReLU-dropout epilogue (into the SB1_LINW1 buffer,
+ * behind its gate bits).  Same bits, same results.  Needs the in-register
+ * attention resp. the `lin1+bad` launch (SUB_OPT_FUSE_EPILOGUES). */
 #define SUB_OPT_SIDE_JOBS 8
 /* SUB_OPT_PACKED_MASKS (default 1; embedding size a multiple of 8): the masks of
  * the two residual dropouts travel from encoder_forward to encoder_backward as one

@@ -204,7 +204,8 @@ struct Handle {
     bool pair_products = true;        // a data gradient and the weight gradient next to it in one launch
     bool finish_in_pair = true;       // deferred column sums are finished inside the last pair launch of the backward pass
     bool relu_from_output = true;     // ReLU: the backward gate is read off DROP2; LIN1 and DROP2MASK are not produced
-    bool side_jobs = true;            // CUs that a product's tiles leave idle draw dropout bits for the launch after it
+    int side_jobs = 1;                // bit 0: CUs that the stacked projections' tiles leave idle draw attention keep bits;
+                                      // bit 1: workgroups behind the first LayerNorm launch draw lin1's keep bits
     bool packed_masks = true;         // DROP1MASK / DROP3MASK travel as one bit per element inside their buffers
     bool skip_unread = true;          // intermediates that neither pass reads are not written (ATT after its bias, LIN2, DLN2, DLN1)
     // where the last forward call's lin1 epilogue left one bit per element of DROP2 (set = positive), or
@@ -886,7 +887,7 @@ void forward(Handle& h, const FwdPtrs& t) {
         // projection + bias in one pass; WKKWQQWVV (the pre-bias copy) is not written.  The CUs its tiles
         // leave idle draw part of the attention's dropout bits, which depend on nothing but the seed.
         GemmSideJob side;
-        if (fused_attention && h.side_jobs) {
+        if (fused_attention && (h.side_jobs & 1)) {
             side.key = make_key(h, SUB_SITE_SOFTMAX, h.p_softmax);
             side.keep = at.keep; side.rows = (uint32_t)((long)at.H * at.B * at.J); side.nk = (uint32_t)at.K;
         }
@@ -925,7 +926,7 @@ void forward(Handle& h, const FwdPtrs& t) {
     // workgroups behind those of bdrln1, a launch that waits for memory with its vector units idle,
     // draw them, into the SB1_LINW1 buffer (unused with that epilogue) behind its B*J*U/8 bytes of gate bits.
     KeepWordsJob keep_job;
-    if (lin1_bad && h.side_jobs && aligned16(F[SB1_LINW1])) {
+    if (lin1_bad && (h.side_jobs & 2) && aligned16(F[SB1_LINW1])) {
         const GemmPlan& p = h.gemm[G_LIN1_BAD];
         keep_job.key = make_key(h, SUB_SITE_ACT, h.p_act);
         keep_job.M = (uint32_t)p.shape.M; keep_job.N = (uint32_t)p.shape.N;
@@ -1372,7 +1373,7 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_PAIR_PRODUCTS) h.pair_products = value != 0;
         else if (option == SUB_OPT_RELU_FROM_OUTPUT) h.relu_from_output = value != 0;
         else if (option == SUB_OPT_FINISH_IN_PAIR) h.finish_in_pair = value != 0;
-        else if (option == SUB_OPT_SIDE_JOBS) h.side_jobs = value != 0;
+        else if (option == SUB_OPT_SIDE_JOBS) h.side_jobs = value & 3;
         else if (option == SUB_OPT_PACKED_MASKS) h.packed_masks = value != 0;
         else if (option == SUB_OPT_SKIP_UNREAD) h.skip_unread = value != 0;
         else if (option == SUB_OPT_FUSE_ATTENTION) {

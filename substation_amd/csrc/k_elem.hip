@@ -54,7 +54,7 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             if (c[u].nv == 0) continue;
-            uint32_t bits = keep_bits8(key, (uint64_t)c[u].row * (uint64_t)rs.R + (uint64_t)c[u].e0);
+            uint32_t bits = keep_pack<FAST>(key, (uint64_t)c[u].row * (uint64_t)rs.R + (uint64_t)c[u].e0);
             h8 lh, oh;
 #pragma unroll
             for (int i = 0; i < 8; ++i) lh[i] = (half_t)(fi[u].v[i] + fb[u].v[i]);

@@ -31,14 +31,22 @@ struct LnRow {
     RowIdx ix;
 };
 
-template <int VPL, bool EXT, bool PACKED, bool MOVE>
+// Where row `ix` of view `v` starts.  FLAT: the row space is flat (RowSpace::flat, what the encoder
+// layer's layouts give), the row is its only index: one multiplication in place of four.
+template <bool FLAT>
+__device__ __forceinline__ long ln_row_offset(const View& v, const RowIdx& ix) {
+    return FLAT ? (long)ix.i3 * v.s3 : view_offset(v, ix);
+}
+
+template <int VPL, bool EXT, bool PACKED, bool MOVE, bool FLAT>
 __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs& a, unsigned row, int lane,
                                             const int (&nv)[VPL], LnRow<VPL>& r) {
-    r.ix = row_index(rs, row);
-    const long oin = view_offset(a.in, r.ix), o1 = view_offset(a.d1, r.ix), odf = view_offset(a.diff, r.ix),
-               omk = view_offset(a.mask, r.ix);
-    const long o2 = EXT ? view_offset(a.d2, r.ix) : 0, odl = EXT ? view_offset(a.dlinear, r.ix) : 0;
-    r.is = (float)a.istd.p[view_offset(a.istd, r.ix)];
+    if (FLAT) { r.ix.i0 = r.ix.i1 = r.ix.i2 = 0; r.ix.i3 = row; }
+    else r.ix = row_index(rs, row);
+    const long oin = ln_row_offset<FLAT>(a.in, r.ix), o1 = ln_row_offset<FLAT>(a.d1, r.ix),
+               odf = ln_row_offset<FLAT>(a.diff, r.ix), omk = ln_row_offset<FLAT>(a.mask, r.ix);
+    const long o2 = EXT ? ln_row_offset<FLAT>(a.d2, r.ix) : 0, odl = EXT ? ln_row_offset<FLAT>(a.dlinear, r.ix) : 0;
+    r.is = (float)a.istd.p[ln_row_offset<FLAT>(a.istd, r.ix)];
 #pragma unroll
     for (int c = 0; c < VPL; ++c) {
         const int e0 = (c * WAVE + lane) * 8;
@@ -64,7 +72,7 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
 // extended form (two incoming gradients, linear-bias and output-bias sums).
 // MOVE: see LnBwdArgs::move_sum (sums of the plain form: d scale, d bias, column sum of d_drop_in; of
 // the extended form: d scale, d bias, column sum of d_drop_in = d output-bias).
-template <int VPL, bool EXT, bool PACKED, bool MOVE>
+template <int VPL, bool EXT, bool PACKED, bool MOVE, bool FLAT>
 __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, float* ws, unsigned nrows) {
     constexpr int NS = MOVE ? 3 : (EXT ? 4 : 2);
     constexpr int S_DROP = MOVE ? 2 : 3;          // which sum takes d_drop_in
@@ -89,14 +97,14 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
     const unsigned stride = gridDim.x * LN_WPB;
     unsigned row = blockIdx.x * LN_WPB + wave;
     LnRow<VPL> cur, nxt;
-    if (row < nrows) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row, lane, nv, cur);
+    if (row < nrows) ln_load_row<VPL, EXT, PACKED, MOVE, FLAT>(rs, a, row, lane, nv, cur);
     for (; row < nrows; row += stride) {
         // the next row's loads are in flight while this one is worked on
         const bool more = row + stride < nrows;
-        if (more) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row + stride, lane, nv, nxt);
+        if (more) ln_load_row<VPL, EXT, PACKED, MOVE, FLAT>(rs, a, row + stride, lane, nv, nxt);
         float g[VPL][8], df[VPL][8];
         float s1 = 0.f, s2 = 0.f;
-        const long og = view_offset(a.g, cur.ix);
+        const long og = ln_row_offset<FLAT>(a.g, cur.ix);
         const float is = cur.is;
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
@@ -124,7 +132,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
         s2 = wave_sum(s2);
         const float c1 = s1 * is * invn;
         const float c2 = s2 * is * is * is * invn;
-        const long oa = view_offset(a.d_ln_in, cur.ix), ob = view_offset(a.d_drop_in, cur.ix);
+        const long oa = ln_row_offset<FLAT>(a.d_ln_in, cur.ix), ob = ln_row_offset<FLAT>(a.d_drop_in, cur.ix);
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
             const int e0 = (c * WAVE + lane) * 8;
@@ -194,16 +202,21 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     const unsigned nrows = (unsigned)rs.rows();
     const int blocks = lnbwd_blocks(nrows);
     const int vpl = rs.R <= 512 ? 1 : 2;
-#define SUB_LNBWD(VPL_, EXT_)                                                                                     \
+#define SUB_LNBWD_F(VPL_, EXT_, FLAT_)                                                                            \
     do {                                                                                                          \
         if (a.mask_bits && a.move_sum)                                                                            \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);  \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, true, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);  \
         else if (a.mask_bits)                                                                                     \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, false, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
         else if (a.move_sum)                                                                                      \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, true>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, true, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
         else                                                                                                      \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, false>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, false, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+    } while (0)
+#define SUB_LNBWD(VPL_, EXT_)                                                                                     \
+    do {                                                                                                          \
+        if (rs.flat) SUB_LNBWD_F(VPL_, EXT_, true);                                                               \
+        else SUB_LNBWD_F(VPL_, EXT_, false);                                                                      \
     } while (0)
     if (ext) {
         if (vpl == 1) SUB_LNBWD(1, true);
@@ -212,6 +225,7 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
         if (vpl == 1) SUB_LNBWD(1, false);
         else SUB_LNBWD(2, false);
     }
+#undef SUB_LNBWD_F
 #undef SUB_LNBWD
     check_launch("fused LayerNorm backward");
     // with move_sum both forms have three sums; the extended form's third is the output-bias gradient

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
                 int nv = nvalid_at(rs.R, e0);
                 if (nv > 0) {
                     h8 a, d;
-                    uint32_t bits = keep_bits8(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0);
+                    uint32_t bits = keep_pack<FAST>(key, (uint64_t)row * (uint64_t)rs.R + (uint64_t)e0);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) a[i] = (half_t)(x[r][c][i] * inv);
                     a = pin(a);
@@ -184,6 +184,17 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
     const int lane = threadIdx.x & 63;
     const unsigned step = row_blocks * WPB * RPW;
     const float invn = 1.0f / (float)rs.R;
+    // the lane's columns of the LayerNorm scale and bias: the same for every row, fetched once
+    // and together with the first row (in the store phase they were a round trip of their own)
+    h8 sc8[VPL], bi8[VPL];
+    if (FAST) {
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            const int e0 = (c * WAVE + lane) * 8, e0s = nvalid_at(rs.R, e0) ? e0 : 0;
+            sc8[c] = ldg8<false>(scale.p + e0s);
+            bi8[c] = ldg8<false>(bias.p + e0s);
+        }
+    }
     for (unsigned row0 = (blockIdx.x * WPB + (threadIdx.x >> 6)) * RPW; row0 < nrows; row0 += step) {
         float x[RPW][VPL][8];
         uint32_t bits[RPW][VPL];
@@ -197,13 +208,26 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
             const long oi = view_offset(in, ix[r]), orr = view_offset(resid, ix[r]);
             const long ol = view_offset(lin, ix[r]), om = view_offset(mask, ix[r]);
             s[r] = 0.f;
+            // every load of the row before the first store: the compiler keeps a load behind a
+            // store that might write what it reads, and the packs of a row would make one round
+            // trip to memory each
+            F8 fis[VPL], frs[VPL], fbs[VPL];
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = live ? nvalid_at(rs.R, e0) : 0;
-                F8 fi = ld8<FAST, true>(in, oi, e0, nv), fr = ld8<FAST>(resid, orr, e0, nv);
-                F8 fb = ld8<FAST>(lin_bias, 0, e0, nv);
-                bits[r][c] = nv > 0 ? keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0) : 0u;
+                fis[c] = ld8<FAST, true>(in, oi, e0, nv);
+                frs[c] = ld8<FAST>(resid, orr, e0, nv);
+                fbs[c] = ld8<FAST>(lin_bias, 0, e0, nv);
+            }
+#pragma unroll
+            for (int c = 0; c < VPL; ++c) {
+                int e0 = (c * WAVE + lane) * 8;
+                int nv = live ? nvalid_at(rs.R, e0) : 0;
+                const F8 &fi = fis[c], &fr = frs[c], &fb = fbs[c];
+                // (FAST: drawn for every lane, no branch between the loads and their first use)
+                bits[r][c] = FAST ? keep_pack<true>(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0)
+                             : nv > 0 ? keep_bits8(key, (uint64_t)(row0 + r) * (uint64_t)rs.R + (uint64_t)e0) : 0u;
                 h8 lh;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) lh[i] = (half_t)(fi.v[i] + fb.v[i]);
@@ -211,7 +235,8 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     float kept = ((bits[r][c] >> i) & 1u) ? (float)lh[i] : 0.f;
-                    x[r][c][i] = i < nv ? kept + fr.v[i] : 0.f;
+                    // (FAST: a chunk outside the row was loaded as zeros and sums to zero)
+                    x[r][c][i] = (FAST || i < nv) ? kept + fr.v[i] : 0.f;
                     s[r] += x[r][c][i];
                 }
                 if (nv > 0) {
@@ -250,7 +275,16 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                 int e0 = (c * WAVE + lane) * 8;
                 int nv = nvalid_at(rs.R, e0);
                 if (nv > 0) {
-                    F8 fs = ld8<FAST>(scale, 0, e0, nv), fb = ld8<FAST>(bias, 0, e0, nv);
+                    F8 fs, fb;
+                    if (FAST) {
+                        // (opaque here: converted ahead of the loop, they would be waited for there,
+                        // before the row's own loads are issued)
+                        const h8 s8 = pin(sc8[c]), b8 = pin(bi8[c]);
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) { fs.v[i] = (float)s8[i]; fb.v[i] = (float)b8[i]; }
+                    } else {
+                        fs = ld8<FAST>(scale, 0, e0, nv); fb = ld8<FAST>(bias, 0, e0, nv);
+                    }
                     h8 d, n, o;
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
@@ -264,6 +298,127 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln(RowSpace rs, View in, View resi
                     st8h<FAST>(out, oo, e0, nv, o);
                 }
             }
+        }
+    }
+}
+
+// k_bdrln for the layouts the encoder layer runs with: every view vectorisable and the row
+// space flat (row r of a view starts r * s3 elements in), one row per wave and pass.  Same
+// arithmetic in the same order, bit for bit; what goes is the generic kernel's bookkeeping
+// (four outer indices and strides per view, a validity count per element: over 1000 vector
+// instructions per row, half of them before the row's loads are issued, with four waves per
+// SIMD taking turns on them; the launch was bound by that, not by memory).  Here a chunk is
+// inside the row or outside it, the row's loads are issued first, together with the lane's
+// columns of the three per-feature vectors, and the keep bits are drawn while they travel.
+template <int VPL>
+__global__ __launch_bounds__(BLOCK) void k_bdrln_flat(int R, unsigned nrows, View in, View resid, View lin_bias,
+                                                      View scale, View bias, View lin, View mask, View diff,
+                                                      View normed, View out, View istd, PhiloxKey key_, float eps,
+                                                      uint8_t* mask_bits, bool write_lin, KeepWordsJob side) {
+    const unsigned row_blocks = gridDim.x - side.blocks;
+    if (blockIdx.x >= row_blocks) {
+        const PhiloxKey skey = resolved(side.key);
+        const uint32_t tiles_n = side.N / 256, items = (side.M / 256) * tiles_n * 512;
+        for (uint32_t id = (blockIdx.x - row_blocks) * BLOCK + threadIdx.x; id < items; id += side.blocks * BLOCK) {
+            const uint32_t tile = id >> 9, tm = tile / tiles_n;
+            const KeepWords k = relu_dropout_keep_words(skey, side.N, tm, tile - tm * tiles_n, (id >> 6) & 7, id & 63);
+            reinterpret_cast<uint4*>(side.out)[id] = make_uint4(k.w[0], k.w[1], k.w[2], k.w[3]);
+        }
+        return;
+    }
+    const int lane = threadIdx.x & 63;
+    const float invn = 1.0f / (float)R;
+    // (the step counter of a captured graph: fetched first and added where the keep bits are drawn, so
+    // that the wait for it stands behind the issue of every other load)
+    uint32_t step_extra = 0;
+    if (key_.step_dev) step_extra = *key_.step_dev;
+    // A chunk outside the row (rows shorter than the lanes cover) reads the row's first pack and has it
+    // and-ed away: no branch around a load or around the first use of one, where the wait for it would go.
+    typedef int i4v __attribute__((ext_vector_type(4)));
+    bool inside[VPL];
+    int e0[VPL], keep_all[VPL];
+    h8 sc8[VPL], bi8[VPL], lb8[VPL];
+#pragma unroll
+    for (int c = 0; c < VPL; ++c) {
+        e0[c] = (c * WAVE + lane) * 8;
+        inside[c] = e0[c] < R;
+        keep_all[c] = inside[c] ? -1 : 0;
+        if (!inside[c]) e0[c] = 0;
+        lb8[c] = ldg8<false>(lin_bias.p + e0[c]);
+        sc8[c] = ldg8<false>(scale.p + e0[c]);
+        bi8[c] = ldg8<false>(bias.p + e0[c]);
+    }
+    auto masked = [&](h8 v, int c) { return __builtin_bit_cast(h8, __builtin_bit_cast(i4v, v) & keep_all[c]); };
+    for (unsigned row = blockIdx.x * WPB + (threadIdx.x >> 6); row < nrows; row += row_blocks * WPB) {
+        h8 vi[VPL], vr[VPL];
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            vi[c] = ldg8<true>(in.p + (long)row * in.s3 + e0[c]);
+            vr[c] = ldg8<false>(resid.p + (long)row * resid.s3 + e0[c]);
+        }
+        // the keep bits are drawn while the loads travel: nothing that waits for one may move up here
+        __builtin_amdgcn_sched_barrier(0);
+        PhiloxKey key = key_;
+        {
+            uint32_t se = step_extra;
+            asm volatile("" : "+v"(se));                         // (not hoisted out of the loop, with its wait)
+            key.step += (uint32_t)__builtin_amdgcn_readfirstlane((int)se);
+            key.step_dev = nullptr;
+        }
+        uint32_t bits[VPL];
+#pragma unroll
+        for (int c = 0; c < VPL; ++c)
+            bits[c] = keep_pack<true>(key, (uint64_t)row * (uint64_t)R + (uint64_t)((c * WAVE + lane) * 8));
+        __builtin_amdgcn_sched_barrier(0);
+        float x[VPL][8];
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            // (opaque here: converted ahead of the loop, the per-feature vectors would be waited for
+            // there, before the row's own loads are issued)
+            const h8 in8 = masked(vi[c], c), re8 = masked(vr[c], c), lbm = masked(pin(lb8[c]), c);
+            h8 lh;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) lh[i] = (half_t)((float)in8[i] + (float)lbm[i]);
+            lh = pin(lh);                                          // LIN is stored; use its rounded value
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float kept = __int_as_float(__float_as_int((float)lh[i]) & __builtin_amdgcn_sbfe((int)bits[c], i, 1));
+                x[c][i] = kept + (float)re8[i];
+                s += x[c][i];
+            }
+            if (inside[c]) {
+                if (write_lin) stg8<true>(lin.p + (long)row * lin.s3 + e0[c], lh);
+                if (mask_bits) mask_bits[(size_t)row * (R >> 3) + (c * WAVE + lane)] = (uint8_t)bits[c];
+                else stg8<true>(mask.p + (long)row * mask.s3 + e0[c], mask_h8(bits[c]));
+            }
+        }
+        const float mean = wave_sum(s) * invn;
+        float q = 0.f;
+#pragma unroll
+        for (int c = 0; c < VPL; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                x[c][i] = __int_as_float(__float_as_int(x[c][i] - mean) & keep_all[c]);
+                q += x[c][i] * x[c][i];
+            }
+        const float is = rsqrtf(wave_sum(q) * invn + eps);       // 1/std
+        if (lane == 0) istd.p[(long)row * istd.s3] = (half_t)is;
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            if (!inside[c]) continue;
+            const h8 s8 = pin(sc8[c]), b8 = pin(bi8[c]);
+            h8 d, n, o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float nn = x[c][i] * is;
+                d[i] = (half_t)x[c][i];
+                n[i] = (half_t)nn;
+                o[i] = (half_t)(nn * (float)s8[i] + (float)b8[i]);
+            }
+            stg8<true>(diff.p + (long)row * diff.s3 + e0[c], d);
+            stg8<true>(normed.p + (long)row * normed.s3 + e0[c], n);
+            stg8<false>(out.p + (long)row * out.s3 + e0[c], o);
         }
     }
 }
@@ -469,6 +624,20 @@ void launch_bdrln(const RowSpace& rs, View in, View resid, View lin_bias, View s
         side->blocks = 0;
     }
     const unsigned extra_blocks = job.blocks;
+    if (fast && rs.flat && (mask.p || mask_bits) && (lin.p || !write_lin)) {
+        const dim3 grid(row_grid(nrows, 1) + extra_blocks);
+#define SUB_BDRLN_FLAT(V) hipLaunchKernelGGL((k_bdrln_flat<V>), grid, dim3(BLOCK), 0, st, rs.R, nrows, in, resid, lin_bias, \
+                                             scale, bias, lin, mask, diff, normed, out, istd, key, eps, mask_bits, write_lin, job)
+        switch (vpl) {
+            case 1: SUB_BDRLN_FLAT(1); break;
+            case 2: SUB_BDRLN_FLAT(2); break;
+            case 4: SUB_BDRLN_FLAT(4); break;
+            default: SUB_BDRLN_FLAT(8); break;
+        }
+#undef SUB_BDRLN_FLAT
+        check_launch("bias-dropout-residual-layernorm");
+        return;
+    }
     SUB_ROW_DISPATCH(k_bdrln, vpl, fast, rs, in, resid, lin_bias, scale, bias, lin, mask, diff, normed,
                      out, istd, key, eps, nrows, mask_bits, write_lin, job);
     check_launch("bias-dropout-residual-layernorm");

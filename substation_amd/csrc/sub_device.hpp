@@ -124,15 +124,15 @@ __device__ __forceinline__ void stg8(half_t* p, h8 v) {
 template <bool FAST, bool NT = false>
 __device__ __forceinline__ F8 ld8(const View& t, long base, int e0, int nvalid, float fill = 0.f) {
     if (FAST) {
+        // A chunk outside the row reads the row's first pack instead (`base` is a valid row
+        // also for a lane without one) and is replaced afterwards.  No branch around the load:
+        // the wait for it would sit inside the branch, and a kernel that reads three tensors
+        // would make three round trips to memory one after the other instead of one.
+        const bool inside = nvalid != 0;
+        const h8 v = ldg8<NT>(t.p + base + (inside ? e0 : 0));
         F8 r;
-        if (nvalid) {
-            h8 v = ldg8<NT>(t.p + base + e0);
 #pragma unroll
-            for (int i = 0; i < 8; ++i) r.v[i] = (float)v[i];
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) r.v[i] = fill;
-        }
+        for (int i = 0; i < 8; ++i) r.v[i] = inside ? (float)v[i] : fill;
         return r;
     }
     return load8(t, base, e0, nvalid, fill);
@@ -182,6 +182,13 @@ __device__ __forceinline__ U4 philox_group_dev(const PhiloxKey& k, uint64_t g) {
         k1 += 0xBB67AE85u;
     }
     return c;
+}
+
+// Keep bits of the 8-pack that starts at canonical element e.  FAST: rows are whole 8-packs, so
+// e is a multiple of 8 and the pack is one Philox group (no second call, no branch on e & 7).
+template <bool FAST>
+__device__ __forceinline__ uint32_t keep_pack(const PhiloxKey& key, uint64_t e) {
+    return FAST ? keep8(philox_group_dev(key, e >> 3), key.thr) : keep_bits8(key, e);
 }
 
 // The 32 keep bits of key tile t of score row `row` in the attention kernels' format (bit k =

@@ -515,6 +515,17 @@ def test_fused_epilogues_match_unfused(which, dims, act):
         outs.append([Y.detach().clone(), X.grad.clone()] + [p.grad.clone() for p in enc.parameters()])
     for a, b in zip(*outs):
         assert torch.isfinite(a.float()).all()
+        if a.dim() == 1 and not torch.equal(a, b):
+            # A per-feature gradient is a sum over all tokens, added up in fp32 in the order of the launch that
+            # forms it (a contraction's epilogue adds slabs of 128 rows, the separate operator chunks of tokens
+            # that fill the CUs): the same terms, a different order, so a sum that lands on a rounding boundary
+            # of fp16 may come out one step apart.
+            x, y = a.float().cpu().numpy(), b.float().cpu().numpy()
+            differ = x != y
+            assert differ.mean() <= 1e-3, differ.sum()
+            ulp = np.spacing(np.maximum(np.abs(x), np.abs(y))[differ].astype(np.float16)).astype(np.float64)
+            assert (np.abs(x[differ].astype(np.float64) - y[differ]) <= ulp).all()
+            continue
         assert torch.equal(a, b)
 
 
@@ -828,7 +839,9 @@ def test_options_that_only_change_where_bytes_go_give_the_same_bits(option):
     B=8 L=512 E=1024, each switched off against the default:
     8 -- the launch of the stacked projections (192 tiles for 256 CUs) draws the
          attention's dropout keep bits for the first key tiles of every score row on
-         the idle CUs, the attention kernel the rest (off: it draws them all);
+         the idle CUs, the attention kernel the rest (off: it draws them all); with
+         bit 1 set as well, workgroups behind the first LayerNorm launch draw the keep
+         bits of lin1's ReLU-dropout epilogue (compared here: both bits against none);
     9 -- the residual dropout masks travel as one bit per element (off: 0/1 tensors);
     10 -- intermediates that nothing reads are not written (off: they are)."""
     from substation_amd import Encoder, layouts as L, _lib
@@ -842,7 +855,7 @@ def test_options_that_only_change_where_bytes_go_give_the_same_bits(option):
             for p in enc.parameters():
                 p.mul_(0.05)
         enc.set_rng(SEED, 3)
-        enc._handle.set_option(option, int(side_jobs))
+        enc._handle.set_option(option, (3 if option == 8 else 1) if side_jobs else 0)
         g0 = torch.Generator().manual_seed(5)
         X = torch.randn(B, Ls, E, generator=g0).half().cuda().requires_grad_(True)
         DY = torch.randn(B, Ls, E, generator=g0).half().cuda()
