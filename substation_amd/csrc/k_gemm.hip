@@ -52,14 +52,28 @@ struct GemmArgs {
     uint32_t side_rows = 0, side_nk = 0, side_tiles_done = 0;
 };
 
+// The arguments every tile of a product needs, fetched in one go at the start of the workgroup
+// (fetch_args_now): the index arithmetic between them would otherwise be interleaved with four or
+// five scalar round trips.
+__device__ __forceinline__ void fetch_gemm_args(const GemmArgs& g) {
+    fetch_args_now(g.A, g.B, g.C, g.M, g.N, g.K1, g.K0, g.sAM, g.sAK1, g.sAK0, g.sBN, g.sBK1, g.sBK0, g.sCM, g.nb1, g.nb2,
+                   g.sAb[0], g.sAb[1], g.sAb[2], g.sBb[0], g.sBb[1], g.sBb[2], g.sCb[0], g.sCb[1], g.sCb[2], g.alpha,
+                   g.bias, g.sbM, g.splits);
+}
+
 // A workgroup that multiplies nothing (see GemmSideJob): workgroup sb of nsb.
 __device__ __forceinline__ void side_block(const GemmArgs& g, unsigned sb, unsigned nsb) {
     const PhiloxKey key = resolved(g.side_key);
     const uint32_t nt = g.side_nk / 32, td = g.side_tiles_done;
-    const uint64_t total = (uint64_t)g.side_rows * td, stride = (uint64_t)nsb * blockDim.x;
-    for (uint64_t w = (uint64_t)sb * blockDim.x + threadIdx.x; w < total; w += stride) {
-        const uint32_t row = (uint32_t)(w / td), t = (uint32_t)(w - (uint64_t)row * td);
+    // word w of rows * td is (row w / td, tile w % td); a thread walks w in steps of `stride`, carrying row
+    // and tile along instead of dividing (a 64-bit division is as long as one of the word's four draws)
+    const uint32_t stride = nsb * blockDim.x, first = sb * blockDim.x + threadIdx.x;
+    const uint32_t srow = stride / td, st = stride - srow * td;
+    uint32_t row = first / td, t = first - row * td;
+    for (; row < g.side_rows; row += srow) {
         g.side_keep[(size_t)row * nt + t] = attention_keep_word(key, row, g.side_nk, t);
+        t += st;
+        if (t >= td) { t -= td; ++row; }
     }
 }
 
@@ -249,13 +263,16 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id,
     // with its own L2), so consecutive logical tiles are given to one XCD, and
     // within a batch tiles are walked in groups of 8 tile-rows so that the
     // workgroups resident together share A and B tiles in that L2.
+    // (32-bit arithmetic: a launch has fewer than 2^31 workgroups, and each 64-bit division here is 130
+    // instructions that stand between the start of the workgroup and its first load)
+    fetch_gemm_args(g);
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    long lid = block_id;
-    if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
-    const int per_batch = tiles_m * tiles_n;
-    const int split = (int)(lid % g.splits);        // k-splits of one tile sit next to each other
-    lid /= g.splits;
-    long bz = lid / per_batch;
+    unsigned lid = (unsigned)block_id;
+    if ((nblocks & 7) == 0) lid = (lid & 7u) * (unsigned)(nblocks >> 3) + (lid >> 3);
+    const unsigned per_batch = (unsigned)(tiles_m * tiles_n);
+    const int split = (int)(lid % (unsigned)g.splits);        // k-splits of one tile sit next to each other
+    lid /= (unsigned)g.splits;
+    const unsigned bz = lid / per_batch;
     int r = (int)(lid - bz * per_batch);
     // (a tall tile's rows are the dearer operand: the 16 tiles an XCD holds of one product as 2 rows x 8
     // columns draw 192 KiB per k-step into its L2, as 8 x 2 288 KiB; measured 0.7 us per pair launch)
@@ -264,8 +281,8 @@ __device__ __forceinline__ void gemm_mfma_body(const GemmArgs& g, long block_id,
     const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
     const int rr = r - grp * GM * tiles_n;
     const int tile_m = first_m + rr % gsz, tile_n = rr / gsz;
-    long b2 = bz % g.nb2; long t = bz / g.nb2;
-    long b1 = t % g.nb1; long b0 = t / g.nb1;
+    const unsigned tq = bz / (unsigned)g.nb2;
+    const long b2 = bz - tq * (unsigned)g.nb2, b0 = tq / (unsigned)g.nb1, b1 = tq - (unsigned)b0 * (unsigned)g.nb1;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const half_t* Ab = g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM;
     const half_t* Bb = g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN;
@@ -669,28 +686,30 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, hi = lane >> 5;
 
+    fetch_gemm_args(g);
     const int tiles_m = g.M / BM, tiles_n = g.N / BN;
-    long lid = blockIdx.x;
+    unsigned lid = blockIdx.x;
     {
-        long nblocks = gridDim.x;
+        unsigned nblocks = gridDim.x;
         if constexpr (NW == 8 && EPI == EPI_PLAIN) {
             if (g.side_blocks) {
                 if (blockIdx.x >= g.side_first) { side_block(g, blockIdx.x - g.side_first, g.side_blocks); return; }
                 nblocks = g.side_first;
             }
         }
-        if ((nblocks & 7) == 0) lid = (lid & 7) * (nblocks >> 3) + (lid >> 3);
+        if ((nblocks & 7) == 0) lid = (lid & 7u) * (nblocks >> 3) + (lid >> 3);
     }
-    const int per_batch = tiles_m * tiles_n;
-    long bz = lid / per_batch;
+    // (32-bit arithmetic, as in the register-staged kernel)
+    const unsigned per_batch = (unsigned)(tiles_m * tiles_n);
+    const unsigned bz = lid / per_batch;
     int r = (int)(lid - bz * per_batch);
     constexpr int GM = 8;
     const int grp = r / (GM * tiles_n), first_m = grp * GM;
     const int gsz = tiles_m - first_m < GM ? tiles_m - first_m : GM;
     const int rr = r - grp * GM * tiles_n;
     const int tile_m = first_m + rr % gsz, tile_n = rr / gsz;
-    long b2 = bz % g.nb2; long t = bz / g.nb2;
-    long b1 = t % g.nb1; long b0 = t / g.nb1;
+    const unsigned tq = bz / (unsigned)g.nb2;
+    const long b2 = bz - tq * (unsigned)g.nb2, b0 = tq / (unsigned)g.nb1, b1 = tq - (unsigned)b0 * (unsigned)g.nb1;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const half_t* pa = g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM;
     const half_t* pb = g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN;

@@ -315,6 +315,9 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln_flat(int R, unsigned nrows, Vie
                                                       View scale, View bias, View lin, View mask, View diff,
                                                       View normed, View out, View istd, PhiloxKey key_, float eps,
                                                       uint8_t* mask_bits, bool write_lin, KeepWordsJob side) {
+    fetch_args_now(R, nrows, in.p, in.s3, resid.p, resid.s3, lin_bias.p, scale.p, bias.p, lin.p, lin.s3, mask.p, mask.s3,
+                   diff.p, diff.s3, normed.p, normed.s3, out.p, out.s3, istd.p, istd.s3, key_.k0, key_.k1, key_.site,
+                   key_.step, key_.thr, key_.step_dev, eps, mask_bits, write_lin, side.blocks);
     const unsigned row_blocks = gridDim.x - side.blocks;
     if (blockIdx.x >= row_blocks) {
         const PhiloxKey skey = resolved(side.key);

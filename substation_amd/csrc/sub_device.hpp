@@ -147,6 +147,18 @@ __device__ __forceinline__ void st8h(const View& t, long base, int e0, int nvali
     }
 }
 
+// Kernel arguments wanted in registers now.  Left alone, the compiler fetches each argument where it is
+// first used, with a wait of its own: a kernel with many of them then starts with four or five scalar
+// round trips to memory one after the other (about half a microsecond each) before its first vector
+// load is issued.  Named here, they are fetched in one go.
+template <typename T>
+__device__ __forceinline__ void fetch_arg_now(const T& v) {
+    if constexpr (sizeof(T) < 4) { const int w = (int)v; asm volatile("" ::"s"(w)); }
+    else asm volatile("" ::"s"(v));
+}
+template <typename... T>
+__device__ __forceinline__ void fetch_args_now(const T&... v) { (fetch_arg_now(v), ...); }
+
 // The key a kernel works with: the device-side step counter, if any, folded in.
 __device__ __forceinline__ PhiloxKey resolved(PhiloxKey k) {
     if (k.step_dev) k.step += *k.step_dev;
