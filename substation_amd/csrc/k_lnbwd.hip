@@ -31,22 +31,14 @@ struct LnRow {
     RowIdx ix;
 };
 
-// Where row `ix` of view `v` starts.  FLAT: the row space is flat (RowSpace::flat, what the encoder
-// layer's layouts give), the row is its only index: one multiplication in place of four.
-template <bool FLAT>
-__device__ __forceinline__ long ln_row_offset(const View& v, const RowIdx& ix) {
-    return FLAT ? (long)ix.i3 * v.s3 : view_offset(v, ix);
-}
-
-template <int VPL, bool EXT, bool PACKED, bool MOVE, bool FLAT>
+template <int VPL, bool EXT, bool PACKED, bool MOVE>
 __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs& a, unsigned row, int lane,
                                             const int (&nv)[VPL], LnRow<VPL>& r) {
-    if (FLAT) { r.ix.i0 = r.ix.i1 = r.ix.i2 = 0; r.ix.i3 = row; }
-    else r.ix = row_index(rs, row);
-    const long oin = ln_row_offset<FLAT>(a.in, r.ix), o1 = ln_row_offset<FLAT>(a.d1, r.ix),
-               odf = ln_row_offset<FLAT>(a.diff, r.ix), omk = ln_row_offset<FLAT>(a.mask, r.ix);
-    const long o2 = EXT ? ln_row_offset<FLAT>(a.d2, r.ix) : 0, odl = EXT ? ln_row_offset<FLAT>(a.dlinear, r.ix) : 0;
-    r.is = (float)a.istd.p[ln_row_offset<FLAT>(a.istd, r.ix)];
+    r.ix = row_index(rs, row);
+    const long oin = view_offset(a.in, r.ix), o1 = view_offset(a.d1, r.ix), odf = view_offset(a.diff, r.ix),
+               omk = view_offset(a.mask, r.ix);
+    const long o2 = EXT ? view_offset(a.d2, r.ix) : 0, odl = EXT ? view_offset(a.dlinear, r.ix) : 0;
+    r.is = (float)a.istd.p[view_offset(a.istd, r.ix)];
 #pragma unroll
     for (int c = 0; c < VPL; ++c) {
         const int e0 = (c * WAVE + lane) * 8;
@@ -72,7 +64,7 @@ __device__ __forceinline__ void ln_load_row(const RowSpace& rs, const LnBwdArgs&
 // extended form (two incoming gradients, linear-bias and output-bias sums).
 // MOVE: see LnBwdArgs::move_sum (sums of the plain form: d scale, d bias, column sum of d_drop_in; of
 // the extended form: d scale, d bias, column sum of d_drop_in = d output-bias).
-template <int VPL, bool EXT, bool PACKED, bool MOVE, bool FLAT>
+template <int VPL, bool EXT, bool PACKED, bool MOVE>
 __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, float* ws, unsigned nrows) {
     constexpr int NS = MOVE ? 3 : (EXT ? 4 : 2);
     constexpr int S_DROP = MOVE ? 2 : 3;          // which sum takes d_drop_in
@@ -97,14 +89,14 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
     const unsigned stride = gridDim.x * LN_WPB;
     unsigned row = blockIdx.x * LN_WPB + wave;
     LnRow<VPL> cur, nxt;
-    if (row < nrows) ln_load_row<VPL, EXT, PACKED, MOVE, FLAT>(rs, a, row, lane, nv, cur);
+    if (row < nrows) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row, lane, nv, cur);
     for (; row < nrows; row += stride) {
         // the next row's loads are in flight while this one is worked on
         const bool more = row + stride < nrows;
-        if (more) ln_load_row<VPL, EXT, PACKED, MOVE, FLAT>(rs, a, row + stride, lane, nv, nxt);
+        if (more) ln_load_row<VPL, EXT, PACKED, MOVE>(rs, a, row + stride, lane, nv, nxt);
         float g[VPL][8], df[VPL][8];
         float s1 = 0.f, s2 = 0.f;
-        const long og = ln_row_offset<FLAT>(a.g, cur.ix);
+        const long og = view_offset(a.g, cur.ix);
         const float is = cur.is;
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
@@ -132,7 +124,7 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
         s2 = wave_sum(s2);
         const float c1 = s1 * is * invn;
         const float c2 = s2 * is * is * is * invn;
-        const long oa = ln_row_offset<FLAT>(a.d_ln_in, cur.ix), ob = ln_row_offset<FLAT>(a.d_drop_in, cur.ix);
+        const long oa = view_offset(a.d_ln_in, cur.ix), ob = view_offset(a.d_drop_in, cur.ix);
 #pragma unroll
         for (int c = 0; c < VPL; ++c) {
             const int e0 = (c * WAVE + lane) * 8;
@@ -172,6 +164,170 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
     }
 }
 
+// The same launch for a flat row space with sixteen waves per workgroup and one row per wave and pass:
+// four waves per SIMD take turns on the 500 vector instructions a row needs, where the kernel above
+// has two (its registers: this row, the next row's loads, 48 column-sum accumulators).  To fit the 128
+// registers that leaves a lane, the row's loads are not held beyond their use, the LayerNorm scale is
+// fetched with the row, and the column sum of d_drop_in does not live in registers: a wave adds its
+// rows' values into its own slab of LDS, which the reduction of the other sums reuses afterwards.
+// Same arithmetic per row; a column sum adds a lane's rows in order, then the waves in order.
+constexpr int LNF_BLOCK = 1024;
+constexpr int LNF_WPB = LNF_BLOCK / WAVE;
+
+template <int VPL, bool EXT, bool PACKED, bool MOVE>
+__global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, float* ws, unsigned nrows) {
+    constexpr int NS = MOVE ? 3 : (EXT ? 4 : 2);
+    constexpr int S_DROP = MOVE ? 2 : 3;          // which sum takes d_drop_in
+    constexpr bool DROP_SUM = EXT || MOVE;
+    constexpr int NR = DROP_SUM ? NS - 1 : NS;    // sums kept in registers
+    __shared__ float red[LNF_WPB][VPL * WAVE * 8];
+    typedef int i4v __attribute__((ext_vector_type(4)));
+    fetch_args_now(R, nrows, a.in.p, a.in.s3, a.d1.p, a.d1.s3, a.diff.p, a.diff.s3, a.istd.p, a.istd.s3, a.scale.p, a.g.p,
+                   a.g.s3, a.d_ln_in.p, a.d_ln_in.s3, a.d_drop_in.p, a.d_drop_in.s3, a.write_g, ws);
+    if (EXT) fetch_args_now(a.d2.p, a.d2.s3);
+    if (EXT && !MOVE) fetch_args_now(a.dlinear.p, a.dlinear.s3);
+    if (PACKED) fetch_args_now(a.mask_bits);
+    else fetch_args_now(a.mask.p, a.mask.s3);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float invn = 1.0f / (float)R;
+    float acc[NR][VPL][8];
+#pragma unroll
+    for (int s = 0; s < NR; ++s)
+#pragma unroll
+        for (int c = 0; c < VPL; ++c)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[s][c][i] = 0.f;
+    // A chunk outside the row reads the row's first pack and has it and-ed away: no branch around a load.
+    bool inside[VPL];
+    int e0[VPL], keep_all[VPL];
+#pragma unroll
+    for (int c = 0; c < VPL; ++c) {
+        e0[c] = (c * WAVE + lane) * 8;
+        inside[c] = e0[c] < R;
+        keep_all[c] = inside[c] ? -1 : 0;
+        if (!inside[c]) e0[c] = 0;
+    }
+    auto masked = [&](h8 v, int c) { return __builtin_bit_cast(h8, __builtin_bit_cast(i4v, v) & keep_all[c]); };
+    float* const slab = &red[wave][lane * 8];     // + c * 512: this lane's 8 columns of pack c
+    bool first_row = true;
+    for (unsigned row = blockIdx.x * LNF_WPB + wave; row < nrows; row += gridDim.x * LNF_WPB) {
+        h8 in[VPL], d1[VPL], d2[VPL], dl[VPL], df[VPL], mk[VPL], sc[VPL];
+        uint32_t mkb[VPL];
+        const half_t isth = a.istd.p[(long)row * a.istd.s3];
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            in[c] = ldg8<true>(a.in.p + (long)row * a.in.s3 + e0[c]);          // saved by the forward pass
+            // the incoming gradient of the plain form is the caller's tensor;
+            // those of the extended form are intermediates on their last use
+            d1[c] = ldg8<EXT>(a.d1.p + (long)row * a.d1.s3 + e0[c]);
+            if (EXT) {
+                d2[c] = ldg8<true>(a.d2.p + (long)row * a.d2.s3 + e0[c]);
+                if (!MOVE) dl[c] = ldg8<true>(a.dlinear.p + (long)row * a.dlinear.s3 + e0[c]);
+            }
+            sc[c] = ldg8<false>(a.scale.p + e0[c]);
+            df[c] = ldg8<true>(a.diff.p + (long)row * a.diff.s3 + e0[c]);
+            if (PACKED) mkb[c] = a.mask_bits[(size_t)row * (R >> 3) + (e0[c] >> 3)];
+            else mk[c] = ldg8<true>(a.mask.p + (long)row * a.mask.s3 + e0[c]);
+        }
+        const float is = (float)isth;
+        float s1 = 0.f, s2 = 0.f;
+        h8 gh[VPL];
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            const h8 in8 = masked(in[c], c), d18 = masked(d1[c], c), sc8 = masked(sc[c], c);
+            h8 d28, dl8;
+            if (EXT) d28 = masked(d2[c], c);
+            if (EXT && !MOVE) dl8 = masked(dl[c], c);
+            df[c] = masked(df[c], c);
+            h8 o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float d = EXT ? (float)d18[i] + (float)d28[i] : (float)d18[i];
+                o[i] = (half_t)(d * (float)sc8[i]);
+                acc[0][c][i] += d * (float)in8[i];
+                acc[1][c][i] += d;
+                if (EXT && !MOVE) acc[2][c][i] += (float)dl8[i];
+            }
+            o = pin(o);
+            if (inside[c] && a.write_g) stg8<true>(a.g.p + (long)row * a.g.s3 + e0[c], o);     // nothing reads G again
+            gh[c] = o;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                s1 += (float)o[i];
+                s2 = __fmaf_rn((float)o[i], (float)df[c][i], s2);
+            }
+            // one pack after the other: interleaved, their converted values do not fit the registers
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        s1 = wave_sum(s1);
+        s2 = wave_sum(s2);
+        const float c1 = s1 * is * invn;
+        const float c2 = s2 * is * is * is * invn;
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            h8 x, y;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = (half_t)ln_bwd_value((float)gh[c][i], (float)df[c][i], is, c1, c2);
+            x = pin(x);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const bool kept = PACKED ? ((mkb[c] >> i) & 1u) != 0 : mk[c][i] != (half_t)0.0f;
+                y[i] = kept ? x[i] : (half_t)0.0f;
+            }
+            if (DROP_SUM) {
+                // (a chunk outside the row: x comes out as -c1, which must not be summed)
+                const h8 ys = masked(y, c);
+                float4 lo = make_float4((float)ys[0], (float)ys[1], (float)ys[2], (float)ys[3]);
+                float4 hi = make_float4((float)ys[4], (float)ys[5], (float)ys[6], (float)ys[7]);
+                if (!first_row) {
+                    const float4 plo = *reinterpret_cast<const float4*>(slab + c * 512);
+                    const float4 phi = *reinterpret_cast<const float4*>(slab + c * 512 + 4);
+                    lo.x += plo.x; lo.y += plo.y; lo.z += plo.z; lo.w += plo.w;
+                    hi.x += phi.x; hi.y += phi.y; hi.z += phi.z; hi.w += phi.w;
+                }
+                *reinterpret_cast<float4*>(slab + c * 512) = lo;
+                *reinterpret_cast<float4*>(slab + c * 512 + 4) = hi;
+            }
+            if (inside[c]) {
+                stg8<false>(a.d_ln_in.p + (long)row * a.d_ln_in.s3 + e0[c], x);
+                stg8<false>(a.d_drop_in.p + (long)row * a.d_drop_in.s3 + e0[c], y);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        first_row = false;
+    }
+    if (DROP_SUM && first_row) {                   // a wave without a row
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            *reinterpret_cast<float4*>(slab + c * 512) = make_float4(0.f, 0.f, 0.f, 0.f);
+            *reinterpret_cast<float4*>(slab + c * 512 + 4) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    // One partial row per block and sum: ws[(s * gridDim.x + block) * R + feature].  The sum of
+    // d_drop_in lies in the slabs already; the others follow from the registers.
+    auto reduce_slabs = [&](int s) {
+        __syncthreads();
+        for (int f = threadIdx.x; f < R; f += LNF_BLOCK) {
+            float t = 0.f;
+#pragma unroll
+            for (int w = 0; w < LNF_WPB; ++w) t += red[w][f];
+            ws[((long)s * gridDim.x + blockIdx.x) * R + f] = t;
+        }
+    };
+    if (DROP_SUM) reduce_slabs(S_DROP);
+#pragma unroll
+    for (int s = 0; s < NR; ++s) {
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            *reinterpret_cast<float4*>(slab + c * 512) = make_float4(acc[s][c][0], acc[s][c][1], acc[s][c][2], acc[s][c][3]);
+            *reinterpret_cast<float4*>(slab + c * 512 + 4) = make_float4(acc[s][c][4], acc[s][c][5], acc[s][c][6], acc[s][c][7]);
+        }
+        // (with MOVE the register sums are 0, 1; without it 0, 1 and for the extended form 2)
+        reduce_slabs(s);
+    }
+}
+
 inline int lnbwd_blocks(long nrows) {
     // two rows per wave where there are enough rows; at most 2048 waves
     long blocks = (nrows + 2L * LN_WPB - 1) / (2L * LN_WPB);
@@ -202,21 +358,22 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     const unsigned nrows = (unsigned)rs.rows();
     const int blocks = lnbwd_blocks(nrows);
     const int vpl = rs.R <= 512 ? 1 : 2;
-#define SUB_LNBWD_F(VPL_, EXT_, FLAT_)                                                                            \
+#define SUB_LNBWD_K(KERNEL_, BLOCK_, FIRST_, VPL_, EXT_)                                                          \
     do {                                                                                                          \
         if (a.mask_bits && a.move_sum)                                                                            \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, true, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows);  \
+            hipLaunchKernelGGL((KERNEL_<VPL_, EXT_, true, true>), dim3(blocks), dim3(BLOCK_), 0, st, FIRST_, a, ws, nrows);  \
         else if (a.mask_bits)                                                                                     \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, true, false, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((KERNEL_<VPL_, EXT_, true, false>), dim3(blocks), dim3(BLOCK_), 0, st, FIRST_, a, ws, nrows); \
         else if (a.move_sum)                                                                                      \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, true, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((KERNEL_<VPL_, EXT_, false, true>), dim3(blocks), dim3(BLOCK_), 0, st, FIRST_, a, ws, nrows); \
         else                                                                                                      \
-            hipLaunchKernelGGL((k_lnbwd<VPL_, EXT_, false, false, FLAT_>), dim3(blocks), dim3(LN_BLOCK), 0, st, rs, a, ws, nrows); \
+            hipLaunchKernelGGL((KERNEL_<VPL_, EXT_, false, false>), dim3(blocks), dim3(BLOCK_), 0, st, FIRST_, a, ws, nrows); \
     } while (0)
+    // (the extended form with its four sums does not fit the sixteen-wave kernel's registers)
 #define SUB_LNBWD(VPL_, EXT_)                                                                                     \
     do {                                                                                                          \
-        if (rs.flat) SUB_LNBWD_F(VPL_, EXT_, true);                                                               \
-        else SUB_LNBWD_F(VPL_, EXT_, false);                                                                      \
+        if (rs.flat && !(EXT_ && !a.move_sum)) SUB_LNBWD_K(k_lnbwd_flat, LNF_BLOCK, rs.R, VPL_, EXT_);            \
+        else SUB_LNBWD_K(k_lnbwd, LN_BLOCK, rs, VPL_, EXT_);                                                      \
     } while (0)
     if (ext) {
         if (vpl == 1) SUB_LNBWD(1, true);
@@ -225,7 +382,7 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
         if (vpl == 1) SUB_LNBWD(1, false);
         else SUB_LNBWD(2, false);
     }
-#undef SUB_LNBWD_F
+#undef SUB_LNBWD_K
 #undef SUB_LNBWD
     check_launch("fused LayerNorm backward");
     // with move_sum both forms have three sums; the extended form's third is the output-bias gradient
