@@ -14,6 +14,7 @@
 // The output is produced transposed in the
 // accumulators (4 consecutive n per lane), staged through LDS and written as
 // full 128-bit rows.
+#include <type_traits>
 #include <cstring>
 
 #include "sub_ops.hpp"
@@ -904,64 +905,93 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) gbits[i] = g.gate_bits[bits_at + i * 64];
     }
+    // The lane's stores walk down the tile RPI rows at a time: running pointers (a 64-bit product
+    // per store otherwise), and one copy of the loop per kind of addend (none, a bias row, a tensor:
+    // chosen per store, the branches joined in a wait for every store issued so far).  Most products
+    // have alpha = 1: no multiplication then.
+    const bool alpha_one = g.alpha == 1.0f;
+    const long c_step = (long)RPI * g.sCM, b_step = (long)RPI * g.sbM;
+    const int row_first = m0 + wm * 32 * TM + lane / LPR, col_first = n0 + wn * 32 * TN + (lane % LPR) * 8;
+    half_t* const c_first = Cb + (long)row_first * g.sCM + col_first;
+    const long b_first = (long)row_first * g.sbM + col_first;        // addend and gate share their strides
+    auto store_tile = [&](auto addend_kind) {
+        constexpr int ADD = decltype(addend_kind)::value;           // 0 none, 1 a bias row, 2 a tensor
+        half_t* cp = c_first;
+        const half_t* bp = ADD == 2 ? biasb + b_first : nullptr;
+        const half_t* gp = (EPI == EPI_GATE_COLSUM && !g.gate_bits) ? g.gate + b_first : nullptr;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int mrow = m0 + wm * 32 * TM + i * 32;
-        uint32_t positive = 0;
+        for (int i = 0; i < TM; ++i) {
+            uint32_t positive = 0;
+            if (alpha_one) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+                for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                h4 w;
-                int ncol = j * 32 + q * 8 + hi * 4;
+                    for (int q = 0; q < 4; ++q) {
+                        h4 w;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[i][j][q * 4 + e] * g.alpha);
-                *reinterpret_cast<h4*>(stage + l32 * STAGE_PITCH + ncol) = w;
+                        for (int e = 0; e < 4; ++e) w[e] = (half_t)acc[i][j][q * 4 + e];
+                        *reinterpret_cast<h4*>(stage + l32 * STAGE_PITCH + j * 32 + q * 8 + hi * 4) = w;
+                    }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        h4 w;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w[e] = (half_t)(acc[i][j][q * 4 + e] * g.alpha);
+                        *reinterpret_cast<h4*>(stage + l32 * STAGE_PITCH + j * 32 + q * 8 + hi * 4) = w;
+                    }
             }
 #pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it) {
-            int rr2 = it * RPI + lane / LPR, c8 = (lane % LPR) * 8;
-            h8 val = *reinterpret_cast<const h8*>(stage + rr2 * STAGE_PITCH + c8);
-            int mm = mrow + rr2, nn = n0 + wn * 32 * TN + c8;
-            if (biasb) {
-                const h8 ad = bias_row ? bias8 : *reinterpret_cast<const h8*>(biasb + (long)mm * g.sbM + nn);
-                val = val + ad;          // packed half add: the same single rounding as through fp32
-            }
-            if (EPI == EPI_GATE_COLSUM) {
-                // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
-                if (g.gate_bits) {
-                    const uint32_t bits = gbits[i] >> (8 * it);
+            for (int it = 0; it < 32 / RPI; ++it) {
+                const int rr2 = it * RPI + lane / LPR, c8 = (lane % LPR) * 8;
+                h8 val = *reinterpret_cast<const h8*>(stage + rr2 * STAGE_PITCH + c8);
+                // packed half add: the same single rounding as through fp32
+                if (ADD == 1) val = val + bias8;
+                if (ADD == 2) val = val + *reinterpret_cast<const h8*>(bp);
+                if (EPI == EPI_GATE_COLSUM) {
+                    // the ReLU layer's backward-dropout-activation: zero where the forward output was not positive
+                    if (g.gate_bits) {
+                        const uint32_t bits = gbits[i] >> (8 * it);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            val[e] = ((bits >> e) & 1u) ? val[e] : (half_t)0.0f;
+                            colsum[e] += (float)val[e];
+                        }
+                    } else {
+                        const h8 gt = *reinterpret_cast<const h8*>(gp);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            val[e] = (float)gt[e] > 0.f ? val[e] : (half_t)0.0f;
+                            colsum[e] += (float)val[e];
+                        }
+                    }
+                }
+                if (RELU_DROP) {
+                    // what the bias-activation-dropout operator does to the rounded sum, with the
+                    // same keep bits (the element index is the offset into the dense output):
+                    // pack c sits in byte 15 - c of the bits drawn in the main loop
+                    const int c = i * (32 / RPI) + it, byte = 15 - c;
+                    const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
+                    val = __builtin_elementwise_max(val, (h8)(half_t)0.0f);       // ReLU, packed
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         val[e] = ((bits >> e) & 1u) ? val[e] : (half_t)0.0f;
-                        colsum[e] += (float)val[e];
-                    }
-                } else {
-                    const h8 gt = *reinterpret_cast<const h8*>(g.gate + (long)mm * g.sbM + nn);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        val[e] = (float)gt[e] > 0.f ? val[e] : (half_t)0.0f;
-                        colsum[e] += (float)val[e];
+                        positive |= (val[e] > (half_t)0.0f ? 1u : 0u) << (8 * it + e);
                     }
                 }
+                *reinterpret_cast<h8*>(cp) = val;
+                cp += c_step;
+                if (ADD == 2) bp += b_step;
+                if (EPI == EPI_GATE_COLSUM) gp += b_step;
             }
-            if (RELU_DROP) {
-                // what the bias-activation-dropout operator does to the rounded sum, with the
-                // same keep bits (the element index is the offset into the dense output):
-                // pack c sits in byte 15 - c of the bits drawn in the main loop
-                const int c = i * (32 / RPI) + it, byte = 15 - c;
-                const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
-                val = __builtin_elementwise_max(val, (h8)(half_t)0.0f);       // ReLU, packed
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    val[e] = ((bits >> e) & 1u) ? val[e] : (half_t)0.0f;
-                    positive |= (val[e] > (half_t)0.0f ? 1u : 0u) << (8 * it + e);
-                }
-            }
-            *reinterpret_cast<h8*>(Cb + (long)mm * g.sCM + nn) = val;
+            if (RELU_DROP && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
         }
-        if (RELU_DROP && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
-    }
+    };
+    if (!biasb) store_tile(std::integral_constant<int, 0>{});
+    else if (bias_row) store_tile(std::integral_constant<int, 1>{});
+    else store_tile(std::integral_constant<int, 2>{});
     if (EPI == EPI_GATE_COLSUM) {
         // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
         // row of partial sums per 128-row slab of the output (a finishing launch adds the slabs)
