@@ -147,13 +147,30 @@ template <int P>
 __device__ __forceinline__ void column_sums(const f16v (&acc)[P / 32], float scale, float* red, float* out,
                                             int tid) {
     const int lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
+    // Five DPP steps per value and no trip through LDS: four total each row of 16 lanes, the fifth
+    // (row_bcast15 into rows 1 and 3) adds the row below, so that lanes 16..31 (48..63) hold the total
+    // of lanes 0..31 (32..63).  All values first and then the store: the chains are independent and
+    // fill each other's wait states.  (With a ds_bpermute as the last step the 32 values of a lane went
+    // through LDS one after the other, 2 to 3 us at the end of every workgroup.)
+    float x[P / 32][16];
 #pragma unroll
     for (int pt = 0; pt < P / 32; ++pt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const float x = group_sum<32>((float)(half_t)(acc[pt][v] * scale));
-            if (l32 == 0) red[wave * P + pt * 32 + reg_pos(v, hi)] = x;
+            float t = (float)(half_t)(acc[pt][v] * scale);
+            t += dpp<0xB1>(t);
+            t += dpp<0x4E>(t);
+            t += dpp<0x141>(t);
+            t += dpp<0x140>(t);
+            t += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(t), 0x142, 0xA, 0xF, false));
+            x[pt][v] = t;
         }
+    if (l32 == 16) {
+#pragma unroll
+        for (int pt = 0; pt < P / 32; ++pt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) red[wave * P + pt * 32 + reg_pos(v, hi)] = x[pt][v];
+    }
     __syncthreads();
     if (tid < P) out[tid] = (red[tid] + red[P + tid]) + (red[2 * P + tid] + red[3 * P + tid]);
 }
