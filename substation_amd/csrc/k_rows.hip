@@ -27,7 +27,7 @@ __device__ __forceinline__ int nvalid_at(int R, int e0) {
 // amask (optional, p == nullptr when absent): additive attention mask indexed by
 // (query position, key position) only, x = beta * scale + amask * mscale
 // (substation/attention.py:65-68 adds it before the scaling, hence mscale).
-template <int VPL, int RPW, bool FAST, int GRP = WAVE, bool MASKED = false>
+template <int VPL, int RPW, bool FAST, bool FLAT = false, int GRP = WAVE, bool MASKED = false>
 __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View alpha, View mask,
                                                    View drop, View amask, float scale, float mscale,
                                                    PhiloxKey key_, unsigned nrows) {
@@ -43,9 +43,9 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
         for (int r = 0; r < RPW; ++r) {
             const unsigned row = row0 + r * SPW + sub;
             const bool live = row < nrows;
-            ix[r] = row_index(rs, live ? row : row0);
-            const long ob = view_offset(beta, ix[r]);
-            const long oam = MASKED ? view_offset(amask, ix[r]) : 0;
+            ix[r] = row_index_of<FLAT>(rs, live ? row : row0);
+            const long ob = view_offset_of<FLAT>(beta, ix[r]);
+            const long oam = MASKED ? view_offset_of<FLAT>(amask, ix[r]) : 0;
             m[r] = -INFINITY;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
             const unsigned row = row0 + r * SPW + sub;
             if (row >= nrows) continue;
             const float inv = 1.0f / s[r];
-            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(drop, ix[r]);
+            const long oa = view_offset_of<FLAT>(alpha, ix[r]), om = view_offset_of<FLAT>(mask, ix[r]), od = view_offset_of<FLAT>(drop, ix[r]);
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * GRP + gl) * 8;
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(BLOCK) void k_softmax(RowSpace rs, View beta, View 
     }
 }
 
-template <int VPL, int RPW, bool FAST, int GRP = WAVE>
+template <int VPL, int RPW, bool FAST, bool FLAT = false, int GRP = WAVE>
 __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask, View ddrop,
                                               View dbeta, float scale, unsigned nrows) {
     constexpr int SPW = WAVE / GRP;
@@ -124,8 +124,8 @@ __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask
         for (int r = 0; r < RPW; ++r) {
             const unsigned row = row0 + r * SPW + sub;
             const bool live = row < nrows;
-            ix[r] = row_index(rs, live ? row : row0);
-            const long oa = view_offset(alpha, ix[r]), om = view_offset(mask, ix[r]), od = view_offset(ddrop, ix[r]);
+            ix[r] = row_index_of<FLAT>(rs, live ? row : row0);
+            const long oa = view_offset_of<FLAT>(alpha, ix[r]), om = view_offset_of<FLAT>(mask, ix[r]), od = view_offset_of<FLAT>(ddrop, ix[r]);
             s[r] = 0.f;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
@@ -145,7 +145,7 @@ __global__ __launch_bounds__(BLOCK) void k_bs(RowSpace rs, View alpha, View mask
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             if (row0 + r * SPW + sub >= nrows) continue;
-            const long oo = view_offset(dbeta, ix[r]);
+            const long oo = view_offset_of<FLAT>(dbeta, ix[r]);
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * GRP + gl) * 8;
@@ -426,7 +426,7 @@ __global__ __launch_bounds__(BLOCK) void k_bdrln_flat(int R, unsigned nrows, Vie
     }
 }
 
-template <int VPL, int RPW, bool FAST>
+template <int VPL, int RPW, bool FAST, bool FLAT = false>
 __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View istd, View diff,
                                                  View mask, View d_ln_in, View d_drop_in, unsigned nrows,
                                                  const uint8_t* mask_bits) {
@@ -441,9 +441,9 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
 #pragma unroll
         for (int r = 0; r < RPW; ++r) {
             const bool live = row0 + r < nrows;
-            ix[r] = row_index(rs, live ? row0 + r : row0);
-            const long oo = view_offset(dout, ix[r]), od = view_offset(diff, ix[r]), om = view_offset(mask, ix[r]);
-            is[r] = (float)istd.p[view_offset(istd, ix[r])];
+            ix[r] = row_index_of<FLAT>(rs, live ? row0 + r : row0);
+            const long oo = view_offset_of<FLAT>(dout, ix[r]), od = view_offset_of<FLAT>(diff, ix[r]), om = view_offset_of<FLAT>(mask, ix[r]);
+            is[r] = (float)istd.p[view_offset_of<FLAT>(istd, ix[r])];
             s1[r] = 0.f; s2[r] = 0.f;
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
@@ -475,7 +475,7 @@ __global__ __launch_bounds__(BLOCK) void k_blnrd(RowSpace rs, View dout, View is
             if (row0 + r >= nrows) continue;
             const float c1 = s1[r] * is[r] * invn;
             const float c2 = s2[r] * is[r] * is[r] * is[r] * invn;
-            const long o1 = view_offset(d_ln_in, ix[r]), o2 = view_offset(d_drop_in, ix[r]);
+            const long o1 = view_offset_of<FLAT>(d_ln_in, ix[r]), o2 = view_offset_of<FLAT>(d_drop_in, ix[r]);
 #pragma unroll
             for (int c = 0; c < VPL; ++c) {
                 int e0 = (c * WAVE + lane) * 8;
@@ -524,6 +524,21 @@ inline unsigned check_rows(const RowSpace& rs, const char* what) {
 // variable of the calling function.)
 #define SUB_ROW_LAUNCH(KERNEL, V, RP, F, ...) \
     hipLaunchKernelGGL((KERNEL<V, RP, F>), dim3(row_grid(nrows, RP) + extra_blocks), dim3(BLOCK), 0, st, __VA_ARGS__)
+#define SUB_ROW_LAUNCH_FLAT(KERNEL, V, RP, ...) \
+    hipLaunchKernelGGL((KERNEL<V, RP, true, true>), dim3(row_grid(nrows, RP) + extra_blocks), dim3(BLOCK), 0, st, __VA_ARGS__)
+// (flat: the fast kernels instantiated for a flat row space, see row_index_of)
+#define SUB_ROW_DISPATCH_FLAT(KERNEL, vpl, ...)                                    \
+    do {                                                                           \
+        const bool many = nrows >= 256u * 16u * 4u;                                \
+        switch (vpl) {                                                             \
+            case 1: if (many) SUB_ROW_LAUNCH_FLAT(KERNEL, 1, 4, __VA_ARGS__);      \
+                    else SUB_ROW_LAUNCH_FLAT(KERNEL, 1, 1, __VA_ARGS__); break;    \
+            case 2: if (many) SUB_ROW_LAUNCH_FLAT(KERNEL, 2, 2, __VA_ARGS__);      \
+                    else SUB_ROW_LAUNCH_FLAT(KERNEL, 2, 1, __VA_ARGS__); break;    \
+            case 4: SUB_ROW_LAUNCH_FLAT(KERNEL, 4, 1, __VA_ARGS__); break;         \
+            default: SUB_ROW_LAUNCH_FLAT(KERNEL, 8, 1, __VA_ARGS__); break;        \
+        }                                                                          \
+    } while (0)
 #define SUB_ROW_DISPATCH(KERNEL, vpl, fast, ...)                                   \
     do {                                                                           \
         if (fast) {                                                                \
@@ -558,7 +573,7 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
     if (fast && rs.R <= 256 && nrows >= 256u * 16u * 4u) {
         // short rows: two or four side by side in every wave
 #define SUB_SM_SHORT(G, RPS, M)                                                                        \
-        hipLaunchKernelGGL((k_softmax<1, 4, true, G, M>), dim3(row_grid(nrows, RPS)), dim3(BLOCK), 0, st, rs, \
+        hipLaunchKernelGGL((k_softmax<1, 4, true, false, G, M>), dim3(row_grid(nrows, RPS)), dim3(BLOCK), 0, st, rs, \
                            beta, alpha, mask, drop, amask, scale, mscale, key, nrows)
         if (rs.R <= 128) { if (masked) SUB_SM_SHORT(16, 16, true); else SUB_SM_SHORT(16, 16, false); }
         else { if (masked) SUB_SM_SHORT(32, 8, true); else SUB_SM_SHORT(32, 8, false); }
@@ -569,7 +584,7 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
     if (masked) {
         // one row per wave; the mask rows are re-read by every head and sample from cache
 #define SUB_SM_MASKED(V, F)                                                                            \
-        hipLaunchKernelGGL((k_softmax<V, 1, F, WAVE, true>), dim3(row_grid(nrows, 1)), dim3(BLOCK), 0, st, rs, \
+        hipLaunchKernelGGL((k_softmax<V, 1, F, false, WAVE, true>), dim3(row_grid(nrows, 1)), dim3(BLOCK), 0, st, rs, \
                            beta, alpha, mask, drop, amask, scale, mscale, key, nrows)
         switch (vpl) {
             case 1: if (fast) SUB_SM_MASKED(1, true); else SUB_SM_MASKED(1, false); break;
@@ -581,7 +596,8 @@ void launch_softmax(const RowSpace& rs, View beta, View alpha, View mask, View d
         check_launch("softmax");
         return;
     }
-    SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
+    if (fast && rs.flat) SUB_ROW_DISPATCH_FLAT(k_softmax, vpl, rs, beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
+    else SUB_ROW_DISPATCH(k_softmax, vpl, fast, rs, beta, alpha, mask, drop, amask, scale, mscale, key, nrows);
     check_launch("softmax");
 }
 
@@ -594,15 +610,16 @@ void launch_bs(const RowSpace& rs, View alpha, View mask, View ddrop, View dbeta
     bool fast = alpha.vec && mask.vec && ddrop.vec && dbeta.vec;
     if (fast && rs.R <= 256 && nrows >= 256u * 16u * 4u) {
         if (rs.R <= 128)
-            hipLaunchKernelGGL((k_bs<1, 4, true, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs, alpha,
+            hipLaunchKernelGGL((k_bs<1, 4, true, false, 16>), dim3(row_grid(nrows, 16)), dim3(BLOCK), 0, st, rs, alpha,
                                mask, ddrop, dbeta, scale, nrows);
         else
-            hipLaunchKernelGGL((k_bs<1, 4, true, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs, alpha,
+            hipLaunchKernelGGL((k_bs<1, 4, true, false, 32>), dim3(row_grid(nrows, 8)), dim3(BLOCK), 0, st, rs, alpha,
                                mask, ddrop, dbeta, scale, nrows);
         check_launch("softmax backward");
         return;
     }
-    SUB_ROW_DISPATCH(k_bs, vpl, fast, rs, alpha, mask, ddrop, dbeta, scale, nrows);
+    if (fast && rs.flat) SUB_ROW_DISPATCH_FLAT(k_bs, vpl, rs, alpha, mask, ddrop, dbeta, scale, nrows);
+    else SUB_ROW_DISPATCH(k_bs, vpl, fast, rs, alpha, mask, ddrop, dbeta, scale, nrows);
     check_launch("softmax backward");
 }
 
@@ -654,7 +671,8 @@ void launch_blnrd(const RowSpace& rs, View dout, View istd, View diff, View mask
     if (nrows == 0) return;
     int vpl = pick_vpl(rs.R, "layernorm backward");
     bool fast = dout.vec && diff.vec && (mask.vec || mask_bits) && d_ln_in.vec && d_drop_in.vec;
-    SUB_ROW_DISPATCH(k_blnrd, vpl, fast, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows, mask_bits);
+    if (fast && rs.flat) SUB_ROW_DISPATCH_FLAT(k_blnrd, vpl, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows, mask_bits);
+    else SUB_ROW_DISPATCH(k_blnrd, vpl, fast, rs, dout, istd, diff, mask, d_ln_in, d_drop_in, nrows, mask_bits);
     check_launch("layernorm backward");
 }
 

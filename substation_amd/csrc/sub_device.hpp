@@ -61,6 +61,18 @@ __device__ __forceinline__ long view_offset(const View& t, const RowIdx& x) {
     return (long)x.i0 * t.s0 + (long)x.i1 * t.s1 + (long)x.i2 * t.s2 + (long)x.i3 * t.s3;
 }
 
+// The same for a kernel instantiated for a flat row space (FLAT: RowSpace::flat, the row is its only
+// index): one multiplication per view in place of three divisions per row and four products per view.
+template <bool FLAT>
+__device__ __forceinline__ RowIdx row_index_of(const RowSpace& rs, unsigned row) {
+    if (FLAT) { RowIdx x; x.i0 = x.i1 = x.i2 = 0; x.i3 = row; return x; }
+    return row_index(rs, row);
+}
+template <bool FLAT>
+__device__ __forceinline__ long view_offset_of(const View& t, const RowIdx& x) {
+    return FLAT ? (long)x.i3 * t.s3 : view_offset(t, x);
+}
+
 // Load 8 row elements e0 .. e0+7 (nvalid of them inside the row) as fp32.
 __device__ __forceinline__ F8 load8(const View& t, long base, int e0, int nvalid, float fill = 0.f) {
     F8 r;
