@@ -24,6 +24,7 @@ struct Chunk {
     RowIdx ix;
 };
 
+template <bool FLAT = false>
 __device__ __forceinline__ Chunk chunk_of(const RowSpace& rs, unsigned idx, unsigned nchunks, unsigned cpr) {
     Chunk c;
     const bool live = idx < nchunks;
@@ -32,11 +33,13 @@ __device__ __forceinline__ Chunk chunk_of(const RowSpace& rs, unsigned idx, unsi
     c.e0 = (int)(id - c.row * cpr) * 8;
     int nv = rs.R - c.e0;
     c.nv = live ? (nv > 8 ? 8 : nv) : 0;
-    c.ix = row_index(rs, c.row);
+    c.ix = row_index_of<FLAT>(rs, c.row);
     return c;
 }
 
-template <bool FAST>
+// ACT, FLAT: the activation and a flat row space as compile-time facts (a choice of activation per element
+// is a branch per element; a strided row space three divisions per pack of 8).
+template <bool FAST, int ACT = -1, bool FLAT = false>
 __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, View lin, View mask,
                                                View out, int act, PhiloxKey key_, unsigned nchunks,
                                                unsigned cpr, int out_only) {
@@ -47,8 +50,8 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
         F8 fi[UNROLL], fb[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            c[u] = chunk_of(rs, base + u * stride, nchunks, cpr);
-            fi[u] = ld8<FAST, true>(in, view_offset(in, c[u].ix), c[u].e0, c[u].nv);
+            c[u] = chunk_of<FLAT>(rs, base + u * stride, nchunks, cpr);
+            fi[u] = ld8<FAST, true>(in, view_offset_of<FLAT>(in, c[u].ix), c[u].e0, c[u].nv);
             fb[u] = ld8<FAST>(bias, 0, c[u].e0, c[u].nv);
         }
 #pragma unroll
@@ -62,14 +65,14 @@ __global__ __launch_bounds__(BLOCK) void k_bad(RowSpace rs, View in, View bias, 
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 float l = (float)lh[i];
-                float a = act == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
+                float a = (ACT < 0 ? act : ACT) == ACT_GELU ? gelu_fwd(l) : fmaxf(l, 0.f);
                 oh[i] = ((bits >> i) & 1u) ? (half_t)a : (half_t)0.0f;
             }
             if (!out_only) {
-                st8h<FAST, true>(lin, view_offset(lin, c[u].ix), c[u].e0, c[u].nv, lh);
-                st8h<FAST, true>(mask, view_offset(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
+                st8h<FAST, true>(lin, view_offset_of<FLAT>(lin, c[u].ix), c[u].e0, c[u].nv, lh);
+                st8h<FAST, true>(mask, view_offset_of<FLAT>(mask, c[u].ix), c[u].e0, c[u].nv, mask_h8(bits));
             }
-            st8h<FAST>(out, view_offset(out, c[u].ix), c[u].e0, c[u].nv, oh);
+            st8h<FAST>(out, view_offset_of<FLAT>(out, c[u].ix), c[u].e0, c[u].nv, oh);
         }
     }
 }
@@ -119,9 +122,13 @@ void launch_bad(const RowSpace& rs, View in, View bias, View lin, View mask, Vie
     unsigned nchunks = check_chunks(rs.rows() * cpr, "bias-activation-dropout");
     if (nchunks == 0) return;
     const bool fast = in.vec && bias.vec && lin.vec && mask.vec && out.vec;
-    if (fast)
-        hipLaunchKernelGGL(k_bad<true>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
-                           mask, out, act, key, nchunks, cpr, out_only ? 1 : 0);
+#define SUB_BAD(...) hipLaunchKernelGGL((k_bad<__VA_ARGS__>), dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin, \
+                                        mask, out, act, key, nchunks, cpr, out_only ? 1 : 0)
+    if (fast && rs.flat && act == ACT_GELU) SUB_BAD(true, ACT_GELU, true);
+    else if (fast && rs.flat) SUB_BAD(true, ACT_RELU, true);
+    else if (fast && act == ACT_GELU) SUB_BAD(true, ACT_GELU, false);
+    else if (fast) SUB_BAD(true, ACT_RELU, false);
+#undef SUB_BAD
     else
         hipLaunchKernelGGL(k_bad<false>, dim3(elem_grid(nchunks)), dim3(BLOCK), 0, st, rs, in, bias, lin,
                            mask, out, act, key, nchunks, cpr, out_only ? 1 : 0);
