@@ -126,7 +126,10 @@ def test_softmax_with_attention_mask(B, L, H, E):
         assert (from_layout(d, 'HBJK', lay) == got * want_mask).all()
 
 
-@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 8, 1, 1024), (1, 4, 1, 4096), (2, 3, 1, 20)])
+# (rows of 1000 and 776 features: the last pack of a lane's two lies outside the row for some lanes;
+# 66000 rows of 64: more rows than the launch has waves, a wave takes several)
+@pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 8, 1, 1024), (1, 4, 1, 4096), (2, 3, 1, 20), (3, 40, 1, 1000),
+                                            (2, 130, 1, 776), (66, 1000, 1, 64)])
 @pytest.mark.parametrize('p', [0.0, 0.3])
 def test_bdrln_and_blnrd(B, L, H, E, p):
     o = _ops(B, L, H, E)
@@ -307,7 +310,9 @@ def test_attention_operator_forward_and_backward(B, H, P, J, K, p, masked, l_q, 
     assert_close(from_layout(dv, 'BKHP', l_kv), want_dv, name='dv')
 
 
-@pytest.mark.parametrize('B,L,H,E', [(2, 128, 4, 512), (4, 64, 1, 1024), (3, 24, 2, 48), (1, 4, 1, 4096)])
+# (1000, 776: rows that end inside a lane's second pack; 5000 rows of 64: more rows than the launch has waves)
+@pytest.mark.parametrize('B,L,H,E', [(2, 128, 4, 512), (4, 64, 1, 1024), (3, 24, 2, 48), (1, 4, 1, 4096),
+                                     (3, 40, 1, 1000), (2, 130, 1, 776), (5, 1000, 1, 64)])
 @pytest.mark.parametrize('extended', [False, True])
 def test_ln_backward_one_launch_or_separate(B, L, H, E, extended):
     """sub_op_ln_backward (bsb + blnrd, or ebsb + blnrd + baob) against the oracle's
