@@ -181,6 +181,7 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
     constexpr bool DROP_SUM = EXT || MOVE;
     constexpr int NR = DROP_SUM ? NS - 1 : NS;    // sums kept in registers
     __shared__ float red[LNF_WPB][VPL * WAVE * 8];
+    __shared__ float red2[LNF_WPB][VPL * WAVE * 8];     // a second set of slabs: two sums per reduction pass
     typedef int i4v __attribute__((ext_vector_type(4)));
     fetch_args_now(R, nrows, a.in.p, a.in.s3, a.d1.p, a.d1.s3, a.diff.p, a.diff.s3, a.istd.p, a.istd.s3, a.scale.p, a.g.p,
                    a.g.s3, a.d_ln_in.p, a.d_ln_in.s3, a.d_drop_in.p, a.d_drop_in.s3, a.write_g, ws);
@@ -304,27 +305,40 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
         }
     }
     // One partial row per block and sum: ws[(s * gridDim.x + block) * R + feature].  The sum of
-    // d_drop_in lies in the slabs already; the others follow from the registers.
-    auto reduce_slabs = [&](int s) {
-        __syncthreads();
+    // d_drop_in lies in the slabs already; the others follow from the registers, through the second
+    // set of slabs and then the first again, two sums per pass.
+    float* const slab2 = &red2[wave][lane * 8];
+    auto put = [&](float* dst, int s) {
+#pragma unroll
+        for (int c = 0; c < VPL; ++c) {
+            *reinterpret_cast<float4*>(dst + c * 512) = make_float4(acc[s][c][0], acc[s][c][1], acc[s][c][2], acc[s][c][3]);
+            *reinterpret_cast<float4*>(dst + c * 512 + 4) = make_float4(acc[s][c][4], acc[s][c][5], acc[s][c][6], acc[s][c][7]);
+        }
+    };
+    auto reduce = [&](const float (*from)[VPL * WAVE * 8], int s) {
         for (int f = threadIdx.x; f < R; f += LNF_BLOCK) {
             float t = 0.f;
 #pragma unroll
-            for (int w = 0; w < LNF_WPB; ++w) t += red[w][f];
+            for (int w = 0; w < LNF_WPB; ++w) t += from[w][f];
             ws[((long)s * gridDim.x + blockIdx.x) * R + f] = t;
         }
     };
-    if (DROP_SUM) reduce_slabs(S_DROP);
-#pragma unroll
-    for (int s = 0; s < NR; ++s) {
+    constexpr int START = DROP_SUM ? 1 : 0;        // register sums that the first pass leaves
+    static_assert(START + 2 >= NR, "one more pass takes the rest");
+    if (DROP_SUM) {
+        put(slab2, 0);
         __syncthreads();
-#pragma unroll
-        for (int c = 0; c < VPL; ++c) {
-            *reinterpret_cast<float4*>(slab + c * 512) = make_float4(acc[s][c][0], acc[s][c][1], acc[s][c][2], acc[s][c][3]);
-            *reinterpret_cast<float4*>(slab + c * 512 + 4) = make_float4(acc[s][c][4], acc[s][c][5], acc[s][c][6], acc[s][c][7]);
-        }
-        // (with MOVE the register sums are 0, 1; without it 0, 1 and for the extended form 2)
-        reduce_slabs(s);
+        reduce(red, S_DROP);
+        reduce(red2, 0);
+    }
+    // (with MOVE the register sums are 0, 1; without it 0, 1 and for the extended form 2)
+    if constexpr (START < NR) {
+        __syncthreads();                           // every wave is done reading both sets
+        put(slab, START);
+        if constexpr (START + 1 < NR) put(slab2, START + 1);
+        __syncthreads();
+        reduce(red, START);
+        if constexpr (START + 1 < NR) reduce(red2, START + 1);
     }
 }
 
