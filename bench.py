@@ -541,6 +541,8 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE readings')
+    ap.add_argument('--activation', choices=['relu', 'gelu'], default=None,
+                    help="the feed-forward activation, instead of the configuration's own (then named in config.workload)")
     ap.add_argument('--decoder', action='store_true',
                     help='time the decoder layer with encoder-decoder attention (both lengths = the '
                          "configuration's L, causal self-attention) instead of the encoder layer; prints its own line")
@@ -558,7 +560,10 @@ def main():
     if args.config == 2:
         bench_fused_ops(args)
         return
-    cfg = CONFIGS[args.config]
+    cfg = dict(CONFIGS[args.config])
+    if args.activation and args.activation != cfg['act']:
+        cfg['act'] = args.activation
+        cfg['name'] += ' [activation: %s]' % args.activation
     if args.decoder:
         bench_decoder(cfg, args)
         return

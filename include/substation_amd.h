@@ -185,7 +185,7 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * other waits.  Results are unchanged.  Profiling names: `dXlin1+dWlin1`,
  * `dXQKV-fused+dWQKV-fused`. */
 #define SUB_OPT_PAIR_PRODUCTS 5
-/* SUB_OPT_RELU_FROM_OUTPUT (default 1; ReLU layers only): the backward pass reads
+/* SUB_OPT_RELU_FROM_OUTPUT (default 1).  ReLU layers: the backward pass reads
  * the gate of dropout and ReLU off the forward output DROP2 = relu(LIN1) * mask,
  * which is positive exactly where the mask kept a positive LIN1
  * (block_bdrlb.cuh:72 reads DROP2MASK and LIN1 for it).  encoder_forward then
@@ -201,6 +201,15 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * handle's latest encoder_forward call wrote and from DROP2 itself otherwise
  * (same results); DDROP2 is not written and DLINB1 sums its terms in another
  * order.
+ * GELU layers, where both products qualify for those epilogues, SUB_OPT_FUSE_EPILOGUES
+ * is on and LIN1, like DROP2, is in BJU order: bias, GELU and dropout run in the
+ * epilogue of lin1, which writes LIN1 (the backward pass needs it) and DROP2 and
+ * leaves the keep bits of the dropout, one per element, in the first B*J*U/8 bytes
+ * of SB1_LINW1 in place of the DROP2MASK tensor; encoder_backward runs bdrlb
+ * (block_bdrlb.cuh:13-146) in the epilogue of dXlin2 from LIN1 and those bits.
+ * DROP2MASK, SB1_LINW1 and DDROP2 are not written; results are bit-identical
+ * (DLINB1 to rounding).  encoder_backward then has to be handed the forward
+ * tensors of the handle's latest encoder_forward call and fails otherwise.
  * Set it to 0 before the forward call when LIN1, DROP2MASK, SB1_LINW1 or
  * DDROP2 are wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6

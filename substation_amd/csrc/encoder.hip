@@ -212,6 +212,9 @@ struct Handle {
     // null: the unused SB1_LINW1 buffer of that call.  The backward call reads its gate from there when it
     // is handed the same buffer, and from DROP2 itself otherwise.
     const void* gate_bits_at = nullptr;
+    // the last forward call ran lin1 with the GELU epilogue: gate_bits_at holds keep bits, no DROP2MASK exists and
+    // the backward call must take the matching epilogue
+    bool gelu_epilogue_ran = false;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
     size_t prof_forward = 0;          // entries of the last forward call, kept by the backward call after it
@@ -662,6 +665,13 @@ void op_bdrlb_from_output(Handle& h, const void* ddrop, const Layout& ld, const 
 
 // Both passes decide this from the handle alone, so they agree.
 bool relu_from_output(const Handle& h) { return h.relu_from_output && h.act == ACT_RELU; }
+// GELU: lin1 with bias, activation and dropout in its epilogue (LIN1 and DROP2 written, the keep bits left in the
+// SB1_LINW1 buffer instead of a DROP2MASK tensor) and dXlin2 with the backward of that in its epilogue.  Both or
+// neither: without DROP2MASK the separate backward operator has nothing to read.
+bool gelu_epilogues(const Handle& h) {
+    return h.relu_from_output && h.act == ACT_GELU && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok &&
+           h.gemm[G_DXLIN2_BDRLB].ok && h.lf[LIN1].str() == "BJU";
+}
 
 void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
@@ -920,13 +930,15 @@ void forward(Handle& h, const FwdPtrs& t) {
     }
     if (!fused_attention) run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
     run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
-    const bool lin1_bad = relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok && aligned16(W[LINB1]) &&
-                          aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]);
+    const bool lin1_gelu = gelu_epilogues(h) && aligned16(F[LIN1]) && F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0;
+    const bool lin1_bad = ((relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok) || lin1_gelu) &&
+                          aligned16(W[LINB1]) && aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]);
+    h.gelu_epilogue_ran = lin1_bad && lin1_gelu;
     // The keep bits of lin1's ReLU-dropout epilogue depend on nothing but seed, step and position:
     // workgroups behind those of bdrln1, a launch that waits for memory with its vector units idle,
     // draw them, into the SB1_LINW1 buffer (unused with that epilogue) behind its B*J*U/8 bytes of gate bits.
     KeepWordsJob keep_job;
-    if (lin1_bad && (h.side_jobs & 2) && aligned16(F[SB1_LINW1])) {
+    if (lin1_bad && !lin1_gelu && (h.side_jobs & 2) && aligned16(F[SB1_LINW1])) {
         const GemmPlan& p = h.gemm[G_LIN1_BAD];
         keep_job.key = make_key(h, SUB_SITE_ACT, h.p_act);
         keep_job.M = (uint32_t)p.shape.M; keep_job.N = (uint32_t)p.shape.N;
@@ -941,7 +953,7 @@ void forward(Handle& h, const FwdPtrs& t) {
                  &keep_job);
     }
     if (lin1_bad) {
-        // product, bias, ReLU and dropout in one launch: SB1_LINW1 (and LIN1, DROP2MASK) are not produced
+        // product, bias, activation and dropout in one launch: SB1_LINW1 and DROP2MASK (ReLU: and LIN1) are not produced
         ProfScope ps(h, "lin1+bad");
         const GemmPlan& p = h.gemm[G_LIN1_BAD];
         GemmEpilogue ep;
@@ -950,6 +962,7 @@ void forward(Handle& h, const FwdPtrs& t) {
         if (keep_job.blocks) ep.keep_words = keep_job.out;
         if (F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0) ep.gate_bits_out = (uint32_t*)F[SB1_LINW1];
         h.gate_bits_at = ep.gate_bits_out;
+        if (lin1_gelu) { ep.act = ACT_GELU; ep.pre_out = (half_t*)F[LIN1]; }
         launch_gemm(p.shape, (const half_t*)F[SB1], (const half_t*)W[LINW1], (half_t*)F[DROP2], p.alpha, ep, h.stream);
     } else {
     h.gate_bits_at = nullptr;
@@ -1032,8 +1045,16 @@ void backward(Handle& h, const BwdPtrs& t) {
                      F[DROP3MASK], h.lf[DROP3MASK], D[DRESID2], h.lb[DRESID2], D[DLIN2], h.lb[DLIN2], packed_masks(h));
         }
     }
-    const bool fuse_bdrlb = relu_from_output(h) && h.fuse_epilogues && h.gemm[G_DXLIN2_BDRLB].ok && aligned16(F[DROP2]) &&
+    const bool bits_here = h.gate_bits_at && h.gate_bits_at == F[SB1_LINW1] &&
+                           h.gemm[G_LIN1_BAD].shape.M == h.gemm[G_DXLIN2_BDRLB].shape.M &&
+                           h.gemm[G_LIN1_BAD].shape.N == h.gemm[G_DXLIN2_BDRLB].shape.N;
+    const bool bdrlb_gelu = h.gelu_epilogue_ran && gelu_epilogues(h) && bits_here && aligned16(F[LIN1]);
+    const bool fuse_bdrlb = ((relu_from_output(h) && h.fuse_epilogues && h.gemm[G_DXLIN2_BDRLB].ok && aligned16(F[DROP2])) ||
+                             bdrlb_gelu) &&
                             aligned16(D[DLIN1]) && aligned16(D[DLIN2]) && aligned16(W[LINW2]);
+    if (h.gelu_epilogue_ran && !fuse_bdrlb)
+        fail("encoder_backward: the forward call ran lin1 with the GELU epilogue (no DROP2MASK was written); the backward "
+             "call needs the same options and forward tensors and 16-byte aligned DLIN1, DLIN2, LINW2, LIN1");
     if (fuse_bdrlb) {
         // product, gate and the column sums of the result in one launch: DDROP2 is not produced
         ProfScope ps(h, "dXlin2+bdrlb");
@@ -1041,10 +1062,9 @@ void backward(Handle& h, const BwdPtrs& t) {
         const int ntc = (int)(p.shape.M / 128), U = (int)p.shape.N;
         float* ws = take_ws(h, (size_t)ntc * U);
         GemmEpilogue ep;
-        ep.gate = (const half_t*)F[DROP2]; ep.sbM = p.sM; ep.sbN = p.sN; ep.colsum = ws;
-        if (h.gate_bits_at && h.gate_bits_at == F[SB1_LINW1] && h.gemm[G_LIN1_BAD].shape.M == p.shape.M &&
-            h.gemm[G_LIN1_BAD].shape.N == p.shape.N)
-            ep.gate_bits = (const uint32_t*)F[SB1_LINW1];
+        ep.gate = (const half_t*)(bdrlb_gelu ? F[LIN1] : F[DROP2]); ep.sbM = p.sM; ep.sbN = p.sN; ep.colsum = ws;
+        if (bits_here) ep.gate_bits = (const uint32_t*)F[SB1_LINW1];
+        if (bdrlb_gelu) ep.act = ACT_GELU;
         launch_gemm(p.shape, (const half_t*)D[DLIN2], (const half_t*)W[LINW2], (half_t*)D[DLIN1], p.alpha, ep, h.stream);
         FinishJob job{ws, FinishArgs{{(half_t*)DW[LINB1], nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};
         if (h.deferring) {

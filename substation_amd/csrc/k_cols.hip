@@ -31,15 +31,6 @@ template <> struct ColTraits<COL_BDRLB> { static constexpr int NS = 1; };
 template <> struct ColTraits<COL_BAOB> { static constexpr int NS = 1; };
 template <> struct ColTraits<COL_BDRLB_OUT> { static constexpr int NS = 1; };
 
-__device__ __forceinline__ float gelu_grad(float x) {
-    const float c = 0.7978845608028654f;
-    float x3 = x * x * x;
-    float u = c * (x + 0.044715f * x3);
-    float t = 1.0f - 2.0f / (1.0f + __expf(2.0f * u));
-    float sech2 = 1.0f - t * t;
-    return 0.5f * t + (1.5f * 0.044715f * c * x3 + 0.5f * c * x) * sech2 + 0.5f;
-}
-
 template <int KIND> struct ColIn;      // which views are read: count and indices into ColArgs::v
 // `nt`: inputs read here for the last time (saved by the forward pass, or the
 // previous launch's output that nothing else consumes): streamed
@@ -95,7 +86,7 @@ __device__ __forceinline__ void col_compute(const ColArgs& a, const RowIdx& ix, 
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             float d = in[0].v[i] * in[1].v[i];
-            float g = a.act == ACT_GELU ? gelu_grad(in[2].v[i]) * d : (in[2].v[i] > 0.f ? d : 0.f);
+            float g = a.act == ACT_GELU ? gelu_bwd(in[2].v[i], d) : (in[2].v[i] > 0.f ? d : 0.f);
             oh[i] = (half_t)g;
         }
         oh = pin(oh);

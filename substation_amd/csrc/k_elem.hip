@@ -11,13 +11,6 @@ namespace {
 constexpr int BLOCK = 256;
 constexpr int UNROLL = 2;
 
-__device__ __forceinline__ float gelu_fwd(float x) {
-    const float c = 0.7978845608028654f;
-    float u = c * (x + 0.044715f * x * x * x);
-    float t = 1.0f - 2.0f / (1.0f + __expf(2.0f * u));   // tanh(u)
-    return 0.5f * x * (1.0f + t);
-}
-
 struct Chunk {
     unsigned row;
     int e0, nv;

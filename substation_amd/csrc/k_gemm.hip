@@ -45,6 +45,8 @@ struct GemmArgs {
     const uint32_t* keep_words = nullptr;  // relu_dropout: the keep bits, drawn ahead (relu_dropout_keep_words)
     uint32_t* gate_bits_out = nullptr;     // relu_dropout: one bit per output, set where it is positive
     const uint32_t* gate_bits = nullptr;   // gate: those bits instead of the values of `gate`
+    int act = ACT_RELU;                    // the activation of relu_dropout / gate (GemmEpilogue::act)
+    half_t* pre_out = nullptr;             // GELU with dropout: where the rounded sum before the activation goes
     // GemmSideJob of the eight-wave asynchronous kernel: workgroups side_first .. gridDim.x - 1 draw
     // the attention keep words of key tiles 0 .. side_tiles_done - 1 of side_rows score rows
     unsigned side_first = 0, side_blocks = 0;
@@ -662,7 +664,11 @@ __device__ __forceinline__ void sched_half_step() {
 // EPI: what the epilogue does after the scaling and the optional addend.  A template
 // parameter so that the plain kernel does not carry the registers of the others.
 // EPI_RELU_DROPOUT_PRE: EPI_RELU_DROPOUT with the keep bits drawn ahead of the launch (GemmEpilogue::keep_words)
-enum { EPI_PLAIN = 0, EPI_RELU_DROPOUT = 1, EPI_GATE_COLSUM = 2, EPI_RELU_DROPOUT_PRE = 3 };
+// EPI_GELU_DROPOUT: as EPI_RELU_DROPOUT with GELU; also stores the rounded sum before the activation
+// (GemmArgs::pre_out, which the backward pass needs) and leaves the keep bits where the ReLU form leaves its gate bits.
+// EPI_GELU_GATE_COLSUM: the backward counterpart: out = keep bit ? gelu'(pre-activation) * product : 0, and column sums.
+enum { EPI_PLAIN = 0, EPI_RELU_DROPOUT = 1, EPI_GATE_COLSUM = 2, EPI_RELU_DROPOUT_PRE = 3, EPI_GELU_DROPOUT = 4,
+       EPI_GELU_GATE_COLSUM = 5 };
 
 template <int TM, int TN, bool AKC, bool BKC, int S, int NW, int EPI = EPI_PLAIN>
 __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
@@ -683,7 +689,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     __shared__ __attribute__((aligned(16))) half_t st2[S > 2 ? STAGE : 8];
     constexpr int L = TA::NV + TB::NV;               // loads per thread per tile
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // (the wave index as a scalar: LDS destinations of the asynchronous loads are then scalar arithmetic)
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, hi = lane >> 5;
 
@@ -712,8 +719,16 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     const unsigned tq = bz / (unsigned)g.nb2;
     const long b2 = bz - tq * (unsigned)g.nb2, b0 = tq / (unsigned)g.nb1, b1 = tq - (unsigned)b0 * (unsigned)g.nb1;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const half_t* pa = g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM;
-    const half_t* pb = g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN;
+    // (the tile pointers are the same for every lane: kept in scalar registers, a load's address is
+    // scalar base + 32-bit lane offset instead of a 64-bit vector addition per load)
+    auto uniform = [](const half_t* p) {
+        const uint64_t v = reinterpret_cast<uint64_t>(p);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+        const uint32_t hi2 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+        return reinterpret_cast<const half_t*>(((uint64_t)hi2 << 32) | lo);
+    };
+    const half_t* pa = uniform(g.A + b0 * g.sAb[0] + b1 * g.sAb[1] + b2 * g.sAb[2] + (long)m0 * g.sAM);
+    const half_t* pb = uniform(g.B + b0 * g.sBb[0] + b1 * g.sBb[1] + b2 * g.sBb[2] + (long)n0 * g.sBN);
 
     const int tiles_per_k1 = g.K1 / BK;
     const int nkt = g.K0 * tiles_per_k1;
@@ -757,12 +772,13 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     // (kb_next & 15); the start is chosen so that the last 16 steps draw packs 0..15 in order.
     constexpr int LPR = 4 * TN;                      // lanes per output row of the wave's slab
     constexpr int RPI = 64 / LPR;                    // rows per store instruction
-    static_assert(EPI != EPI_RELU_DROPOUT || TM * (32 / RPI) == 16, "16 packs of keep bits per lane");
+    constexpr bool DRAWS = EPI == EPI_RELU_DROPOUT || EPI == EPI_GELU_DROPOUT;    // keep bits drawn in the main loop
+    static_assert(!DRAWS || TM * (32 / RPI) == 16, "16 packs of keep bits per lane");
     PhiloxKey rd_key = g.key;
     uint32_t kb[4] = {0u, 0u, 0u, 0u};
     uint64_t kb_group0 = 0;
     int kb_next = 0;
-    if (EPI == EPI_RELU_DROPOUT) {
+    if (DRAWS) {
         rd_key = resolved(g.key);
         const uint64_t row = (uint64_t)(m0 + wm * 32 * TM + lane / LPR);
         kb_group0 = (row * (uint64_t)g.sCM + (uint64_t)(n0 + wn * 32 * TN + (lane % LPR) * 8)) >> 3;
@@ -801,7 +817,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                 if (late) SUB_DMA_ISSUE(nx_);                                                     \
                 __builtin_amdgcn_sched_barrier(0);                                                \
             }                                                                                     \
-            if (NW == 8 && EPI == EPI_RELU_DROPOUT && ks == BK / 16 - 1) {                        \
+            if (NW == 8 && DRAWS && ks == BK / 16 - 1) {                                          \
                 /* the last k-slice shares its issue slots with the keep bits: the fragments of  \
                    the slice before are dead by now, so the draw costs no registers */           \
                 sched_half_step<0, TM * TN, TM * RA_ + TN * RB_>();                               \
@@ -820,9 +836,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                                                                        acc[i][j], 0, 0, 0);       \
         }                                                                                         \
         /* second half: the reads of k-slice 3 between the products of k-slice 2 */               \
-        if constexpr (NW == 8 && EPI != EPI_RELU_DROPOUT)                                         \
+        if constexpr (NW == 8 && !DRAWS)                                                          \
             sched_half_step<0, 2 * TM * TN, TM * RA_ + TN * RB_>();                               \
-        if constexpr (NW == 8 && EPI == EPI_RELU_DROPOUT) sched_mfma_valu<TM * TN, 12>();         \
+        if constexpr (NW == 8 && DRAWS) sched_mfma_valu<TM * TN, 12>();                           \
     } while (0)
 
     // One step: tile kt is complete once at most the L loads of tile kt+1 are
@@ -867,7 +883,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         if (rem >= 1) SUB_DMA_STEP(st0, st2);
         if (rem >= 2) SUB_DMA_STEP(st1, st0);
     }
-    if (EPI == EPI_RELU_DROPOUT)
+    if (DRAWS)
         for (int c = nkt; c < 16; ++c) SUB_DMA_KEEP();        // a contraction shorter than 16 steps
 #undef SUB_DMA_STEP
 #undef SUB_DMA_COMPUTE
@@ -894,6 +910,8 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
     // output shape reads 1/16 of what the outputs themselves would cost it.
     constexpr bool RELU_DROP = EPI == EPI_RELU_DROPOUT || EPI == EPI_RELU_DROPOUT_PRE;
+    constexpr bool GELU_DROP = EPI == EPI_GELU_DROPOUT;
+    constexpr bool GATED = EPI == EPI_GATE_COLSUM || EPI == EPI_GELU_GATE_COLSUM;
     static_assert(EPI == EPI_PLAIN || 32 / RPI == 4, "four packs of 8 outputs per lane and slab");
     const long bits_at = (((long)tile_m * tiles_n + tile_n) * NW + wave) * (TM * 64) + lane;
     if (EPI == EPI_RELU_DROPOUT_PRE) {
@@ -901,7 +919,7 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         kb[0] = w.x; kb[1] = w.y; kb[2] = w.z; kb[3] = w.w;
     }
     uint32_t gbits[TM];
-    if (EPI == EPI_GATE_COLSUM && g.gate_bits) {
+    if (GATED && g.gate_bits) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) gbits[i] = g.gate_bits[bits_at + i * 64];
     }
@@ -918,7 +936,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         constexpr int ADD = decltype(addend_kind)::value;           // 0 none, 1 a bias row, 2 a tensor
         half_t* cp = c_first;
         const half_t* bp = ADD == 2 ? biasb + b_first : nullptr;
-        const half_t* gp = (EPI == EPI_GATE_COLSUM && !g.gate_bits) ? g.gate + b_first : nullptr;
+        // (the GELU form reads the pre-activation values there, and the keep bits besides)
+        const half_t* gp = (EPI == EPI_GELU_GATE_COLSUM || (EPI == EPI_GATE_COLSUM && !g.gate_bits)) ? g.gate + b_first : nullptr;
+        half_t* lp = GELU_DROP ? g.pre_out + (c_first - Cb) : nullptr;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             uint32_t positive = 0;
@@ -968,6 +988,30 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                         }
                     }
                 }
+                if (EPI == EPI_GELU_GATE_COLSUM) {
+                    // the GELU layer's backward-dropout-activation, as the operator computes it
+                    const uint32_t bits = gbits[i] >> (8 * it);
+                    const h8 lin = *reinterpret_cast<const h8*>(gp);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        // (computed for every element and then selected: no branch per element)
+                        const float gv = gelu_bwd((float)lin[e], (float)val[e]);
+                        val[e] = ((bits >> e) & 1u) ? (half_t)gv : (half_t)0.0f;
+                        colsum[e] += (float)val[e];
+                    }
+                }
+                if (GELU_DROP) {
+                    *reinterpret_cast<h8*>(lp) = val;              // the pre-activation, for the backward pass
+                    lp += c_step;
+                    const int c = i * (32 / RPI) + it, byte = 15 - c;
+                    const uint32_t bits = kb[byte >> 2] >> ((byte & 3) * 8);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float gv = gelu_fwd((float)val[e]);       // for every element, then selected: no branches
+                        val[e] = ((bits >> e) & 1u) ? (half_t)gv : (half_t)0.0f;
+                    }
+                    positive |= (bits & 0xffu) << (8 * it);        // here: the keep bits
+                }
                 if (RELU_DROP) {
                     // what the bias-activation-dropout operator does to the rounded sum, with the
                     // same keep bits (the element index is the offset into the dense output):
@@ -984,15 +1028,15 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
                 *reinterpret_cast<h8*>(cp) = val;
                 cp += c_step;
                 if (ADD == 2) bp += b_step;
-                if (EPI == EPI_GATE_COLSUM) gp += b_step;
+                if (GATED) gp += b_step;
             }
-            if (RELU_DROP && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
+            if ((RELU_DROP || GELU_DROP) && g.gate_bits_out) g.gate_bits_out[bits_at + i * 64] = positive;
         }
     };
-    if (!biasb) store_tile(std::integral_constant<int, 0>{});
+    if (GATED || !biasb) store_tile(std::integral_constant<int, 0>{});     // (a gated product has no addend)
     else if (bias_row) store_tile(std::integral_constant<int, 1>{});
     else store_tile(std::integral_constant<int, 2>{});
-    if (EPI == EPI_GATE_COLSUM) {
+    if (GATED) {
         // lanes LPR apart hold the same 8 columns for other rows: add them up, then one fp32
         // row of partial sums per 128-row slab of the output (a finishing launch adds the slabs)
 #pragma unroll
@@ -1076,7 +1120,7 @@ Canon canonicalise(const GemmShape& s, const half_t* A, const half_t* B, half_t*
     a.alpha = alpha; a.bias = ep.bias;
     a.relu_dropout = ep.relu_dropout ? 1 : 0; a.key = ep.key;
     a.gate = ep.gate; a.colsum = ep.colsum; a.gate_bits_out = ep.gate_bits_out; a.gate_bits = ep.gate_bits;
-    a.keep_words = ep.keep_words;
+    a.keep_words = ep.keep_words; a.act = ep.act; a.pre_out = ep.pre_out;
     a.splits = 1; a.partial = nullptr;
     c.ok_c = a.sCN == 1;
     return c;
@@ -1096,6 +1140,9 @@ int pick_kind(const Canon& c, bool& akc, bool& bkc) {
                     al16(a.bias)))
         return 0;
     if (a.gate && !(a.sbN == 1 && mult8(a.sbM) && al16(a.gate) && !a.bias && a.colsum)) return 0;
+    // GELU: the backward form needs the keep bits, the forward form a place for the pre-activation and for those bits
+    if (a.act == ACT_GELU && a.gate && !a.gate_bits) return 0;
+    if (a.act == ACT_GELU && a.relu_dropout && !(a.pre_out && al16(a.pre_out) && a.gate_bits_out && !a.keep_words)) return 0;
     // every 16-byte access must be aligned and whole
     bool ok = mult8(a.N) && mult8(a.sCM) && mult8(a.sCb[0]) && mult8(a.sCb[1]) && mult8(a.sCb[2]);
     ok = ok && mult8(a.sAK0) && mult8(a.sAb[0]) && mult8(a.sAb[1]) && mult8(a.sAb[2]);
@@ -1143,7 +1190,9 @@ void launch_dma2(const GemmArgs& a, bool akc, bool bkc, dim3 grid, hipStream_t s
     if (a.relu_dropout || a.gate) {
         // only the eight-wave 256x256 kernel carries these epilogues
         if constexpr (NW == 8) {
-            if (a.gate) launch_dma3<TM, TN, S, NW, EPI_GATE_COLSUM>(a, akc, bkc, grid, st);
+            if (a.gate && a.act == ACT_GELU) launch_dma3<TM, TN, S, NW, EPI_GELU_GATE_COLSUM>(a, akc, bkc, grid, st);
+            else if (a.gate) launch_dma3<TM, TN, S, NW, EPI_GATE_COLSUM>(a, akc, bkc, grid, st);
+            else if (a.act == ACT_GELU) launch_dma3<TM, TN, S, NW, EPI_GELU_DROPOUT>(a, akc, bkc, grid, st);
             else if (a.keep_words) launch_dma3<TM, TN, S, NW, EPI_RELU_DROPOUT_PRE>(a, akc, bkc, grid, st);
             else launch_dma3<TM, TN, S, NW, EPI_RELU_DROPOUT>(a, akc, bkc, grid, st);
             return;

@@ -330,4 +330,47 @@ __device__ __forceinline__ h8 mask_h8(uint32_t bits) {
     return m;
 }
 
+// tanh-form GELU (substation/transformer.py:11-28) written through the logistic function:
+// 0.5 x (1 + tanh(u)) = x s(2u) with u = sqrt(2/pi) (x + 0.044715 x^3), s(z) = e^z / (1 + e^z), and
+// its derivative s + x s (1 - s) d(2u)/dx.  One v_exp_f32 and one v_rcp_f32 per value.  The order
+// of the operations is fixed (no contraction left to the compiler), so that the operator kernels
+// and the epilogues of the contractions give the same bits.
+struct GeluTerms {
+    float s, r;                   // s(2u) and 1 - s(2u)
+};
+
+__device__ __forceinline__ GeluTerms gelu_terms(float x, float x2) {
+#pragma clang fp contract(off)
+    const float k0 = 2.302208198144325f;             // 2 sqrt(2/pi) log2(e)
+    const float k1 = 0.1029432395800235f;           // k0 * 0.044715
+    float w = x * __builtin_fmaf(x2, k1, k0);        // 2u log2(e)
+    w = fminf(w, 64.0f);                             // e^z stays finite: s = 1 from there on anyway
+    const float e = __builtin_amdgcn_exp2f(w);
+    GeluTerms t;
+    t.r = __builtin_amdgcn_rcpf(1.0f + e);
+    t.s = e * t.r;
+    return t;
+}
+
+// (The results pass through a register as fp32: a conversion to fp16 that follows rounds that value,
+// whereas fused with the last multiplication into one instruction it would round the exact product.)
+__device__ __forceinline__ float gelu_fwd(float x) {
+#pragma clang fp contract(off)
+    float g = x * gelu_terms(x, x * x).s;
+    asm volatile("" : "+v"(g));
+    return g;
+}
+
+// gelu'(x) * d
+__device__ __forceinline__ float gelu_bwd(float x, float d) {
+#pragma clang fp contract(off)
+    const float x2 = x * x;
+    const GeluTerms t = gelu_terms(x, x2);
+    const float zp = __builtin_fmaf(x2, 0.21406444881780073f, 1.5957691216057308f);   // d(2u)/dx
+    const float q = (x * zp) * t.r;
+    float g = __builtin_fmaf(t.s, q, t.s) * d;
+    asm volatile("" : "+v"(g));
+    return g;
+}
+
 }  // namespace sub

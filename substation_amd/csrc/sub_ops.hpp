@@ -205,6 +205,12 @@ struct GemmEpilogue {
     // relu_dropout: the keep bits drawn ahead by a KeepWordsJob with the same key, M and N; without
     // them the kernel draws them itself during the contraction
     const uint32_t* keep_words = nullptr;
+    // The activation of relu_dropout and gate.  ACT_GELU: relu_dropout computes keep ? gelu(x) : 0, also
+    // stores x (the rounded sum with its addend, which the backward pass needs) to `pre_out`, laid out
+    // like C, and writes the keep bits to gate_bits_out (both required; no keep_words); gate computes
+    // keep ? gelu'(gate) * x : 0 with `gate` the pre-activation values and gate_bits those keep bits (required).
+    int act = ACT_RELU;
+    half_t* pre_out = nullptr;
 };
 // Work that needs no memory path, offered to a product whose 256x256 tiles leave CUs idle: the
 // keep bits of the attention dropout (attention_keep_word) for the first `tiles_done` key tiles of

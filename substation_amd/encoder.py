@@ -40,7 +40,8 @@ class Encoder(torch.nn.Module):
         """``compact_activation``: with ReLU the backward pass reads its gate off the
         dropout output, so the pre-activation LIN1 and DROP2MASK are neither written
         nor read; allocate 8 elements for each instead of B*L*4E (at B=8 L=512
-        E=1024: 64 MiB less per layer call).  ``persistent_workspace``: the intermediates are allocated once and reused
+        E=1024: 64 MiB less per layer call; GELU layers need LIN1 and ignore the
+        request).  ``persistent_workspace``: the intermediates are allocated once and reused
         by every call instead of 37 ``torch.empty`` per iteration
         (pytorch_module/encoder.py:78-85,113-119); a forward call then overwrites
         what an earlier forward call saved for its backward pass, which backward()

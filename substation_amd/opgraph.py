@@ -25,7 +25,7 @@ OPERATORS = [
     ('out', 'fwd', ('WO', 'GAMMA', 'ATT')),
     ('bdrln1', 'fwd', ('ATT', 'X', 'DROP1MASK', 'LN1DIFF', 'LN1', 'SB1', 'LN1STD')),
     ('lin1', 'fwd', ('SB1', 'LINW1', 'SB1_LINW1')),
-    ('lin1+bad', 'fwd', ('SB1', 'LINW1', 'DROP2')),
+    ('lin1+bad', 'fwd', ('SB1', 'LINW1', 'DROP2', 'LIN1')),                   # LIN1: GELU layers only
     ('bad', 'fwd', ('SB1_LINW1', 'LIN1', 'DROP2MASK', 'DROP2')),
     ('lin2', 'fwd', ('DROP2', 'LINW2', 'DROP2_LINW2')),
     ('bdrln2', 'fwd', ('DROP2_LINW2', 'SB1', 'LIN2', 'DROP3MASK', 'LN2DIFF', 'LN2', 'SB2', 'LN2STD')),
@@ -34,7 +34,7 @@ OPERATORS = [
     ('blnrd1', 'bwd', ('DLN2', 'LN2STD', 'LN2DIFF', 'DROP3MASK', 'DRESID2', 'DLIN2')),
     ('dXlin2', 'bwd', ('DLIN2', 'LINW2', 'DDROP2')),
     ('dWlin2', 'bwd', ('DLIN2', 'DROP2', 'LINW2')),
-    ('dXlin2+bdrlb', 'bwd', ('DLIN2', 'LINW2', 'DROP2', 'DLIN1')),
+    ('dXlin2+bdrlb', 'bwd', ('DLIN2', 'LINW2', 'DROP2', 'LIN1', 'DLIN1')),    # GELU: LIN1 and keep bits, not DROP2
     ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DROP2', 'DLIN1')),      # ReLU: the gate is read off DROP2
     ('dXlin1+dWlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1', 'SB1')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),

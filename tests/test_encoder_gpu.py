@@ -215,17 +215,21 @@ def test_bench_path_matches_the_oracle(dims, which):
     _compare(want, got, names=OUTPUTS)
 
 
-@pytest.mark.parametrize('dims', [(96, 128, 4, 256),      # contraction of lin1: 4 steps of 64
-                                  (5, 512, 20, 1280),     # 20 steps
-                                  (3, 512, 36, 2304)])    # 36 steps
-def test_relu_dropout_epilogue_over_short_and_long_contractions(dims):
-    """lin1 with bias, ReLU and dropout in its epilogue draws the keep bits during the
+@pytest.mark.parametrize('dims,act', [((96, 128, 4, 256), 'relu'),      # contraction of lin1: 4 steps of 64
+                                      ((5, 512, 20, 1280), 'relu'),     # 20 steps
+                                      ((3, 512, 36, 2304), 'relu'),     # 36 steps
+                                      # GELU takes the epilogues only where dXlin2 qualifies as well (tiles for 0.9 of the CUs)
+                                      ((128, 128, 4, 256), 'gelu'), ((6, 512, 20, 1280), 'gelu')])
+def test_activation_dropout_epilogue_over_short_and_long_contractions(dims, act):
+    """lin1 with bias, activation and dropout in its epilogue draws the keep bits during the
     contraction, one pack per step of 64 and 16 packs per lane: contractions of fewer
-    than 16 steps, of 16 (the benchmark's) and of more, not a multiple of 16.  The
-    helper also checks that DROP2 is zero exactly where the seeded mask drops."""
+    than 16 steps, of 16 (the benchmark's) and of more, not a multiple of 16.  With ReLU the
+    helper also checks that DROP2 is zero exactly where the seeded mask drops; with GELU
+    the backward pass reads the keep bits the epilogue left, so a wrong bit shows in DX
+    and the gradients."""
     launches = []
-    want, got = run_layer_default(*dims, 0.1, seed_data=23, w_std=0.02, act='relu', launches=launches)
-    assert 'lin1+bad' in launches, launches
+    want, got = run_layer_default(*dims, 0.1, seed_data=23, w_std=0.02, act=act, launches=launches)
+    assert 'lin1+bad' in launches and (act == 'relu' or 'dXlin2+bdrlb' in launches), launches
     _compare(want, got, names=OUTPUTS)
 
 
@@ -638,17 +642,23 @@ def test_compact_attention_buffers_give_the_same_results_and_refuse_a_fallback()
         enc(X)
 
 
-@pytest.mark.parametrize('dims', [(2, 256, 4, 256), (8, 512, 16, 1024),
-                                  (15, 256, 8, 512, 4352),      # 15 x 17 tiles of 256 x 256: odd counts both ways
-                                  (16, 512, 8, 512, 2048)])     # 32 x 8 tiles
-def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
+@pytest.mark.parametrize('dims,activation', [
+    ((2, 256, 4, 256), 'relu'), ((8, 512, 16, 1024), 'relu'),
+    ((15, 256, 8, 512, 4352), 'relu'),      # 15 x 17 tiles of 256 x 256: odd counts both ways
+    ((16, 512, 8, 512, 2048), 'relu'),      # 32 x 8 tiles
+    ((2, 256, 4, 256), 'gelu'),             # too few tiles for the epilogues: the operators either way
+    ((8, 512, 16, 1024), 'gelu'), ((15, 256, 8, 512, 4352), 'gelu')])
+def test_relu_gate_from_the_forward_output_is_bit_identical(dims, activation):
     """ReLU layers (the default of the module, as in the reference) read the gate
     of dropout and ReLU in the backward pass off DROP2 = relu(LIN1) * mask, which
     is positive exactly where the mask kept a positive LIN1; LIN1 and DROP2MASK are
     then neither written nor read, and the two operators run in the epilogues of
     the products before them.  Output and every gradient must equal, bit for bit,
     those with the option off (block_bdrlb.cuh:72: gate from DROP2MASK and LIN1);
-    the bias gradient that is a column sum over 4096 terms agrees to rounding."""
+    the bias gradient that is a column sum over 4096 terms agrees to rounding.
+    GELU layers under the same option: the two operators run in those epilogues as
+    well, with LIN1 written for the backward pass and the keep bits in place of
+    DROP2MASK; the same equalities must hold."""
     from substation_amd import Encoder, layouts as L
     lay = L.mi355x_layouts()
     B, Ls, H, E = dims[:4]
@@ -657,7 +667,7 @@ def test_relu_gate_from_the_forward_output_is_bit_identical(dims):
     for from_output in (0, 1):
         torch.manual_seed(0)
         enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
-                      intermediate_size=U).cuda()
+                      intermediate_size=U, activation=activation).cuda()
         enc._handle.set_option(6, from_output)
         enc.set_rng(SEED, 0)
         g = torch.Generator().manual_seed(5)
