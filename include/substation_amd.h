@@ -208,8 +208,9 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * of SB1_LINW1 in place of the DROP2MASK tensor; encoder_backward runs bdrlb
  * (block_bdrlb.cuh:13-146) in the epilogue of dXlin2 from LIN1 and those bits.
  * DROP2MASK, SB1_LINW1 and DDROP2 are not written; results are bit-identical
- * (DLINB1 to rounding).  encoder_backward then has to be handed the forward
- * tensors of the handle's latest encoder_forward call and fails otherwise.
+ * (DLINB1 to rounding).  encoder_backward knows from the options and the pointers
+ * it is handed, which are the forward call's, that the bits lie in SB1_LINW1:
+ * the option must not change between a forward call and its backward call.
  * Set it to 0 before the forward call when LIN1, DROP2MASK, SB1_LINW1 or
  * DDROP2 are wanted (debug capture). */
 #define SUB_OPT_RELU_FROM_OUTPUT 6

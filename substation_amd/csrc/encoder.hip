@@ -212,9 +212,6 @@ struct Handle {
     // null: the unused SB1_LINW1 buffer of that call.  The backward call reads its gate from there when it
     // is handed the same buffer, and from DROP2 itself otherwise.
     const void* gate_bits_at = nullptr;
-    // the last forward call ran lin1 with the GELU epilogue: gate_bits_at holds keep bits, no DROP2MASK exists and
-    // the backward call must take the matching epilogue
-    bool gelu_epilogue_ran = false;
     std::vector<ProfEntry> prof;
     size_t prof_used = 0;
     size_t prof_forward = 0;          // entries of the last forward call, kept by the backward call after it
@@ -672,6 +669,13 @@ bool gelu_epilogues(const Handle& h) {
     return h.relu_from_output && h.act == ACT_GELU && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok &&
            h.gemm[G_DXLIN2_BDRLB].ok && h.lf[LIN1].str() == "BJU";
 }
+// What the forward call adds to that from the tensors it is handed.  The backward call is handed the same ones and
+// asks the same question: it knows from the handle's options and these pointers alone whether the keep bits of
+// the forward call it belongs to lie in SB1_LINW1 (whichever forward call of the handle that was).
+bool lin1_takes_gelu_epilogue(const Handle& h, void* const* W, void* const* F) {
+    return gelu_epilogues(h) && aligned16(F[LIN1]) && F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0 &&
+           aligned16(W[LINB1]) && aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]);
+}
 
 void op_baob(Handle& h, const void* datt, const Layout& l, void* dbo) {
     Space sp = make_space(h.sz, {dB, dJ}, dI);
@@ -930,10 +934,9 @@ void forward(Handle& h, const FwdPtrs& t) {
     }
     if (!fused_attention) run_gemm(h, G_GAMMA, VV, F[ATTN_DROP], F[GAMMA], "gamma");
     run_gemm(h, G_OUT, W[WO], F[GAMMA], F[ATT], "out");
-    const bool lin1_gelu = gelu_epilogues(h) && aligned16(F[LIN1]) && F[SB1_LINW1] && ((uintptr_t)F[SB1_LINW1] & 3) == 0;
-    const bool lin1_bad = ((relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok) || lin1_gelu) &&
-                          aligned16(W[LINB1]) && aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]);
-    h.gelu_epilogue_ran = lin1_bad && lin1_gelu;
+    const bool lin1_gelu = lin1_takes_gelu_epilogue(h, W, F);
+    const bool lin1_bad = lin1_gelu || (relu_from_output(h) && h.fuse_epilogues && h.gemm[G_LIN1_BAD].ok &&
+                                        aligned16(W[LINB1]) && aligned16(F[DROP2]) && aligned16(F[SB1]) && aligned16(W[LINW1]));
     // The keep bits of lin1's ReLU-dropout epilogue depend on nothing but seed, step and position:
     // workgroups behind those of bdrln1, a launch that waits for memory with its vector units idle,
     // draw them, into the SB1_LINW1 buffer (unused with that epilogue) behind its B*J*U/8 bytes of gate bits.
@@ -1048,13 +1051,13 @@ void backward(Handle& h, const BwdPtrs& t) {
     const bool bits_here = h.gate_bits_at && h.gate_bits_at == F[SB1_LINW1] &&
                            h.gemm[G_LIN1_BAD].shape.M == h.gemm[G_DXLIN2_BDRLB].shape.M &&
                            h.gemm[G_LIN1_BAD].shape.N == h.gemm[G_DXLIN2_BDRLB].shape.N;
-    const bool bdrlb_gelu = h.gelu_epilogue_ran && gelu_epilogues(h) && bits_here && aligned16(F[LIN1]);
+    const bool bdrlb_gelu = lin1_takes_gelu_epilogue(h, W, F);       // the forward call's own test: its keep bits lie in SB1_LINW1
     const bool fuse_bdrlb = ((relu_from_output(h) && h.fuse_epilogues && h.gemm[G_DXLIN2_BDRLB].ok && aligned16(F[DROP2])) ||
                              bdrlb_gelu) &&
                             aligned16(D[DLIN1]) && aligned16(D[DLIN2]) && aligned16(W[LINW2]);
-    if (h.gelu_epilogue_ran && !fuse_bdrlb)
-        fail("encoder_backward: the forward call ran lin1 with the GELU epilogue (no DROP2MASK was written); the backward "
-             "call needs the same options and forward tensors and 16-byte aligned DLIN1, DLIN2, LINW2, LIN1");
+    if (bdrlb_gelu && !fuse_bdrlb)
+        fail("encoder_backward: the forward call ran lin1 with the GELU epilogue (no DROP2MASK was written), and its "
+             "backward epilogue needs 16-byte aligned DLIN1, DLIN2 and LINW2");
     if (fuse_bdrlb) {
         // product, gate and the column sums of the result in one launch: DDROP2 is not produced
         ProfScope ps(h, "dXlin2+bdrlb");
@@ -1063,7 +1066,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         float* ws = take_ws(h, (size_t)ntc * U);
         GemmEpilogue ep;
         ep.gate = (const half_t*)(bdrlb_gelu ? F[LIN1] : F[DROP2]); ep.sbM = p.sM; ep.sbN = p.sN; ep.colsum = ws;
-        if (bits_here) ep.gate_bits = (const uint32_t*)F[SB1_LINW1];
+        if (bits_here || bdrlb_gelu) ep.gate_bits = (const uint32_t*)F[SB1_LINW1];
         if (bdrlb_gelu) ep.act = ACT_GELU;
         launch_gemm(p.shape, (const half_t*)D[DLIN2], (const half_t*)W[LINW2], (half_t*)D[DLIN1], p.alpha, ep, h.stream);
         FinishJob job{ws, FinishArgs{{(half_t*)DW[LINB1], nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};

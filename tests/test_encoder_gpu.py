@@ -797,13 +797,16 @@ def test_compact_activation_buffers_give_the_same_results_and_refuse_the_other_g
     assert ys[0][2] < ys[1][2] - 2 * 2 * (B * Ls * 4 * E * 2 - 16)
 
 
-def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to():
+@pytest.mark.parametrize('activation', ['relu', 'gelu'])
+def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to(activation):
     """With lin1's fused epilogue the forward call leaves one bit per element of DROP2
     (positive or not) in the unused SB1_LINW1 buffer, and the backward call takes its
     ReLU gate from there -- but only from the buffer the latest forward call wrote.
     A backward pass that belongs to an earlier forward call (here: two forward calls,
     then the backward pass of the first) must read the gate off its own DROP2 and
-    give what a forward-backward sequence without the second call gives, bit for bit."""
+    give what a forward-backward sequence without the second call gives, bit for bit.
+    GELU: the bits are the dropout's keep bits and the only copy of them; the backward
+    pass of the first call must find them in the buffers of the first call."""
     from substation_amd import Encoder, layouts as L
     lay = L.mi355x_layouts()
     B, Ls, H, E = 128, 128, 4, 256          # 256 tiles of 256x256: both products take the kernel that carries the epilogues
@@ -811,7 +814,7 @@ def test_relu_gate_comes_from_the_buffers_of_the_forward_call_it_belongs_to():
     def make():
         torch.manual_seed(0)
         enc = Encoder('unused', B, Ls, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, seed=SEED,
-                      profiling=True).cuda()
+                      profiling=True, activation=activation).cuda()
         with torch.no_grad():
             for p in enc.parameters():
                 p.mul_(0.1)
