@@ -795,6 +795,29 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
         ++kb_next;                                                                                \
     } while (0)
 
+    // What the epilogue reads besides the accumulators is requested here, ahead of the contraction: behind it the
+    // round trip to memory would stand in the open (the loads complete in order, ahead of the tiles').
+    half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
+    const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
+    // a bias row (the same for every row of the output): a lane's 8 columns are the same in all of its
+    // packs, so it loads them once instead of before every store
+    const bool bias_row = biasb && g.sbM == 0;
+    h8 bias8 = (h8)(half_t)0.0f;
+    if (bias_row) bias8 = *reinterpret_cast<const h8*>(biasb + n0 + wn * 32 * TN + (lane % LPR) * 8);
+    // One bit per output of the ReLU-dropout epilogue (set = positive), a dword per lane and 32-row
+    // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
+    // output shape reads 1/16 of what the outputs themselves would cost it.
+    constexpr bool RELU_DROP = EPI == EPI_RELU_DROPOUT || EPI == EPI_RELU_DROPOUT_PRE;
+    constexpr bool GELU_DROP = EPI == EPI_GELU_DROPOUT;
+    constexpr bool GATED = EPI == EPI_GATE_COLSUM || EPI == EPI_GELU_GATE_COLSUM;
+    static_assert(EPI == EPI_PLAIN || 32 / RPI == 4, "four packs of 8 outputs per lane and slab");
+    const long bits_at = (((long)tile_m * tiles_n + tile_n) * NW + wave) * (TM * 64) + lane;
+    uint32_t gbits[TM];
+    if (GATED && g.gate_bits) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) gbits[i] = g.gate_bits[bits_at + i * 64];
+    }
+
     constexpr int RA_ = AKC ? 1 : 2, RB_ = BKC ? 1 : 2;      // LDS reads per fragment
     const int fbase_a = TA::frag_base(wm * TM * 32, lane), fbase_b = TB::frag_base(wn * TN * 32, lane);
 #define SUB_DMA_FRAG_A(i_, ks_) (AKC && NW == 8 ? TA::frag_at(sA, ba_, i_, ks_) : TA::frag(sA, (wm * TM + (i_)) * 32, ks_, lane))
@@ -899,29 +922,9 @@ __global__ __launch_bounds__(NW * 64) void k_gemm_dma(GemmArgs g) {
     float colsum[8];              // gate mode: this lane's 8 columns summed over its rows of the wave's slab
 #pragma unroll
     for (int e = 0; e < 8; ++e) colsum[e] = 0.f;
-    half_t* Cb = g.C + b0 * g.sCb[0] + b1 * g.sCb[1] + b2 * g.sCb[2];
-    const half_t* biasb = g.bias ? g.bias + b0 * g.sbb[0] + b1 * g.sbb[1] + b2 * g.sbb[2] : nullptr;
-    // a bias row (the same for every row of the output): a lane's 8 columns are the same in all of its
-    // packs, so it loads them once instead of before every store
-    const bool bias_row = biasb && g.sbM == 0;
-    h8 bias8 = (h8)(half_t)0.0f;
-    if (bias_row) bias8 = *reinterpret_cast<const h8*>(biasb + n0 + wn * 32 * TN + (lane % LPR) * 8);
-    // One bit per output of the ReLU-dropout epilogue (set = positive), a dword per lane and 32-row
-    // slab in the order this epilogue walks the tile: the gate epilogue of a product with the same
-    // output shape reads 1/16 of what the outputs themselves would cost it.
-    constexpr bool RELU_DROP = EPI == EPI_RELU_DROPOUT || EPI == EPI_RELU_DROPOUT_PRE;
-    constexpr bool GELU_DROP = EPI == EPI_GELU_DROPOUT;
-    constexpr bool GATED = EPI == EPI_GATE_COLSUM || EPI == EPI_GELU_GATE_COLSUM;
-    static_assert(EPI == EPI_PLAIN || 32 / RPI == 4, "four packs of 8 outputs per lane and slab");
-    const long bits_at = (((long)tile_m * tiles_n + tile_n) * NW + wave) * (TM * 64) + lane;
     if (EPI == EPI_RELU_DROPOUT_PRE) {
         const uint4 w = reinterpret_cast<const uint4*>(g.keep_words)[(((long)tile_m * tiles_n + tile_n) * NW + wave) * 64 + lane];
         kb[0] = w.x; kb[1] = w.y; kb[2] = w.z; kb[3] = w.w;
-    }
-    uint32_t gbits[TM];
-    if (GATED && g.gate_bits) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) gbits[i] = g.gate_bits[bits_at + i * 64];
     }
     // The lane's stores walk down the tile RPI rows at a time: running pointers (a 64-bit product
     // per store otherwise), and one copy of the loop per kind of addend (none, a bias row, a tensor:
