@@ -351,6 +351,15 @@ int sub_op_bdrlb(void* handle, const void* ddrop, const char* l_ddrop, const voi
                  const char* l_dlinear, void* dbias);
 /* block_baob.cuh:79-97 */
 int sub_op_baob(void* handle, const void* datt, const char* l_datt, void* dbo);
+/* Operator calls between sub_ops_defer(h, 1) and sub_ops_defer(h, 0) leave the second
+ * stage of their column sums (bsb, ebsb, bdrlb, baob, ln_backward: the bias and
+ * scale gradients) to one launch that sub_ops_defer(h, 0) issues, as
+ * encoder_backward does for its own (encoder.cu:158-299 has one kernel per
+ * reduction; no counterpart there).  The gradient vectors are complete only after
+ * that call; same bits as without.  When the list (6 entries) or the scratch buffer
+ * is full, what is on the list is finished early.  encoder_backward refuses to run
+ * in between. */
+int sub_ops_defer(void* handle, int on);
 /* block_aib.cuh:64-155, on the Q-stacked tensors */
 int sub_op_aib(void* handle, const void* in, const char* l_in, const void* bias, const char* l_bias,
                void* out, const char* l_out);
@@ -405,6 +414,16 @@ int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, c
  * substation/transformer.py:41-52 with its bias), or a product added to a residual
  * (block_bei.cuh:12-106).  T may be C (accumulate in place).  Fails when the layouts
  * lead to a kernel that has no epilogue. */
+/* Two independent contractions, the first with an optional addend T1 (null: none) as
+ * in sub_op_einsum_add, in one launch where the pair qualifies (a data gradient and the
+ * weight gradient next to it, as encoder_backward pairs dXlin1 with dWlin1 and dXQKV with
+ * dWQKV: gemm.cuh:134-147 twice, encoder.cu:235-239,268-276), else one after the other;
+ * *paired (optional) says which.  Same results either way.  Neither output may be an
+ * input of the other product. */
+int sub_op_einsum_pair(void* handle, const void* A1, const char* l_A1, const void* B1, const char* l_B1,
+                       const void* T1, const char* l_T1, void* C1, const char* l_C1, float alpha1,
+                       const void* A2, const char* l_A2, const void* B2, const char* l_B2, void* C2,
+                       const char* l_C2, float alpha2, int* paired);
 int sub_op_einsum_add(void* handle, const void* A, const char* l_A, const void* B, const char* l_B,
                       const void* T, const char* l_T, void* C, const char* l_C, float alpha);
 

@@ -62,6 +62,7 @@ SIGNATURES = {
     'sub_set_rng_counter': (_I, [_VP, _VP]),
     'sub_last_error': (_CP, []),
     'sub_set_option': (_I, [_VP, _I, _I]),
+    'sub_ops_defer': (_I, [_VP, _I]),
     'sub_get_option': (_I, [_VP, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
     'sub_attention_in_registers': (_I, [_VP, ctypes.POINTER(_I)]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
@@ -93,6 +94,8 @@ SIGNATURES = {
                                        _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
     'sub_op_einsum': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_einsum_add': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
+    'sub_op_einsum_pair': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F,
+                                _VP, _CP, _VP, _CP, _VP, _CP, _F, ctypes.POINTER(ctypes.c_int)]),
     'sub_layout_strides': (_I, [_VP, _CP, ctypes.POINTER(ctypes.c_int64)]),
     'sub_einsum_classify': (_I, [_VP, _CP, _CP, _CP, ctypes.POINTER(ctypes.c_int64)]),
     'sub_philox_fields_host': (_I, [_U64, _U32, _U32, _U64, _U64, ctypes.POINTER(ctypes.c_uint16)]),
@@ -191,6 +194,10 @@ class Handle:
     def set_attention_mask(self, device_ptr, layout='JK'):
         check(self.lib.sub_set_attention_mask(self.ptr, ctypes.c_void_p(device_ptr or 0), layout.encode()),
               'sub_set_attention_mask')
+
+    def defer_column_sums(self, on):
+        """sub_ops_defer: between on=True and on=False the operators' column sums are finished by one launch."""
+        check(self.lib.sub_ops_defer(self.ptr, 1 if on else 0), 'sub_ops_defer')
 
     def set_option(self, option, value):
         check(self.lib.sub_set_option(self.ptr, option, value), 'sub_set_option')

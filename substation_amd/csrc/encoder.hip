@@ -186,6 +186,7 @@ struct Handle {
     size_t ws_need_bwd = 0;       // sum over the backward pass's column reductions
     float* static_ws = nullptr;   // set for the duration of a call that must not allocate: take_ws hands it out
     bool deferring = false;       // backward pass: finish all column reductions in one launch
+    bool ops_deferring = false;   // the same across operator calls, between sub_ops_defer(h, 1) and sub_ops_defer(h, 0)
     size_t ws_cursor = 0;
     FinishJobs deferred;
     float* gws = nullptr;         // split-k partials of the small-output contractions
@@ -317,12 +318,21 @@ float* take_ws(Handle& h, size_t floats) {
         ensure_ws(h, floats);
         return h.ws;
     }
-    if (h.ws_cursor + floats > h.ws_floats) fail("column-reduction workspace exhausted");
+    if (h.ws_cursor + floats > h.ws_floats) {
+        // Out of room (operator calls that defer size nothing ahead): finish what is on the list, whose
+        // partials the stream has complete by then, and start over at the front of the buffer.
+        if (!h.ops_deferring) fail("column-reduction workspace exhausted");
+        if (h.deferred.n > 0) launch_colfinish(h.deferred, h.stream);
+        h.deferred.n = 0;
+        h.ws_cursor = 0;
+        ensure_ws(h, floats);
+    }
     float* p = h.ws + h.ws_cursor;
     h.ws_cursor += (floats + 63) & ~(size_t)63;
     return p;
 }
-FinishJobs* defer_of(Handle& h) { return h.deferring ? &h.deferred : nullptr; }
+// (a call on the static scratch array has one region for all its reductions: nothing is put off there)
+FinishJobs* defer_of(Handle& h) { return h.deferring && !h.static_ws ? &h.deferred : nullptr; }
 
 // ---------------------------------------------------------------------------
 // Configuration
@@ -1003,6 +1013,7 @@ void backward(Handle& h, const BwdPtrs& t) {
     // at the end of the pass finishes them all (or workgroups of the last pair of
     // products do).  Per-operator timing times this same schedule: the finishing
     // stage is part of the launch that carries it, or an entry of its own.
+    if (h.ops_deferring) fail("encoder_backward: column sums are being deferred across operator calls (sub_ops_defer)");
     ensure_ws(h, h.ws_need_bwd);
     h.deferring = true;
     h.ws_cursor = 0;
@@ -1070,13 +1081,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         if (bdrlb_gelu) ep.act = ACT_GELU;
         launch_gemm(p.shape, (const half_t*)D[DLIN2], (const half_t*)W[LINW2], (half_t*)D[DLIN1], p.alpha, ep, h.stream);
         FinishJob job{ws, FinishArgs{{(half_t*)DW[LINB1], nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};
-        if (h.deferring) {
-            if (h.deferred.n >= kMaxFinishJobs) fail("encoder_backward: too many deferred reductions");
-            h.deferred.j[h.deferred.n++] = job;
-        } else {
-            FinishJobs one; one.n = 1; one.j[0] = job;
-            launch_colfinish(one, h.stream);
-        }
+        finish_or_defer(defer_of(h), job, h.stream);
     } else {
         run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
     }
@@ -1154,13 +1159,7 @@ void backward(Handle& h, const BwdPtrs& t) {
         auto finish = [&](float* ws, int ns, int ntc, half_t* o0, half_t* o1) {
             FinishJob job{ws, FinishArgs{{o0, o1, nullptr, nullptr}, 0, lbias.stride[dH], lbias.stride[dP], H}, ns, H,
                           ntc, P};
-            if (h.deferring) {
-                if (h.deferred.n >= kMaxFinishJobs) fail("encoder_backward: too many deferred reductions");
-                h.deferred.j[h.deferred.n++] = job;
-            } else {
-                FinishJobs one; one.n = 1; one.j[0] = job;
-                launch_colfinish(one, h.stream);
-            }
+            finish_or_defer(defer_of(h), job, h.stream);
         };
         {
             ProfScope ps(h, "attention-bwd-dQ");
@@ -1672,6 +1671,23 @@ int sub_op_bdrlb(void* handle, const void* ddrop, const char* l_ddrop, const voi
     });
 }
 
+int sub_ops_defer(void* handle, int on) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        if (on) {
+            if (h.ops_deferring) return;
+            h.ops_deferring = h.deferring = true;
+            h.ws_cursor = 0;
+            h.deferred.n = 0;
+        } else if (h.ops_deferring) {
+            h.ops_deferring = h.deferring = false;
+            FinishJobs jobs = h.deferred;
+            h.deferred.n = 0;
+            if (jobs.n > 0) launch_colfinish(jobs, h.stream);
+        }
+    });
+}
+
 int sub_op_baob(void* handle, const void* datt, const char* l_datt, void* dbo) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
@@ -1730,6 +1746,40 @@ int sub_op_einsum_add(void* handle, const void* A, const char* l_A, const void* 
                  "must be contiguous along the same free dims)");
         ensure_gws(h, gemm_splitk_ws_floats(g));
         launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)C, alpha, ep, h.stream, h.gws, h.gws_floats);
+    });
+}
+
+int sub_op_einsum_pair(void* handle, const void* A1, const char* l_A1, const void* B1, const char* l_B1,
+                       const void* T1, const char* l_T1, void* C1, const char* l_C1, float alpha1,
+                       const void* A2, const char* l_A2, const void* B2, const char* l_B2, void* C2,
+                       const char* l_C2, float alpha2, int* paired) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        const Layout lc1 = L(h, l_C1);
+        GemmShape g1 = classify_einsum(L(h, l_A1), L(h, l_B1), lc1);
+        GemmShape g2 = classify_einsum(L(h, l_A2), L(h, l_B2), L(h, l_C2));
+        GemmEpilogue ep1;
+        if (T1) {
+            if (!l_T1 || !addend_strides(g1, L(h, l_T1), lc1, ep1.sbM, ep1.sbN, ep1.sbb))
+                fail(std::string("sub_op_einsum_pair: the dims of the addend are not free or batch dims of ") + l_C1 +
+                     " in one dense run each");
+            ep1.bias = (const half_t*)T1;
+            if (gemm_kernel_kind(g1, A1, B1, C1, ep1) != 1)
+                fail("sub_op_einsum_pair: these layouts go to the kernel without an epilogue (addend and output "
+                     "must be contiguous along the same free dims)");
+        }
+        size_t need = gemm_splitk_ws_floats(g1), need2 = gemm_splitk_ws_floats(g2);
+        ensure_gws(h, need > need2 ? need : need2);
+        bool done = h.pair_products &&
+                    launch_gemm_pair(g1, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, alpha1, ep1, g2,
+                                     (const half_t*)A2, (const half_t*)B2, (half_t*)C2, alpha2, GemmEpilogue{},
+                                     h.stream, h.gws, h.gws_floats);
+        if (!done) {
+            launch_gemm(g1, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, alpha1, ep1, h.stream, h.gws, h.gws_floats);
+            launch_gemm(g2, (const half_t*)A2, (const half_t*)B2, (half_t*)C2, alpha2, GemmEpilogue{}, h.stream, h.gws,
+                        h.gws_floats);
+        }
+        if (paired) *paired = done ? 1 : 0;
     });
 }
 

@@ -249,13 +249,7 @@ void run_col(const RowSpace& rs, const ColArgs& a, FinishArgs fo, float* ws, hip
                            a, ws, p.lpr_log2, p.rows_per_block, nrows);
     check_launch(what);
     FinishJob job{ws, fo, NS, nbatch, p.ntc, rs.R};
-    if (defer) {
-        if (defer->n >= kMaxFinishJobs) fail(std::string(what) + ": too many deferred reductions");
-        defer->j[defer->n++] = job;
-    } else {
-        FinishJobs one; one.n = 1; one.j[0] = job;
-        launch_colfinish(one, st);
-    }
+    finish_or_defer(defer, job, st);
 }
 
 // One wave per (i0,i1,i2): sum over i3 and the row.

@@ -402,13 +402,7 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     // with move_sum both forms have three sums; the extended form's third is the output-bias gradient
     FinishArgs fo{{sums[0], sums[1], a.move_sum && ext ? sums[3] : sums[2], sums[3]}, 0, 0, 1, 1};
     FinishJob job{ws, fo, a.move_sum ? 3 : (ext ? 4 : 2), 1, blocks, rs.R};
-    if (defer) {
-        if (defer->n >= kMaxFinishJobs) fail("fused LayerNorm backward: too many deferred reductions");
-        defer->j[defer->n++] = job;
-    } else {
-        FinishJobs one; one.n = 1; one.j[0] = job;
-        launch_colfinish(one, st);
-    }
+    finish_or_defer(defer, job, st);
 }
 
 }  // namespace sub

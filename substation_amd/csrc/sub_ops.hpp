@@ -75,6 +75,20 @@ struct FinishJobs {
     int n = 0;
 };
 void launch_colfinish(const FinishJobs& jobs, hipStream_t st);
+// Hands a reduction's second stage to the list, or launches it at once when there is none.  A full list is
+// finished first (its partials are complete by the time that launch runs: the stream orders them).
+inline void finish_or_defer(FinishJobs* defer, const FinishJob& job, hipStream_t st) {
+    if (!defer) {
+        FinishJobs one; one.n = 1; one.j[0] = job;
+        launch_colfinish(one, st);
+        return;
+    }
+    if (defer->n >= kMaxFinishJobs) {
+        launch_colfinish(*defer, st);
+        defer->n = 0;
+    }
+    defer->j[defer->n++] = job;
+}
 size_t colreduce_ws_floats(const RowSpace& rs, int nsums);
 void launch_bsb(const RowSpace& rs, View in, View dout, View scale, View din, ColOut dscale,
                 ColOut dbias, float* ws, hipStream_t st, FinishJobs* defer = nullptr);

@@ -17,6 +17,7 @@ encoder module: {0,1} masks from the seeded Philox streams, ``y = x * mask``
 without rescaling; as in the reference there is none on the attention
 probabilities of this layer.
 """
+import contextlib
 import math
 
 import torch
@@ -162,6 +163,14 @@ def _make_function(m):
             w = dict(zip(names, params))
             s = ctx.saved
             dy = dy.contiguous()
+            # the second stage of every column sum of the pass (eight bias / scale gradients) in one launch at its end
+            with contextlib.ExitStack() as stack:
+                for ops in ({id(o): o, id(os_): os_}).values():
+                    stack.enter_context(ops.deferred_column_sums())
+                return DecoderFunction._backward(w, s, x, enc, dy)
+
+        @staticmethod
+        def _backward(w, s, x, enc, dy):
             e = o.empty
             g = {n: torch.empty_like(w[n]) for n in names}
             # norm3, residual, feed-forward                           transformer.py:371-395
@@ -173,8 +182,8 @@ def _make_function(m):
             o.einsum(dff, 'BJI', s['ff1'], 'BJU', g['linear2_w'], 'IU')
             o.bdrlb(dff1, 'BJU', s['mask3'], 'BJU', s['lin1'], 'BJU', dlin1, 'BJU', g['linear1_b'])
             dnormed2_linear = e('BJI')
-            o.einsum(dlin1, 'BJU', w['linear1_w'], 'UI', dnormed2_linear, 'BJI')
-            o.einsum(dlin1, 'BJU', s['normed2'], 'BJI', g['linear1_w'], 'UI')
+            o.einsum_pair((dlin1, 'BJU', w['linear1_w'], 'UI', dnormed2_linear, 'BJI'),
+                          (dlin1, 'BJU', s['normed2'], 'BJI', g['linear1_w'], 'UI'))
             # norm2, residual, encoder-decoder attention              transformer.py:396-413
             dln2, dres2, datt2 = e('BJI'), e('BJI'), e('BJI')
             o.ln_backward(s['ln2'], 'BJI', w['norm2_scale'], dres3, 'BJI', s['istd2'], 'BJ', s['diff2'], 'BJI',
@@ -182,20 +191,20 @@ def _make_function(m):
                           dout2=dnormed2_linear, l_dout2='BJI', dlinear=dff, l_dlinear='BJI',
                           dlinear_bias=g['linear2_b'], dout_bias=g['edattn_out_b'])
             dgamma2 = e('BJHP')
-            o.einsum(datt2, 'BJI', s['gamma2'], 'BJHP', g['edattn_wo'], 'IHP')
-            o.einsum(w['edattn_wo'], 'IHP', datt2, 'BJI', dgamma2, 'BJHP')
+            o.einsum_pair((w['edattn_wo'], 'IHP', datt2, 'BJI', dgamma2, 'BJHP'),
+                          (datt2, 'BJI', s['gamma2'], 'BJHP', g['edattn_wo'], 'IHP'))
             dq2, dk2, dv2 = e('BJHP'), os_.empty('BKHP'), os_.empty('BKHP')
             o.attention_backward(s['q2'], 'BJHP', s['k2'], s['v2'], 'BKHP', s['gamma2'], 'BJHP', dgamma2, 'BJHP',
                                  s['stats2'], s['keep2'], dq2, 'BJHP', dk2, dv2, 'BKHP', scale)
             dnormed1_attn = e('BJI')
-            o.einsum(dq2, 'BJHP', w['edattn_wq'], 'HPI', dnormed1_attn, 'BJI')
-            o.einsum(dq2, 'BJHP', s['normed1'], 'BJI', g['edattn_wq'], 'HPI')
+            o.einsum_pair((dq2, 'BJHP', w['edattn_wq'], 'HPI', dnormed1_attn, 'BJI'),
+                          (dq2, 'BJHP', s['normed1'], 'BJI', g['edattn_wq'], 'HPI'))
             o.baob(dq2, 'BJI', g['edattn_in_b'][0])         # [B,J,H,P] is [B,J,I] in memory: sums over (b, j)
             denc = os_.empty('BKI')
-            os_.einsum(dk2, 'BKHP', w['edattn_wk'], 'HPI', denc, 'BKI')
-            os_.einsum(dv2, 'BKHP', w['edattn_wv'], 'HPI', denc, 'BKI', addend=denc, l_addend='BKI')
-            os_.einsum(dk2, 'BKHP', enc, 'BKI', g['edattn_wk'], 'HPI')
-            os_.einsum(dv2, 'BKHP', enc, 'BKI', g['edattn_wv'], 'HPI')
+            os_.einsum_pair((dk2, 'BKHP', w['edattn_wk'], 'HPI', denc, 'BKI'),
+                            (dk2, 'BKHP', enc, 'BKI', g['edattn_wk'], 'HPI'))
+            os_.einsum_pair((dv2, 'BKHP', w['edattn_wv'], 'HPI', denc, 'BKI', denc, 'BKI'),
+                            (dv2, 'BKHP', enc, 'BKI', g['edattn_wv'], 'HPI'))
             os_.baob(dk2, 'BJI', g['edattn_in_b'][1])
             os_.baob(dv2, 'BJI', g['edattn_in_b'][2])
             # norm1, residual, self-attention                         transformer.py:414-434
@@ -206,16 +215,16 @@ def _make_function(m):
                           dout2=dnormed1_attn, l_dout2='BJI', dlinear=datt2, l_dlinear='BJI',
                           dlinear_bias=unused, dout_bias=g['sattn_out_b'])
             dgamma1 = e('BJHP')
-            o.einsum(datt1, 'BJI', s['gamma1'], 'BJHP', g['sattn_wo'], 'IHP')
-            o.einsum(w['sattn_wo'], 'IHP', datt1, 'BJI', dgamma1, 'BJHP')
+            o.einsum_pair((w['sattn_wo'], 'IHP', datt1, 'BJI', dgamma1, 'BJHP'),
+                          (datt1, 'BJI', s['gamma1'], 'BJHP', g['sattn_wo'], 'IHP'))
             dkqv = e('QBJHP')
             kqv = s['kqv']
             o.attention_backward(kqv[1], 'BJHP', kqv[0], kqv[2], 'BKHP', s['gamma1'], 'BJHP', dgamma1, 'BJHP',
                                  s['stats1'], s['keep1'], dkqv[1], 'BJHP', dkqv[0], dkqv[2], 'BKHP', scale,
                                  attn_mask=s['mask'])
             dx = e('BJI')
-            o.einsum(w['sattn_wkqv'], 'QHPI', dkqv, 'QBJHP', dx, 'BJI', addend=dres1, l_addend='BJI')
-            o.einsum(dkqv, 'QBJHP', x, 'BJI', g['sattn_wkqv'], 'QHPI')
+            o.einsum_pair((w['sattn_wkqv'], 'QHPI', dkqv, 'QBJHP', dx, 'BJI', dres1, 'BJI'),
+                          (dkqv, 'QBJHP', x, 'BJI', g['sattn_wkqv'], 'QHPI'))
             o.baib(dkqv, 'QBJHP', g['sattn_in_b'], 'QHP')
             return (dx, denc) + tuple(g[n] for n in names)
 

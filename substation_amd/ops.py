@@ -5,6 +5,7 @@ The units pytorch_module/benchmark.py generates, compiles and times one by one
 prebuilt library.  Every tensor argument is a contiguous fp16 CUDA tensor whose
 dimension order is given by the layout string that follows it.
 """
+import contextlib
 import ctypes
 
 import torch
@@ -47,6 +48,19 @@ class Ops:
 
     def set_rng(self, seed, step=0):
         self.handle.set_rng(seed, step)
+
+    @contextlib.contextmanager
+    def deferred_column_sums(self):
+        """Inside the block the operators that reduce over tokens (bsb, ebsb, bdrlb, baob,
+        ln_backward) leave the second stage of their column sums to one launch issued
+        when the block ends: their bias and scale gradients are complete only then."""
+        self._pre()
+        self.handle.defer_column_sums(True)
+        try:
+            yield self
+        finally:
+            self._pre()
+            self.handle.defer_column_sums(False)
 
     def softmax(self, beta, l_beta, alpha, l_alpha, mask, l_mask, drop, l_drop, scale=1.0, p=0.0,
                 site=0, attn_mask=None, l_attn_mask='JK', mask_scale=1.0):
@@ -147,6 +161,20 @@ class Ops:
     def bei(self, dxatt, l_dxatt, dresid1, l_dresid1, dx, l_dx):
         _lib.check(self.lib.sub_op_bei(self._pre(), _p(dxatt), _s(l_dxatt), _p(dresid1),
                                        _s(l_dresid1), _p(dx), _s(l_dx)), 'bei')
+
+    def einsum_pair(self, first, second):
+        """Two independent contractions, in one launch where the pair qualifies (a data
+        gradient and the weight gradient next to it).  ``first`` = (a, l_a, b, l_b, c, l_c)
+        or with (addend, l_addend) appended; ``second`` = (a, l_a, b, l_b, c, l_c).
+        Returns True when they ran as one launch."""
+        a1, la1, b1, lb1, c1, lc1 = first[:6]
+        t1, lt1 = (first[6], first[7]) if len(first) > 6 else (None, None)
+        a2, la2, b2, lb2, c2, lc2 = second
+        paired = ctypes.c_int(0)
+        _lib.check(self.lib.sub_op_einsum_pair(
+            self._pre(), _p(a1), _s(la1), _p(b1), _s(lb1), _p(t1), _s(lt1) if lt1 else None, _p(c1), _s(lc1), 1.0,
+            _p(a2), _s(la2), _p(b2), _s(lb2), _p(c2), _s(lc2), 1.0, ctypes.byref(paired)), 'einsum_pair')
+        return bool(paired.value)
 
     def einsum(self, a, l_a, b, l_b, c, l_c, alpha=1.0, addend=None, l_addend=None):
         """c = alpha * einsum(a, b) [+ addend, broadcast over the dims it lacks]."""

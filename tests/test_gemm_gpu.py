@@ -80,3 +80,60 @@ def test_wide_tiles_every_operand_orientation(E, H):
             o.einsum(to_layout(A, la, la), la, to_layout(Bm, lb, lb), lb, C, lc)
             torch.cuda.synchronize()
             assert_close(from_layout(C, lc, lc), want, name=f'{la},{lb}->{lc} K={E}')
+
+
+@pytest.mark.parametrize('B,L,H,E,expect_pair', [(8, 512, 16, 1024, True), (2, 128, 4, 256, False)])
+def test_two_contractions_in_one_call(B, L, H, E, expect_pair):
+    """sub_op_einsum_pair: a data gradient (with and without a residual added in its
+    epilogue) and the weight gradient next to it, as one launch at the bench workload's
+    sizes, and at small sizes (paired or not, as the launcher decides); either way against
+    numpy.einsum and equal to what the two single calls give (to rounding where a
+    small output's contraction is split differently)."""
+    from substation_amd.ops import Ops
+    o = Ops(B, L, H, E)
+    sz = o.sizes
+    rng = np.random.default_rng(11)
+    mk = lambda lay, s=1.0: h16(s * rng.normal(size=tuple(sz[d] for d in lay)))
+    nan = lambda lay: torch.full(tuple(sz[d] for d in lay), float('nan'), dtype=torch.float16, device='cuda')
+    cases = [
+        # dXlin1 + dWlin1
+        (('BJU', 'UI', 'BJI', None), ('BJU', 'BJI', 'UI')),
+        # dXQKV + residual, dWQKV
+        (('QHPI', 'QBJHP', 'BJI', 'BJI'), ('QBJHP', 'BJI', 'QHPI')),
+        # dXout, dWout
+        (('IHP', 'BJI', 'BJHP', None), ('BJI', 'BJHP', 'IHP')),
+    ]
+    for (la1, lb1, lc1, lt1), (la2, lb2, lc2) in cases:
+        # the shared operand is the same tensor in both products, as in a backward pass
+        shared = {}
+        def operand(lay, s=1.0):
+            if lay not in shared:
+                shared[lay] = mk(lay, s)
+            return shared[lay]
+        A1, B1 = operand(la1, 0.5), operand(lb1, 0.5)
+        A2, B2 = operand(la2, 0.5), operand(lb2, 0.5)
+        T1 = mk(lt1) if lt1 else None
+        want1 = np.einsum(f'{la1},{lb1}->{lc1}'.lower(), A1, B1) + (T1 if lt1 else 0)
+        want2 = np.einsum(f'{la2},{lb2}->{lc2}'.lower(), A2, B2)
+        dev = {k: to_layout(v, k, k) for k, v in shared.items()}
+        t1 = to_layout(T1, lt1, lt1) if lt1 else None
+        C1, C2 = nan(lc1), nan(lc2)
+        first = (dev[la1], la1, dev[lb1], lb1, C1, lc1) + ((t1, lt1) if lt1 else ())
+        paired = o.einsum_pair(first, (dev[la2], la2, dev[lb2], lb2, C2, lc2))
+        torch.cuda.synchronize()
+        S1, S2 = nan(lc1), nan(lc2)
+        o.einsum(dev[la1], la1, dev[lb1], lb1, S1, lc1, addend=t1, l_addend=lt1)
+        o.einsum(dev[la2], la2, dev[lb2], lb2, S2, lc2)
+        torch.cuda.synchronize()
+        name = f'{la1},{lb1}->{lc1} + {la2},{lb2}->{lc2}'
+        assert_close(from_layout(C1, lc1, lc1), want1, name=name + ' (first)')
+        assert_close(from_layout(C2, lc2, lc2), want2, name=name + ' (second)')
+        assert_close(C1.float().cpu().numpy(), S1.float().cpu().numpy(), tol=2e-3, name=name + ' first vs single')
+        assert_close(C2.float().cpu().numpy(), S2.float().cpu().numpy(), tol=2e-3, name=name + ' second vs single')
+    if expect_pair:
+        # the pair the layer itself launches must have gone out as one launch here too
+        la1, lb1, lc1 = 'BJU', 'UI', 'BJI'
+        la2, lb2, lc2 = 'BJU', 'BJI', 'UI'
+        d = {k: to_layout(mk(k, 0.5), k, k) for k in ('BJU', 'UI', 'BJI')}
+        assert o.einsum_pair((d['BJU'], 'BJU', d['UI'], 'UI', nan('BJI'), 'BJI'),
+                             (d['BJU'], 'BJU', d['BJI'], 'BJI', nan('UI'), 'UI'))

@@ -192,6 +192,47 @@ def test_bad_and_bdrlb(B, L, H, E, act):
         assert_close(dbias.float().cpu().numpy(), w_dbias, name='DLINB1', tol=2e-2)
 
 
+def test_deferred_column_sums_give_the_same_bits():
+    """sub_ops_defer: between the two calls the column sums of the operators (here
+    nine of them: more than the list of six holds, so it is finished early once,
+    and the scratch buffer has to start over as well) are finished by shared
+    launches; every gradient vector must equal, bit for bit, what the operator gives
+    when it finishes its sums itself, and must be complete once the block ends."""
+    B, L, H, E = 4, 256, 4, 512
+    o = _ops(B, L, H, E)
+    rng = np.random.default_rng(9)
+    dev = lambda v: torch.from_numpy(h16(v)).to(torch.float16).cuda()
+    scale = dev(1 + 0.1 * rng.normal(size=E))
+    tensors = [(dev(rng.normal(size=(B, L, E))), dev(rng.normal(size=(B, L, E)))) for _ in range(3)]
+    vec = lambda: torch.zeros(E, dtype=torch.float16, device='cuda')
+
+    def run():
+        outs = []
+        for inp, dout in tensors:
+            din, ds, db, dbo = o.empty('BJI'), vec(), vec(), vec()
+            o.bsb(inp, 'BJI', scale, dout, 'BJI', din, 'BJI', ds, db)
+            o.baob(dout, 'BJI', dbo)
+            dl = vec()
+            din2, ds2, db2 = o.empty('BJI'), vec(), vec()
+            o.ebsb(inp, 'BJI', scale, dout, 'BJI', inp, 'BJI', dout, 'BJI', din2, 'BJI', ds2, db2, dl)
+            outs += [din, ds, db, dbo, din2, ds2, db2, dl]
+        return outs
+
+    plain = run()
+    torch.cuda.synchronize()
+    with o.deferred_column_sums():
+        deferred = run()
+    torch.cuda.synchronize()
+    for a, b in zip(plain, deferred):
+        assert float(a.float().abs().max()) > 0
+        assert torch.equal(a, b)
+    # the handle is back to finishing every reduction in its own call
+    dbo = vec()
+    o.baob(tensors[0][1], 'BJI', dbo)
+    torch.cuda.synchronize()
+    assert torch.equal(dbo, plain[3])
+
+
 @pytest.mark.parametrize('B,L,H,E', SIZES + [(2, 3, 1, 20), (4, 64, 1, 1024), (2, 8, 1, 4096)])
 def test_bsb_ebsb_baob_bei(B, L, H, E):
     o = _ops(B, L, H, E)
