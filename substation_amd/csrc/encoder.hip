@@ -325,7 +325,8 @@ float* take_ws(Handle& h, size_t floats) {
         if (h.deferred.n > 0) launch_colfinish(h.deferred, h.stream);
         h.deferred.n = 0;
         h.ws_cursor = 0;
-        ensure_ws(h, floats);
+        // twice the size as well: after a few calls the buffer holds every reduction of a block of calls
+        ensure_ws(h, floats > 2 * h.ws_floats ? floats : 2 * h.ws_floats);
     }
     float* p = h.ws + h.ws_cursor;
     h.ws_cursor += (floats + 63) & ~(size_t)63;

@@ -220,8 +220,9 @@ def test_deferred_column_sums_give_the_same_bits():
 
     plain = run()
     torch.cuda.synchronize()
-    with o.deferred_column_sums():
-        deferred = run()
+    for _ in range(3):                  # the scratch buffer grows to hold a whole block within a few blocks
+        with o.deferred_column_sums():
+            deferred = run()
     torch.cuda.synchronize()
     for a, b in zip(plain, deferred):
         assert float(a.float().abs().max()) > 0
