@@ -414,6 +414,27 @@ int sub_op_einsum(void* handle, const void* A, const char* l_A, const void* B, c
  * substation/transformer.py:41-52 with its bias), or a product added to a residual
  * (block_bei.cuh:12-106).  T may be C (accumulate in place).  Fails when the layouts
  * lead to a kernel that has no epilogue. */
+/* The feed-forward activation in the epilogues of the products next to it, as
+ * encoder_forward / encoder_backward run them under SUB_OPT_RELU_FROM_OUTPUT:
+ * sub_op_einsum_bad: out = dropout(act(einsum(A, B) + bias)) (gemm.cuh:134-147 followed
+ * by block_bad.cuh:28-145) with the handle's activation and the keep bits of (seed,
+ * step, site, p); `out` in BJU order; `bits` receives B*J*U/8 bytes (ReLU: one bit per
+ * output, set where it is positive; GELU: the keep bits) in the kernel's own order, for
+ * sub_op_einsum_bdrlb only; GELU also stores the pre-activation to `lin`, laid out like
+ * `out` (ReLU: ignored, may be null).
+ * sub_op_einsum_bdrlb: dlinear = act'(.) * keep * einsum(A, B) and dbias = its sum over
+ * the tokens (gemm.cuh:134-147 followed by block_bdrlb.cuh:13-146); `gate` is the forward
+ * output (ReLU) or the pre-activation (GELU), laid out like `dlinear` (BJU), `bits`
+ * what sub_op_einsum_bad left.
+ * *applied = 0 and nothing launched when the product does not qualify for the kernel
+ * that carries these epilogues (whole 256 x 256 tiles for most of the CUs, 16-byte
+ * aligned tensors): the caller then runs the product and the operator one after the other. */
+int sub_op_einsum_bad(void* handle, const void* A, const char* l_A, const void* B, const char* l_B, const void* bias,
+                      const char* l_bias, void* lin, void* out, const char* l_out, void* bits, float p, uint32_t site,
+                      int* applied);
+int sub_op_einsum_bdrlb(void* handle, const void* A, const char* l_A, const void* B, const char* l_B, const void* gate,
+                        const char* l_gate, const void* bits, void* dlinear, const char* l_dlinear, void* dbias,
+                        int* applied);
 /* Two independent contractions, the first with an optional addend T1 (null: none) as
  * in sub_op_einsum_add, in one launch where the pair qualifies (a data gradient and the
  * weight gradient next to it, as encoder_backward pairs dXlin1 with dWlin1 and dXQKV with

@@ -94,6 +94,10 @@ SIGNATURES = {
                                        _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
     'sub_op_einsum': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_einsum_add': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
+    'sub_op_einsum_bad': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _CP, _VP, _F, _U32,
+                               ctypes.POINTER(ctypes.c_int)]),
+    'sub_op_einsum_bdrlb': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _CP, _VP,
+                                 ctypes.POINTER(ctypes.c_int)]),
     'sub_op_einsum_pair': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F,
                                 _VP, _CP, _VP, _CP, _VP, _CP, _F, ctypes.POINTER(ctypes.c_int)]),
     'sub_layout_strides': (_I, [_VP, _CP, ctypes.POINTER(ctypes.c_int64)]),

@@ -1784,6 +1784,57 @@ int sub_op_einsum_pair(void* handle, const void* A1, const char* l_A1, const voi
     });
 }
 
+int sub_op_einsum_bad(void* handle, const void* A, const char* l_A, const void* B, const char* l_B, const void* bias,
+                      const char* l_bias, void* lin, void* out, const char* l_out, void* bits, float p, uint32_t site,
+                      int* applied) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        if (!applied) fail("sub_op_einsum_bad: null `applied`");
+        *applied = 0;
+        const Layout lc = L(h, l_out);
+        GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), lc);
+        GemmEpilogue ep;
+        if (!bias || !bits || !addend_strides(g, L(h, l_bias), lc, ep.sbM, ep.sbN, ep.sbb)) return;
+        ep.bias = (const half_t*)bias;
+        ep.relu_dropout = true; ep.key = make_key(h, site, p);
+        ep.gate_bits_out = (uint32_t*)bits;
+        if (h.act == ACT_GELU) { ep.act = ACT_GELU; ep.pre_out = (half_t*)lin; }
+        // the keep bits are indexed by the offset into the output: it has to be dense in canonical order
+        if (lc.str() != "BJU" || ((uintptr_t)bits & 3) || !aligned16(bias) || !aligned16(out) || !aligned16(A) ||
+            !aligned16(B) || (h.act == ACT_GELU && (!lin || !aligned16(lin))) ||
+            !gemm_relu_dropout_ok(g, A, B, out, ep))
+            return;
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)out, 1.f, ep, h.stream);
+        *applied = 1;
+    });
+}
+
+int sub_op_einsum_bdrlb(void* handle, const void* A, const char* l_A, const void* B, const char* l_B, const void* gate,
+                        const char* l_gate, const void* bits, void* dlinear, const char* l_dlinear, void* dbias,
+                        int* applied) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        if (!applied) fail("sub_op_einsum_bdrlb: null `applied`");
+        *applied = 0;
+        const Layout lc = L(h, l_dlinear);
+        GemmShape g = classify_einsum(L(h, l_A), L(h, l_B), lc);
+        GemmEpilogue ep;
+        if (!gate || !bits || !dbias || !addend_strides(g, L(h, l_gate), lc, ep.sbM, ep.sbN, ep.sbb)) return;
+        ep.gate = (const half_t*)gate; ep.gate_bits = (const uint32_t*)bits; ep.colsum = (float*)16;
+        if (h.act == ACT_GELU) ep.act = ACT_GELU;
+        if (lc.str() != "BJU" || ep.sbb[0] != 0 || ((uintptr_t)bits & 3) || !aligned16(gate) || !aligned16(dlinear) ||
+            !aligned16(A) || !aligned16(B) || !gemm_relu_dropout_ok(g, A, B, dlinear, ep))
+            return;
+        const int ntc = (int)(g.M / 128), U = (int)g.N;
+        float* ws = take_ws(h, (size_t)ntc * U);
+        ep.colsum = ws;
+        launch_gemm(g, (const half_t*)A, (const half_t*)B, (half_t*)dlinear, 1.f, ep, h.stream);
+        FinishJob job{ws, FinishArgs{{(half_t*)dbias, nullptr, nullptr, nullptr}, 0, 0, 1, 1}, 1, 1, ntc, U};
+        finish_or_defer(defer_of(h), job, h.stream);
+        *applied = 1;
+    });
+}
+
 int sub_layout_strides(void* handle, const char* layout, int64_t strides[8]) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);

@@ -49,6 +49,8 @@ class DecoderLayer(torch.nn.Module):
         self.probs = (sattn_dropout_p, edattn_dropout_p, linear1_dropout_p, ff_dropout_p)
         self.activation = activation
         self.seed, self.step = seed, 0
+        self.activation_epilogues = True     # linear1 / its backward with the activation in their epilogues where they qualify
+        self.ffn_in_epilogues = False        # whether the last forward call took them
         self.ops_t = Ops(B, Lt, H, E, activation=activation, seed=seed, intermediate_size=U)   # target-side sizes
         self.ops_s = Ops(B, Ls, H, E, activation=activation, seed=seed, intermediate_size=U)   # source-side sizes
 
@@ -140,9 +142,21 @@ def _make_function(m):
                     mask2, 'BJI', diff2, 'BJI', ln2, 'BJI', normed2, 'BJI', istd2, 'BJ', p=p_edattn,
                     site=SITE_EDATTN)
             # feed-forward, residual, norm3                           transformer.py:322-331
-            lin1, mask3, ff1 = e('BJU'), e('BJU'), e('BJU')
-            o.einsum(normed2, 'BJI', w['linear1_w'], 'UI', lin1, 'BJU')
-            o.bad(lin1, 'BJU', w['linear1_b'], lin1, 'BJU', mask3, 'BJU', ff1, 'BJU', p=p_linear1, site=SITE_LINEAR1)
+            # linear1 with bias, activation and dropout in its epilogue where the product qualifies (the keep bits
+            # then travel as bits, no mask tensor; ReLU needs no pre-activation either); else operator by operator
+            ff1 = e('BJU')
+            lin1 = e('BJU') if m.activation != 'relu' else None
+            bits = torch.empty(ff1.numel() // 8, dtype=torch.uint8, device=ff1.device)
+            mask3 = None
+            if not (m.activation_epilogues and
+                    o.einsum_bad(normed2, 'BJI', w['linear1_w'], 'UI', w['linear1_b'], 'U', lin1, ff1, 'BJU', bits,
+                                 p=p_linear1, site=SITE_LINEAR1)):
+                bits = None
+                lin1, mask3 = e('BJU'), e('BJU')
+                o.einsum(normed2, 'BJI', w['linear1_w'], 'UI', lin1, 'BJU')
+                o.bad(lin1, 'BJU', w['linear1_b'], lin1, 'BJU', mask3, 'BJU', ff1, 'BJU', p=p_linear1,
+                      site=SITE_LINEAR1)
+            m.ffn_in_epilogues = bits is not None
             ff = e('BJI')
             o.einsum(ff1, 'BJU', w['linear2_w'], 'IU', ff, 'BJI')
             mask4, diff3, ln3, y, istd3 = e('BJI'), e('BJI'), e('BJI'), e('BJI'), e('BJ')
@@ -152,7 +166,7 @@ def _make_function(m):
             ctx.saved = dict(kqv=kqv, stats1=stats1, keep1=keep1, gamma1=gamma1, mask1=mask1, diff1=diff1, ln1=ln1,
                              normed1=normed1, istd1=istd1, q2=q2, k2=k2, v2=v2, stats2=stats2, keep2=keep2,
                              gamma2=gamma2, mask2=mask2, diff2=diff2, ln2=ln2, normed2=normed2, istd2=istd2,
-                             lin1=lin1, mask3=mask3, ff1=ff1, mask4=mask4, diff3=diff3, ln3=ln3, istd3=istd3,
+                             lin1=lin1, mask3=mask3, ff1=ff1, bits=bits, mask4=mask4, diff3=diff3, ln3=ln3, istd3=istd3,
                              mask=mask)
             m.last_masks = dict(sattn=mask1, edattn=mask2, linear1=mask3, ff=mask4)
             return y
@@ -177,10 +191,17 @@ def _make_function(m):
             dln3, dres3, dff = e('BJI'), e('BJI'), e('BJI')
             o.ln_backward(s['ln3'], 'BJI', w['norm3_scale'], dy, 'BJI', s['istd3'], 'BJ', s['diff3'], 'BJI',
                           s['mask4'], 'BJI', dln3, 'BJI', dres3, 'BJI', dff, 'BJI', g['norm3_scale'], g['norm3_bias'])
-            dff1, dlin1 = e('BJU'), e('BJU')
-            o.einsum(dff, 'BJI', w['linear2_w'], 'IU', dff1, 'BJU')
+            dlin1 = e('BJU')
+            gate = s['ff1'] if m.activation == 'relu' else s['lin1']
+            if s['bits'] is None or not o.einsum_bdrlb(dff, 'BJI', w['linear2_w'], 'IU', gate, 'BJU', s['bits'],
+                                                       dlin1, 'BJU', g['linear1_b']):
+                if s['mask3'] is None:
+                    raise RuntimeError('DecoderLayer: the forward pass ran linear1 with its activation epilogue, the '
+                                       'backward pass cannot (tensors not 16-byte aligned?)')
+                dff1 = e('BJU')
+                o.einsum(dff, 'BJI', w['linear2_w'], 'IU', dff1, 'BJU')
+                o.bdrlb(dff1, 'BJU', s['mask3'], 'BJU', s['lin1'], 'BJU', dlin1, 'BJU', g['linear1_b'])
             o.einsum(dff, 'BJI', s['ff1'], 'BJU', g['linear2_w'], 'IU')
-            o.bdrlb(dff1, 'BJU', s['mask3'], 'BJU', s['lin1'], 'BJU', dlin1, 'BJU', g['linear1_b'])
             dnormed2_linear = e('BJI')
             o.einsum_pair((dlin1, 'BJU', w['linear1_w'], 'UI', dnormed2_linear, 'BJI'),
                           (dlin1, 'BJU', s['normed2'], 'BJI', g['linear1_w'], 'UI'))

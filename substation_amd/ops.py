@@ -162,6 +162,26 @@ class Ops:
         _lib.check(self.lib.sub_op_bei(self._pre(), _p(dxatt), _s(l_dxatt), _p(dresid1),
                                        _s(l_dresid1), _p(dx), _s(l_dx)), 'bei')
 
+    def einsum_bad(self, a, l_a, b, l_b, bias, l_bias, lin, out, l_out, bits, p=0.0, site=2):
+        """out = dropout(act(einsum(a, b) + bias)) in one launch where the product qualifies
+        (then True; False: nothing was launched).  ``bits``: a uint8 tensor of numel(out) / 8
+        bytes for einsum_bdrlb; ``lin`` receives the pre-activation (GELU; may be None with ReLU)."""
+        applied = ctypes.c_int(0)
+        _lib.check(self.lib.sub_op_einsum_bad(
+            self._pre(), _p(a), _s(l_a), _p(b), _s(l_b), _p(bias), _s(l_bias), _p(lin), _p(out), _s(l_out),
+            ctypes.c_void_p(bits.data_ptr()), p, site, ctypes.byref(applied)), 'einsum_bad')
+        return bool(applied.value)
+
+    def einsum_bdrlb(self, a, l_a, b, l_b, gate, l_gate, bits, dlinear, l_dlinear, dbias):
+        """dlinear = act'(.) * keep * einsum(a, b) and dbias = its sum over the tokens, in one
+        launch where the product qualifies (then True; False: nothing was launched).  ``gate``:
+        the output of einsum_bad (ReLU) or its pre-activation (GELU); ``bits``: what it left."""
+        applied = ctypes.c_int(0)
+        _lib.check(self.lib.sub_op_einsum_bdrlb(
+            self._pre(), _p(a), _s(l_a), _p(b), _s(l_b), _p(gate), _s(l_gate), ctypes.c_void_p(bits.data_ptr()),
+            _p(dlinear), _s(l_dlinear), _p(dbias), ctypes.byref(applied)), 'einsum_bdrlb')
+        return bool(applied.value)
+
     def einsum_pair(self, first, second):
         """Two independent contractions, in one launch where the pair qualifies (a data
         gradient and the weight gradient next to it).  ``first`` = (a, l_a, b, l_b, c, l_c)

@@ -41,14 +41,17 @@ def _oracle_params(layer):
     ((2, 128, 256, 2, 128), 0.1, True),        # target shorter than source, head size 64, causal self-attention
     ((2, 256, 128, 2, 256), 0.0, True),        # target longer than source, head size 128
     ((3, 128, 128, 4, 256), 0.2, False),       # no mask on the self-attention
+    ((8, 512, 256, 4, 256, 4096), 0.1, True),  # 16 x 16 tiles of 256 x 256 in the feed-forward products: linear1 and
+                                               # its backward carry the activation in their epilogues
 ])
 def test_decoder_layer_matches_the_oracle(dims, p, masked):
     from substation_amd import DecoderLayer
     from substation_amd.decoder import SITE_EDATTN, SITE_FF, SITE_LINEAR1, SITE_SATTN
-    B, Lt, Ls, H, E = dims
+    B, Lt, Ls, H, E = dims[:5]
     torch.manual_seed(Lt + Ls + H)
     layer = DecoderLayer(B, Lt, Ls, H, E, p, p, p, p, activation='gelu', seed=SEED,
-                         sattn_mask='causal' if masked else None).cuda()
+                         sattn_mask='causal' if masked else None,
+                         intermediate_size=dims[5] if len(dims) > 5 else None).cuda()
     with torch.no_grad():      # biases and norms away from their trivial initial values
         for n in layer.param_names:
             q = getattr(layer, n)
@@ -68,7 +71,10 @@ def test_decoder_layer_matches_the_oracle(dims, p, masked):
                       edattn=ph.dropout_mask((B, Lt, E), p, SEED, SITE_EDATTN, step=3, dtype=np.float64),
                       linear1=ph.dropout_mask((B, Lt, U), p, SEED, SITE_LINEAR1, step=3, dtype=np.float64),
                       ff=ph.dropout_mask((B, Lt, E), p, SEED, SITE_FF, step=3, dtype=np.float64))
+    assert layer.ffn_in_epilogues == (len(dims) > 5)
     for k, v in want_masks.items():
+        if k == 'linear1' and layer.ffn_in_epilogues:
+            continue        # no mask tensor on that path: a wrong keep bit shows in y and in every gradient below
         assert (_f64(layer.last_masks[k]) == v).all(), k + ' mask differs from the seeded oracle mask'
 
     op = _oracle_params(layer)
@@ -122,3 +128,36 @@ def test_decoder_layer_steps_draw_new_masks_and_rejects_unsupported_sizes():
         DecoderLayer(1, 100, 128, 2, 128)          # target length not a multiple of 128
     with pytest.raises(ValueError):
         DecoderLayer(1, 128, 128, 4, 128)          # head size 32
+
+
+@pytest.mark.parametrize('activation', ['relu', 'gelu'])
+def test_decoder_activation_epilogues_match_the_operators(activation):
+    """linear1 with bias, activation and dropout in its epilogue and the backward of that in
+    the epilogue of the product before it (sub_op_einsum_bad, sub_op_einsum_bdrlb) against
+    the same layer run operator by operator: output and every gradient bit for bit, the
+    bias gradient of linear1 (column sums added in another order) to rounding."""
+    from substation_amd import DecoderLayer
+    B, Lt, Ls, H, E, U = 8, 512, 128, 4, 256, 4096
+    outs = []
+    for fused in (True, False):
+        torch.manual_seed(1)
+        layer = DecoderLayer(B, Lt, Ls, H, E, 0.1, 0.1, 0.1, 0.1, activation=activation, seed=SEED,
+                             intermediate_size=U).cuda()
+        layer.activation_epilogues = fused
+        g = torch.Generator().manual_seed(5)
+        x = torch.randn(B, Lt, E, generator=g).half().cuda().requires_grad_(True)
+        enc = torch.randn(B, Ls, E, generator=g).half().cuda().requires_grad_(True)
+        dy = torch.randn(B, Lt, E, generator=g).half().cuda()
+        layer.set_rng(SEED, 1)
+        y = layer(x, enc)
+        y.backward(dy)
+        torch.cuda.synchronize()
+        assert layer.ffn_in_epilogues == fused
+        outs.append([('y', y.detach().clone()), ('dx', x.grad.clone()), ('denc', enc.grad.clone())] +
+                    [('d' + n, getattr(layer, n).grad.clone()) for n in layer.param_names])
+    for (name, a), (_, b) in zip(*outs):
+        assert torch.isfinite(a.float()).all() and float(a.float().abs().max()) > 0, name
+        if name == 'dlinear1_b':
+            assert_close(_f64(a), _f64(b), tol=2e-3, name=name)
+        else:
+            assert torch.equal(a, b), name
