@@ -305,6 +305,18 @@ int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const voi
                               const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
                               const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale);
 
+/* sub_op_attention_backward that also sums dq, dk, dv over samples and positions:
+ * dq_bias, dk_bias, dv_bias are [H, P] vectors (null: not wanted; dk_bias and dv_bias
+ * both or neither), the gradients of the projection biases
+ * (BackwardAttentionInputBiases, block_baib.cuh:15-211, encoder.cu:288-290), formed in
+ * the attention launches instead of in launches that read dq, dk, dv again. */
+int sub_op_attention_backward_biases(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                                     const void* k, const void* v, const char* l_kv, const void* out,
+                                     const char* l_out, const void* d_out, const char* l_dout, void* stats,
+                                     const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
+                                     const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale,
+                                     void* dq_bias, void* dk_bias, void* dv_bias);
+
 /* block_softmax.cuh:127-188; `scale` multiplies the input (1 in the layer, where
  * the factor is the GEMM's alpha, encoder.cu:116). */
 int sub_op_softmax(void* handle, const void* beta, const char* l_beta, void* alpha,

@@ -76,6 +76,8 @@ SIGNATURES = {
                                       _F, _F, _U32]),
     'sub_op_attention_backward': (_I, [_VP, _I, _I, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP,
                                        _VP, _CP, _VP, _VP, _CP, _VP, _CP, _F]),
+    'sub_op_attention_backward_biases': (_I, [_VP, _I, _I, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP,
+                                              _VP, _CP, _VP, _VP, _CP, _VP, _CP, _F, _VP, _VP, _VP]),
     'sub_op_bs': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F]),
     'sub_op_bdrln': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP, _CP, _VP, _CP, _VP, _CP,
                           _VP, _CP, _VP, _CP, _VP, _CP, _F, _U32]),

@@ -1505,8 +1505,21 @@ int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const voi
                               const char* l_out, const void* d_out, const char* l_dout, void* stats,
                               const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
                               const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale) {
+    return sub_op_attention_backward_biases(handle, n_queries, n_keys, q, l_q, k, v, l_kv, out, l_out, d_out, l_dout,
+                                            stats, keep, dq, l_dq, dk, dv, l_dkv, attn_mask, l_attn_mask, scale,
+                                            nullptr, nullptr, nullptr);
+}
+
+int sub_op_attention_backward_biases(void* handle, int n_queries, int n_keys, const void* q, const char* l_q,
+                                     const void* k, const void* v, const char* l_kv, const void* out,
+                                     const char* l_out, const void* d_out, const char* l_dout, void* stats,
+                                     const void* keep, void* dq, const char* l_dq, void* dk, void* dv,
+                                     const char* l_dkv, const void* attn_mask, const char* l_attn_mask, float scale,
+                                     void* dq_bias, void* dk_bias, void* dv_bias) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
+        if ((dk_bias == nullptr) != (dv_bias == nullptr))
+            fail("attention backward: dk_bias and dv_bias come from one launch, give both or neither");
         AttnArgs a;
         op_attention_args(h, n_queries, n_keys, q, l_q, k, v, l_kv, out, l_out, stats, const_cast<void*>(keep),
                           attn_mask, l_attn_mask, scale, a);
@@ -1516,8 +1529,20 @@ int sub_op_attention_backward(void* handle, int n_queries, int n_keys, const voi
             !attn_side(dk, make_layout(l_dkv, z), dK, a.dk) || !attn_side(dv, make_layout(l_dkv, z), dK, a.dv))
             fail("attention backward: d_out and dq take a layout over B, J, H, P and dk, dv one over B, K, H, P, "
                  "P innermost");
-        launch_mha_backward_dq(a, (int)h.sz.n[dP], h.stream);
-        launch_mha_backward_dkv(a, (int)h.sz.n[dP], h.stream);
+        // the sums over (sample, position) of dq, dk, dv start in these launches (one partial row per block of
+        // 128 positions) and end in the finishing stage of the column sums, deferred or not
+        const int P = (int)h.sz.n[dP], H = (int)h.sz.n[dH];
+        const int ntq = a.B * (a.J / 128), ntk = a.B * (a.K / 128);
+        auto finish = [&](float* ws, int ns, int ntc, void* o0, void* o1) {
+            FinishJob job{ws, FinishArgs{{(half_t*)o0, (half_t*)o1, nullptr, nullptr}, 0, P, 1, H}, ns, H, ntc, P};
+            finish_or_defer(defer_of(h), job, h.stream);
+        };
+        if (dq_bias) a.bias_q = take_ws(h, (size_t)H * ntq * P);
+        launch_mha_backward_dq(a, P, h.stream);
+        if (dq_bias) finish(a.bias_q, 1, ntq, dq_bias, nullptr);
+        if (dk_bias) a.bias_kv = take_ws(h, (size_t)2 * H * ntk * P);
+        launch_mha_backward_dkv(a, P, h.stream);
+        if (dk_bias) finish(a.bias_kv, 2, ntk, dk_bias, dv_bias);
     });
 }
 

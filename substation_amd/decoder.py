@@ -216,18 +216,16 @@ def _make_function(m):
                           (datt2, 'BJI', s['gamma2'], 'BJHP', g['edattn_wo'], 'IHP'))
             dq2, dk2, dv2 = e('BJHP'), os_.empty('BKHP'), os_.empty('BKHP')
             o.attention_backward(s['q2'], 'BJHP', s['k2'], s['v2'], 'BKHP', s['gamma2'], 'BJHP', dgamma2, 'BJHP',
-                                 s['stats2'], s['keep2'], dq2, 'BJHP', dk2, dv2, 'BKHP', scale)
+                                 s['stats2'], s['keep2'], dq2, 'BJHP', dk2, dv2, 'BKHP', scale,
+                                 dq_bias=g['edattn_in_b'][0], dk_bias=g['edattn_in_b'][1], dv_bias=g['edattn_in_b'][2])
             dnormed1_attn = e('BJI')
             o.einsum_pair((dq2, 'BJHP', w['edattn_wq'], 'HPI', dnormed1_attn, 'BJI'),
                           (dq2, 'BJHP', s['normed1'], 'BJI', g['edattn_wq'], 'HPI'))
-            o.baob(dq2, 'BJI', g['edattn_in_b'][0])         # [B,J,H,P] is [B,J,I] in memory: sums over (b, j)
             denc = os_.empty('BKI')
             os_.einsum_pair((dk2, 'BKHP', w['edattn_wk'], 'HPI', denc, 'BKI'),
                             (dk2, 'BKHP', enc, 'BKI', g['edattn_wk'], 'HPI'))
             os_.einsum_pair((dv2, 'BKHP', w['edattn_wv'], 'HPI', denc, 'BKI', denc, 'BKI'),
                             (dv2, 'BKHP', enc, 'BKI', g['edattn_wv'], 'HPI'))
-            os_.baob(dk2, 'BJI', g['edattn_in_b'][1])
-            os_.baob(dv2, 'BJI', g['edattn_in_b'][2])
             # norm1, residual, self-attention                         transformer.py:414-434
             dln1, dres1, datt1 = e('BJI'), e('BJI'), e('BJI')
             unused = torch.empty_like(g['sattn_out_b'])          # the column sums of the third input are not needed here
@@ -242,11 +240,11 @@ def _make_function(m):
             kqv = s['kqv']
             o.attention_backward(kqv[1], 'BJHP', kqv[0], kqv[2], 'BKHP', s['gamma1'], 'BJHP', dgamma1, 'BJHP',
                                  s['stats1'], s['keep1'], dkqv[1], 'BJHP', dkqv[0], dkqv[2], 'BKHP', scale,
-                                 attn_mask=s['mask'])
+                                 attn_mask=s['mask'], dq_bias=g['sattn_in_b'][1], dk_bias=g['sattn_in_b'][0],
+                                 dv_bias=g['sattn_in_b'][2])
             dx = e('BJI')
             o.einsum_pair((w['sattn_wkqv'], 'QHPI', dkqv, 'QBJHP', dx, 'BJI', dres1, 'BJI'),
                           (dkqv, 'QBJHP', x, 'BJI', g['sattn_wkqv'], 'QHPI'))
-            o.baib(dkqv, 'QBJHP', g['sattn_in_b'], 'QHP')
             return (dx, denc) + tuple(g[n] for n in names)
 
     return DecoderFunction

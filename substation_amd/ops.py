@@ -90,12 +90,15 @@ class Ops:
             scale, p, site), 'attention_forward')
 
     def attention_backward(self, q, l_q, k, v, l_kv, out, l_out, d_out, l_dout, stats, keep, dq, l_dq, dk, dv,
-                           l_dkv, scale, attn_mask=None, l_attn_mask='JK'):
+                           l_dkv, scale, attn_mask=None, l_attn_mask='JK', dq_bias=None, dk_bias=None, dv_bias=None):
+        """``dq_bias``, ``dk_bias``, ``dv_bias``: optional [H, P] outputs, the sums of dq, dk, dv over samples
+        and positions (the gradients of the projection biases), formed in the same launches."""
         nq, nk = q.shape[l_q.index('J')], k.shape[l_kv.index('K')]
-        _lib.check(self.lib.sub_op_attention_backward(
+        _lib.check(self.lib.sub_op_attention_backward_biases(
             self._pre(), nq, nk, _p(q), _s(l_q), _p(k), _p(v), _s(l_kv), _p(out), _s(l_out), _p(d_out),
             _s(l_dout), ctypes.c_void_p(stats.data_ptr()), ctypes.c_void_p(keep.data_ptr()), _p(dq), _s(l_dq),
-            _p(dk), _p(dv), _s(l_dkv), _p(attn_mask), _s(l_attn_mask), scale), 'attention_backward')
+            _p(dk), _p(dv), _s(l_dkv), _p(attn_mask), _s(l_attn_mask), scale, _p(dq_bias), _p(dk_bias),
+            _p(dv_bias)), 'attention_backward')
 
     def bs(self, alpha, l_alpha, mask, l_mask, ddrop, l_ddrop, dbeta, l_dbeta, scale=1.0):
         _lib.check(self.lib.sub_op_bs(self._pre(), _p(alpha), _s(l_alpha), _p(mask), _s(l_mask),
