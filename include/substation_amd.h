@@ -141,7 +141,8 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * BackwardLayerNormResidualDropout (encoder.cu:160-166) as one launch, and
  * ExtendedBackwardScaleBias + BackwardLayerNormResidualDropout +
  * BackwardAttnOutBias (encoder.cu:196-212) as another, where the embedding size
- * (<= 1024) and the layouts (feature dim contiguous) allow it.  Every tensor the
+ * (<= 4096; beyond 1024 a row is shared by two or four waves) and the layouts
+ * (feature dim contiguous, dense rows) allow it.  Every tensor the
  * separate kernels write is still written, from the same fp16-rounded
  * intermediates; the bias / scale gradients are summed in a different order
  * (fp32), so results can differ from the separate launches in the last bit. */
@@ -378,7 +379,8 @@ int sub_op_aib(void* handle, const void* in, const char* l_in, const void* bias,
 /* block_baib.cuh:161-211, on the Q-stacked tensors */
 int sub_op_baib(void* handle, const void* d, const char* l_d, void* dbias, const char* l_dbias);
 /* The backward pass around one LayerNorm in one launch where the sizes and layouts
- * allow (rows of up to 1024 contiguous features), else as the separate operators,
+ * allow (rows of up to 1024 contiguous features; the plain form also dense rows of up
+ * to 4096), else as the separate operators,
  * with the same results.  extended = 0: block_bsb_ebsb.cuh:12-204 (bsb) followed
  * by block_blnrd.cuh:14-259: g = dout1 * scale, dscale, dbias, then d_ln_in and
  * d_drop_in from g.  extended = 1: block_bsb_ebsb.cuh:206-420 (ebsb: g =

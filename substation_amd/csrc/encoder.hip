@@ -825,6 +825,9 @@ bool op_lnbwd(Handle& h, bool ext, const void* in, const Layout& lin_, const voi
                     &a.d_drop_in});
     a.scale = vector_view(scale, sp.rs.R);
     if (!lnbwd_supported(sp.rs, a, ext)) return false;
+    // on the static scratch array, rows beyond 1024 features stay with the separate operators, whose
+    // partial rows fit it for every shape (the one-launch form needs up to 256 partial rows of 4096 per sum)
+    if (h.static_ws && sp.rs.R > 1024) return false;
     if (mode.dry) return true;
     float* ws = take_ws(h, lnbwd_ws_floats(sp.rs, ext));
     half_t* sums[4] = {(half_t*)dscale, (half_t*)dbias, (half_t*)dlinear_bias, (half_t*)dout_bias};
@@ -1040,8 +1043,9 @@ void backward(Handle& h, const BwdPtrs& t) {
     if (h.fuse_ln_backward) {
         // DLINB2 is the column sum of DLIN2, which the first of the two launches writes and the second
         // would only read for that sum: when both run, the first one sums it
+        // (asked with the sum moved: rows beyond 1024 features take the second launch only in that form)
         LnBwdMode probe = ln_mode;
-        probe.dry = true;
+        probe.dry = true; probe.move_sum = true;
         ln_mode.move_sum = ln2_backward(probe) && ln1_backward(probe);
     }
     if (h.fuse_ln_backward) {

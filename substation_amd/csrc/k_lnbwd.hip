@@ -171,11 +171,18 @@ __global__ __launch_bounds__(LN_BLOCK) void k_lnbwd(RowSpace rs, LnBwdArgs a, fl
 // fetched with the row, and the column sum of d_drop_in does not live in registers: a wave adds its
 // rows' values into its own slab of LDS, which the reduction of the other sums reuses afterwards.
 // Same arithmetic per row; a column sum adds a lane's rows in order, then the waves in order.
+// SEG > 1: rows of up to SEG * 1024 features, a row shared by SEG waves that take 1024 features each
+// (a lane still owns 16 columns, so the column sums stay in registers); the two sums over the row that
+// the LayerNorm backward needs meet in LDS, in wave order, behind one barrier per pass -- which is why
+// every wave then makes the same number of passes, a wave without a row walking row 0 and keeping nothing.
 constexpr int LNF_BLOCK = 1024;
 constexpr int LNF_WPB = LNF_BLOCK / WAVE;
 
-template <int VPL, bool EXT, bool PACKED, bool MOVE>
+template <int VPL, bool EXT, bool PACKED, bool MOVE, int SEG = 1>
 __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, float* ws, unsigned nrows) {
+    static_assert(SEG == 1 || VPL == 2, "a segment is 1024 features: two packs per lane");
+    constexpr int ROWS = LNF_WPB / SEG;           // rows per workgroup and pass
+    __shared__ float stat[2][LNF_WPB][2];         // SEG > 1: the waves' shares of the two row sums, by pass parity
     constexpr int NS = MOVE ? 3 : (EXT ? 4 : 2);
     constexpr int S_DROP = MOVE ? 2 : 3;          // which sum takes d_drop_in
     constexpr bool DROP_SUM = EXT || MOVE;
@@ -190,6 +197,7 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
     if (PACKED) fetch_args_now(a.mask_bits);
     else fetch_args_now(a.mask.p, a.mask.s3);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rslot = SEG > 1 ? wave / SEG : wave, seg = SEG > 1 ? wave % SEG : 0;
     const float invn = 1.0f / (float)R;
     float acc[NR][VPL][8];
 #pragma unroll
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
     int e0[VPL], keep_all[VPL];
 #pragma unroll
     for (int c = 0; c < VPL; ++c) {
-        e0[c] = (c * WAVE + lane) * 8;
+        e0[c] = seg * (VPL * WAVE * 8) + (c * WAVE + lane) * 8;
         inside[c] = e0[c] < R;
         keep_all[c] = inside[c] ? -1 : 0;
         if (!inside[c]) e0[c] = 0;
@@ -211,7 +219,12 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
     auto masked = [&](h8 v, int c) { return __builtin_bit_cast(h8, __builtin_bit_cast(i4v, v) & keep_all[c]); };
     float* const slab = &red[wave][lane * 8];     // + c * 512: this lane's 8 columns of pack c
     bool first_row = true;
-    for (unsigned row = blockIdx.x * LNF_WPB + wave; row < nrows; row += gridDim.x * LNF_WPB) {
+    const unsigned row_stride = gridDim.x * ROWS;
+    const unsigned npass = SEG > 1 ? (nrows + row_stride - 1) / row_stride : 0;
+    unsigned row_at = blockIdx.x * ROWS + rslot;
+    for (unsigned pass = 0; SEG > 1 ? pass < npass : row_at < nrows; ++pass, row_at += row_stride) {
+        const bool active = SEG == 1 || row_at < nrows;
+        const unsigned row = active ? row_at : 0;
         h8 in[VPL], d1[VPL], d2[VPL], dl[VPL], df[VPL], mk[VPL], sc[VPL];
         uint32_t mkb[VPL];
         const half_t isth = a.istd.p[(long)row * a.istd.s3];
@@ -241,16 +254,20 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
             if (EXT && !MOVE) dl8 = masked(dl[c], c);
             df[c] = masked(df[c], c);
             h8 o;
+            if (active) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float d = EXT ? (float)d18[i] + (float)d28[i] : (float)d18[i];
-                o[i] = (half_t)(d * (float)sc8[i]);
-                acc[0][c][i] += d * (float)in8[i];
-                acc[1][c][i] += d;
-                if (EXT && !MOVE) acc[2][c][i] += (float)dl8[i];
+                for (int i = 0; i < 8; ++i) {
+                    const float d = EXT ? (float)d18[i] + (float)d28[i] : (float)d18[i];
+                    o[i] = (half_t)(d * (float)sc8[i]);
+                    acc[0][c][i] += d * (float)in8[i];
+                    acc[1][c][i] += d;
+                    if (EXT && !MOVE) acc[2][c][i] += (float)dl8[i];
+                }
+            } else {
+                o = (h8)(half_t)0.0f;
             }
             o = pin(o);
-            if (inside[c] && a.write_g) stg8<true>(a.g.p + (long)row * a.g.s3 + e0[c], o);     // nothing reads G again
+            if (active && inside[c] && a.write_g) stg8<true>(a.g.p + (long)row * a.g.s3 + e0[c], o);     // nothing reads G again
             gh[c] = o;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -262,6 +279,14 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
         }
         s1 = wave_sum(s1);
         s2 = wave_sum(s2);
+        if constexpr (SEG > 1) {
+            float (*st)[2] = stat[pass & 1];
+            if (lane == 0) { st[wave][0] = s1; st[wave][1] = s2; }
+            __syncthreads();          // every wave, every pass (a wave two passes on writes the other half of `stat`)
+            s1 = 0.f; s2 = 0.f;
+#pragma unroll
+            for (int k = 0; k < SEG; ++k) { s1 += st[rslot * SEG + k][0]; s2 += st[rslot * SEG + k][1]; }
+        }
         const float c1 = s1 * is * invn;
         const float c2 = s2 * is * is * is * invn;
 #pragma unroll
@@ -275,7 +300,7 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
                 const bool kept = PACKED ? ((mkb[c] >> i) & 1u) != 0 : mk[c][i] != (half_t)0.0f;
                 y[i] = kept ? x[i] : (half_t)0.0f;
             }
-            if (DROP_SUM) {
+            if (DROP_SUM && active) {
                 // (a chunk outside the row: x comes out as -c1, which must not be summed)
                 const h8 ys = masked(y, c);
                 float4 lo = make_float4((float)ys[0], (float)ys[1], (float)ys[2], (float)ys[3]);
@@ -289,13 +314,13 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
                 *reinterpret_cast<float4*>(slab + c * 512) = lo;
                 *reinterpret_cast<float4*>(slab + c * 512 + 4) = hi;
             }
-            if (inside[c]) {
+            if (active && inside[c]) {
                 stg8<false>(a.d_ln_in.p + (long)row * a.d_ln_in.s3 + e0[c], x);
                 stg8<false>(a.d_drop_in.p + (long)row * a.d_drop_in.s3 + e0[c], y);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        first_row = false;
+        if (active) first_row = false;
     }
     if (DROP_SUM && first_row) {                   // a wave without a row
 #pragma unroll
@@ -315,11 +340,13 @@ __global__ __launch_bounds__(LNF_BLOCK) void k_lnbwd_flat(int R, LnBwdArgs a, fl
             *reinterpret_cast<float4*>(dst + c * 512 + 4) = make_float4(acc[s][c][4], acc[s][c][5], acc[s][c][6], acc[s][c][7]);
         }
     };
+    // (feature f lies in the slabs of the waves of its segment)
     auto reduce = [&](const float (*from)[VPL * WAVE * 8], int s) {
         for (int f = threadIdx.x; f < R; f += LNF_BLOCK) {
+            const int sg = SEG > 1 ? f / (VPL * WAVE * 8) : 0, fl = SEG > 1 ? f % (VPL * WAVE * 8) : f;
             float t = 0.f;
 #pragma unroll
-            for (int w = 0; w < LNF_WPB; ++w) t += from[w][f];
+            for (int w = 0; w < ROWS; ++w) t += from[w * SEG + sg][fl];
             ws[((long)s * gridDim.x + blockIdx.x) * R + f] = t;
         }
     };
@@ -353,7 +380,9 @@ inline int lnbwd_blocks(long nrows) {
 }  // namespace
 
 bool lnbwd_supported(const RowSpace& rs, const LnBwdArgs& a, bool ext) {
-    if (rs.R <= 0 || rs.R > 1024 || rs.R % 8 != 0) return false;
+    if (rs.R <= 0 || rs.R > 4096 || rs.R % 8 != 0) return false;
+    // rows beyond 1024 features: only the sixteen-wave kernel, whose waves share a row
+    if (rs.R > 1024 && !(rs.flat && !(ext && !a.move_sum))) return false;
     if (rs.rows() <= 0 || rs.rows() >= (1L << 31)) return false;
     bool ok = a.in.vec && a.d1.vec && a.diff.vec && (a.mask.vec || a.mask_bits) && a.g.vec && a.d_ln_in.vec && a.d_drop_in.vec &&
               a.scale.vec;
@@ -372,6 +401,26 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     const unsigned nrows = (unsigned)rs.rows();
     const int blocks = lnbwd_blocks(nrows);
     const int vpl = rs.R <= 512 ? 1 : 2;
+    if (rs.R > 1024) {
+        // (lnbwd_supported has ruled out the extended form without move_sum: MOVE_ is EXT_ || move_sum)
+#define SUB_LNBWD_WIDE(EXT_, MOVE_, SEG_)                                                                         \
+    do {                                                                                                          \
+        if (a.mask_bits)                                                                                          \
+            hipLaunchKernelGGL((k_lnbwd_flat<2, EXT_, true, MOVE_, SEG_>), dim3(blocks), dim3(LNF_BLOCK), 0, st, rs.R, a, ws, nrows); \
+        else                                                                                                      \
+            hipLaunchKernelGGL((k_lnbwd_flat<2, EXT_, false, MOVE_, SEG_>), dim3(blocks), dim3(LNF_BLOCK), 0, st, rs.R, a, ws, nrows); \
+    } while (0)
+#define SUB_LNBWD_WIDE_SEG(SEG_)                                                                                  \
+    do {                                                                                                          \
+        if (ext) SUB_LNBWD_WIDE(true, true, SEG_);                                                                \
+        else if (a.move_sum) SUB_LNBWD_WIDE(false, true, SEG_);                                                   \
+        else SUB_LNBWD_WIDE(false, false, SEG_);                                                                  \
+    } while (0)
+        if (rs.R <= 2048) SUB_LNBWD_WIDE_SEG(2);
+        else SUB_LNBWD_WIDE_SEG(4);
+#undef SUB_LNBWD_WIDE_SEG
+#undef SUB_LNBWD_WIDE
+    } else {
 #define SUB_LNBWD_K(KERNEL_, BLOCK_, FIRST_, VPL_, EXT_)                                                          \
     do {                                                                                                          \
         if (a.mask_bits && a.move_sum)                                                                            \
@@ -398,6 +447,7 @@ void launch_lnbwd(const RowSpace& rs, const LnBwdArgs& a, bool ext, half_t* cons
     }
 #undef SUB_LNBWD_K
 #undef SUB_LNBWD
+    }
     check_launch("fused LayerNorm backward");
     // with move_sum both forms have three sums; the extended form's third is the output-bias gradient
     FinishArgs fo{{sums[0], sums[1], a.move_sum && ext ? sums[3] : sums[2], sums[3]}, 0, 0, 1, 1};

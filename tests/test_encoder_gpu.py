@@ -328,9 +328,10 @@ def test_config5_one_sample_matches_the_oracle():
     """BASELINE configs[4] at its real widths and sequence length -- L=2048, H=32,
     E=4096, P=128, FF=16384, GELU -- for one sample (the oracle's fp64 score tensors
     are 1 GiB each): score rows of 2048 keys (four packs per lane in the softmax
-    kernels), LayerNorm rows of 4096 features (eight packs per lane; beyond what the
-    one-launch LayerNorm backward takes, so bsb, blnrd, ebsb, baob run separately with
-    the deferred finish), the attention kernels at head size 128 over 16 key blocks.
+    kernels), LayerNorm rows of 4096 features (eight packs per lane in the forward
+    kernels; in the one-launch LayerNorm backward of the path as shipped four waves to a
+    row; bsb, blnrd, ebsb, baob separately with the deferred finish in the
+    operator-by-operator path), the attention kernels at head size 128 over 16 key blocks.
     Every tensor of the operator-by-operator path, then output, DX and the 12 gradients
     of the path as shipped, against one oracle run."""
     dims = (1, 2048, 32, 4096)

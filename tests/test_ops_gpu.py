@@ -352,14 +352,18 @@ def test_attention_operator_forward_and_backward(B, H, P, J, K, p, masked, l_q, 
     assert_close(from_layout(dv, 'BKHP', l_kv), want_dv, name='dv')
 
 
-# (1000, 776: rows that end inside a lane's second pack; 5000 rows of 64: more rows than the launch has waves)
+# (1000, 776: rows that end inside a lane's second pack; 5000 rows of 64: more rows than the launch has waves;
+# 2048, 3000, 4096 features: a row shared by two or four waves -- 150 and 1200 rows make several passes with a
+# last one that leaves waves without a row, 3000 leaves the fourth wave of a row without features)
 @pytest.mark.parametrize('B,L,H,E', [(2, 128, 4, 512), (4, 64, 1, 1024), (3, 24, 2, 48), (1, 4, 1, 4096),
-                                     (3, 40, 1, 1000), (2, 130, 1, 776), (5, 1000, 1, 64)])
+                                     (3, 40, 1, 1000), (2, 130, 1, 776), (5, 1000, 1, 64),
+                                     (3, 50, 1, 2048), (2, 70, 1, 3000), (4, 300, 1, 4096)])
 @pytest.mark.parametrize('extended', [False, True])
 def test_ln_backward_one_launch_or_separate(B, L, H, E, extended):
     """sub_op_ln_backward (bsb + blnrd, or ebsb + blnrd + baob) against the oracle's
     operators, for sizes and layouts the one-launch kernel takes (rows of up to 1024
-    contiguous features) and for ones it hands to the separate operators."""
+    contiguous features, of up to 4096 in its plain form) and for ones it hands to the
+    separate operators."""
     o = _ops(B, L, H, E)
     rng = np.random.default_rng(12)
     g = lambda: h16(rng.normal(size=(B, L, E)))
