@@ -112,9 +112,11 @@ def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_
     # attention with the scores in registers: 2 / 3 / 4 products of the size of QKT
     # (the backward launches form the scores again); bytes: the projections, the
     # output or gradients, one keep bit per score
-    w['attention'] = ('mfma', 2 * attn[0], 2 * 4 * bji + hbjk // 8)
-    w['attention-bwd-dQ'] = ('mfma', 3 * attn[0], 2 * 6 * bji + hbjk // 8)
-    w['attention-bwd-dKdV'] = ('mfma', 4 * attn[0], 2 * 6 * bji + hbjk // 8)
+    # (a fourth entry: the products the algorithm has -- QKT, gamma forward; dX1gamma, dX1QKT and
+    # dX2gamma, dX2QKT backward -- without the scores and their gradient formed a second time)
+    w['attention'] = ('mfma', 2 * attn[0], 2 * 4 * bji + hbjk // 8, 2 * attn[0])
+    w['attention-bwd-dQ'] = ('mfma', 3 * attn[0], 2 * 6 * bji + hbjk // 8, 2 * attn[0])
+    w['attention-bwd-dKdV'] = ('mfma', 4 * attn[0], 2 * 6 * bji + hbjk // 8, 2 * attn[0])
     # two products in one launch
     w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
     w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
@@ -291,7 +293,7 @@ def cpu_baseline_config1(warmups=3, runs=10):
             'omp_num_threads': os.environ.get('OMP_NUM_THREADS'), 'blas': blas}
 
 
-def bench_fused_ops(args):
+def fused_op_rows(steps, warmup, only=None):
     """BASELINE configs[1] and the other memory-bound operators on their own, through the
     operator entry points of the C ABI (the units pytorch_module/benchmark.py times, whose
     shipped results are perf_softmax.txt, perf_bad.txt, perf_bsb.txt, perf_bdrln.txt):
@@ -392,6 +394,8 @@ def bench_fused_ops(args):
     ]
     rows = []
     for name, ntens, layout, make, run in specs:
+        if only is not None and name not in only:
+            continue
         nbytes = ntens * bytes_of[layout]
         nsets = max(2, -(-(640 << 20) // nbytes))            # > 2.5 x the memory-side cache in rotation
         sets = [make() for _ in range(nsets)]
@@ -406,9 +410,9 @@ def bench_fused_ops(args):
                 for d in sets:
                     run(d)
         torch.cuda.synchronize()
-        for _ in range(max(1, args.warmup // 10)):
+        for _ in range(max(1, warmup // 10)):
             graph.replay()
-        reps = max(3, args.steps // 10)
+        reps = max(3, steps // 10)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
@@ -420,6 +424,14 @@ def bench_fused_ops(args):
                          unit='GB/s', frac=round(nbytes / t / HBM_PEAK, 4), bytes=nbytes, buffer_sets=nsets))
         del sets, graph
         torch.cuda.empty_cache()
+    return rows
+
+
+def bench_fused_ops(args):
+    """`--config 2`: the line of the fused operators standing alone (fused_op_rows) beside the vendor's
+    streaming kernels on tensors of the same sizes."""
+    import torch
+    rows = fused_op_rows(args.steps, args.warmup)
     # What the same box gives vendor streaming kernels of the same shapes (torch elementwise kernels, timed the
     # same way): a ceiling for 1 read + 1 write (copy), 2 reads + 1 write (add) and 1 write (fill) at the two
     # sizes the operators above have, 8 MiB and 64 MiB per tensor.
@@ -525,6 +537,116 @@ def bench_decoder(cfg, args):
                       'config': {'workload': f'decoder layer B={B} target=source={L} H={H} E={E} causal, 4 dropouts p=0.1'}}))
 
 
+def make_step(enc, X, DY):
+    """One training step of the layer: forward, then backward from DY (run_encoder.py:361-368)."""
+    params = list(enc.parameters())
+
+    def step():
+        X.grad = None
+        for q in params:       # as optimizer.zero_grad(set_to_none=True): no accumulate kernels
+            q.grad = None
+        Y = enc(X)
+        Y.backward(DY)
+    return step
+
+
+def spin(ms, _state={}):
+    """Keeps the current stream busy for about `ms` milliseconds with a spin kernel (what the
+    reference's gpuwait/wait_kernel.cu is for): the host issues the launches that follow while it
+    runs, so they execute back to back whatever the host's issue rate.  The kernel counts clock
+    ticks and ends by itself; its rate is measured once."""
+    import torch
+    if 'ticks_per_ms' not in _state:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda._sleep(1000)
+        torch.cuda.synchronize()
+        e0.record(); torch.cuda._sleep(1_000_000); e1.record()
+        torch.cuda.synchronize()
+        _state['ticks_per_ms'] = 1_000_000 / max(e0.elapsed_time(e1), 1e-3)
+    torch.cuda._sleep(int(min(ms, 200.0) * _state['ticks_per_ms']))
+
+
+def gpu_step_us(step, n, lead_ms):
+    """GPU time of one step in microseconds: n steps issued behind a spin kernel of about n * lead_ms,
+    from an event in front of the first to one behind the last."""
+    import torch
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    spin(n * lead_ms)
+    e0.record()
+    for _ in range(n):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n
+
+
+def pass_times(enc, X, DY, n, lead_ms):
+    """Forward and backward pass timed apart, as pytorch_module/run_encoder.py:359-383 does: an event
+    before the forward call, one between the passes, one after the backward call, n steps; median,
+    min, max and standard deviation of each pass in ms (the three events of a step cost a few
+    microseconds, which stay in the figures)."""
+    import torch
+    params = list(enc.parameters())
+    done = []
+    for first in range(0, n, 10):              # ten steps at a time behind one spin kernel
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(min(10, n - first))]
+        spin(len(evs) * lead_ms)
+        for a, b, c in evs:
+            X.grad = None
+            for q in params:
+                q.grad = None
+            a.record()
+            Y = enc(X)
+            b.record()
+            Y.backward(DY)
+            c.record()
+        torch.cuda.synchronize()
+        done += [(a.elapsed_time(b), b.elapsed_time(c)) for a, b, c in evs]
+    out = {}
+    for name, ts in (('forward', [d[0] for d in done]), ('backward', [d[1] for d in done])):
+        out[name] = {'median_ms': round(statistics.median(ts), 4), 'min_ms': round(min(ts), 4),
+                     'max_ms': round(max(ts), 4), 'stdev_ms': round(statistics.pstdev(ts), 4)}
+    out['steps'] = len(done)
+    return out
+
+
+def other_workloads(args):
+    """The BASELINE workloads the headline figure does not cover, each for a fraction of a second of GPU
+    time: configs[3] and configs[4] as ms per layer (the headline's protocol -- warm-ups, then steps
+    between two synchronisations on the host clock -- and the GPU's own time per step behind a spin
+    kernel), configs[1] as the fused operators standing alone on buffers larger than the memory-side cache."""
+    import torch
+    out = {}
+    for cid, steps, warmup in ((4, 20, 5), (5, 6, 2)):
+        cfg = dict(CONFIGS[cid])
+        enc, X, DY = make_encoder(cfg, args.layouts)
+        step = make_step(enc, X, DY)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        gpu_ms = gpu_step_us(step, min(steps, 10), 1.2 * ms) * 1e-3
+        U, P = 4 * cfg['E'], cfg['E'] // cfg['H']
+        flops = 3 * (2 * cfg['B'] * cfg['L'] * (4 * cfg['E'] ** 2 + 2 * cfg['E'] * U)
+                     + 4 * cfg['B'] * cfg['H'] * cfg['L'] ** 2 * P)
+        out['configs[%d]' % (cid - 1)] = {'workload': cfg['name'], 'ms_per_layer': round(ms, 4),
+                                          'gpu_ms_per_layer': round(gpu_ms, 4), 'steps': steps, 'warmup': warmup,
+                                          'tflops': round(flops / (gpu_ms * 1e-3) / 1e12, 1),
+                                          'frac_of_mfma_peak': round(flops / (gpu_ms * 1e-3) / MFMA_PEAK_F16, 4)}
+        del enc, X, DY, step
+        torch.cuda.empty_cache()
+    rows = fused_op_rows(30, 10, only=('softmax', 'bs', 'bad', 'bdrln'))
+    out['configs[1]'] = {'workload': 'softmax (scale 1/8, dropout p=0.1 seeded) and its backward on scores [16,8,512,512], '
+                                     'bad and bdrln at B=8 L=512 E=1024 FF=4096, each operator alone, fp16 masks and every '
+                                     'output written (the reference operators\' tensors)',
+                         'ops': [{k: r[k] for k in ('op', 'us', 'achieved', 'unit', 'frac', 'bytes')} for r in rows]}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -534,6 +656,8 @@ def main():
     ap.add_argument('--layouts', default='mi355x', choices=['mi355x', 'ref'])
     ap.add_argument('--profile-steps', type=int, default=20)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-other-workloads', action='store_true',
+                    help='leave out the short runs of BASELINE configs[1], [3] and [4] that the default line carries')
     ap.add_argument('--per-op', action='store_true', help='print the per-operator table to stderr')
     ap.add_argument('--option', action='append', default=[], metavar='ID=VALUE',
                     help='library option to set (sub_set_option), e.g. 2=0 runs the LayerNorm backward '
@@ -571,15 +695,7 @@ def main():
     for item in args.option:
         k, v = item.split('=')
         enc._handle.set_option(int(k), int(v))
-
-    params = list(enc.parameters())
-
-    def step():
-        X.grad = None
-        for q in params:       # as optimizer.zero_grad(set_to_none=True): no accumulate kernels
-            q.grad = None
-        Y = enc(X)
-        Y.backward(DY)
+    step = make_step(enc, X, DY)
 
     for _ in range(args.warmup):
         step()
@@ -598,13 +714,34 @@ def main():
         torch.cuda.synchronize()
         del a, b
 
-    # Per-launch durations: HIP events recorded by the library around every launch, on the
-    # stream the kernels run on; the launches are the timed region's.  Two steps are issued
-    # back to back and the events of the second are read after its backward pass, so that
-    # no start event sits on an idle stream (host time before a launch would land in it).
+    if args.profile_steps <= 0:        # timing only
+        print(json.dumps({'metric': 'fwd+bwd ms/layer', 'value': round(ms_per_step, 4), 'unit': 'ms',
+                          'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                          'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False}))
+        return
+
+    # Everything below is timed on the GPU's own clock (HIP events on the launch stream) behind a spin
+    # kernel, so that the host has issued the launches before they run: a figure does not depend on how
+    # fast this host issues them.
+    lead_ms = 1.5 * max(ms_per_step, 0.4)
+    # Forward and backward pass apart, an event between them (pytorch_module/run_encoder.py:359-383).
+    passes = pass_times(enc, X, DY, max(10, min(args.steps, 50)), lead_ms)
+    # The cost of the library's per-launch events, calibrated directly: the same steps back to back with
+    # and without them, in turns; the difference per launch is taken off every entry below.
+    n_cal = 10
+    plain, inst = [], []
+    for _ in range(3):
+        plain.append(gpu_step_us(step, n_cal, lead_ms))
+        enc._handle.profile_enable(True)
+        inst.append(gpu_step_us(step, n_cal, 2 * lead_ms))
+        enc._handle.profile_enable(False)
+    gpu_us_per_step = statistics.median(plain)
+    # Per-launch durations: an event in front of every launch and one at the end of each pass, a launch
+    # lasting from its event to the next; the launches are the timed region's.
     enc._handle.profile_enable(True)
     per_op = {}
     for _ in range(args.profile_steps):
+        spin(2 * 2 * lead_ms)
         step()
         step()
         for n, ms in enc.profile():
@@ -614,40 +751,41 @@ def main():
                             relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
                             packed_masks='9=0' not in args.option and cfg['E'] % 8 == 0,
                             skip_unread='10=0' not in args.option)
-    # Memory-bound launches are priced on the bytes of the reference's operators (each distinct big
-    # tensor read once and written once, masks as fp16 tensors, every named output written); what
-    # this build's launches still have to move after options 9 and 10 is reported beside it.
+    # Memory-bound launches: `achieved` and `frac` are the bytes the launch moves (each big tensor it reads
+    # or writes once, the residual dropout masks as bits, outputs nothing reads not written) per second; what
+    # the reference's operators would have moved for the same result (masks as fp16 tensors, every named
+    # output written) is reported beside it as effective_gbps_ref_bytes.
     work_ref = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
                                 relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
                                 packed_masks=False, skip_unread=False)
-    # The events themselves cost time: a step with an event in front of every launch takes longer
-    # than the timed steps without them.  That difference, spread evenly over the launches, is taken
-    # off every entry, so that the entries add up to the timed step.
     raw_us = {n: statistics.mean(ts) * 1e3 for n, ts in per_op.items()}
-    event_us = max(0.0, (sum(raw_us.values()) - ms_per_step * 1e3) / max(1, len(raw_us))) if raw_us else 0.0
+    event_us = (statistics.median(inst) - gpu_us_per_step) / max(1, len(raw_us))
     ops = []
     for n in per_op:
         t = max(raw_us[n] - event_us, 0.5) * 1e-6
         kind = work[n]
         if kind[0] == 'hbm':
             ref_bytes = work_ref[n][1]
-            ops.append(dict(op=n, bound='hbm', us=round(t * 1e6, 2), achieved=round(ref_bytes / t / 1e9, 1),
-                            peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(ref_bytes / t / HBM_PEAK, 4),
-                            bytes=ref_bytes, moved_bytes=kind[1], moved_gbps=round(kind[1] / t / 1e9, 1)))
+            ops.append(dict(op=n, bound='hbm', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e9, 1),
+                            peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(kind[1] / t / HBM_PEAK, 4),
+                            bytes=kind[1], ref_bytes=ref_bytes,
+                            effective_gbps_ref_bytes=round(ref_bytes / t / 1e9, 1)))
         else:
-            ops.append(dict(op=n, bound='mfma', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e12, 1),
-                            peak=MFMA_PEAK_F16 / 1e12, unit='TFLOP/s', frac=round(kind[1] / t / MFMA_PEAK_F16, 4),
-                            flops=kind[1], hbm_gbps=round(kind[2] / t / 1e9, 1)))
+            o = dict(op=n, bound='mfma', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e12, 1),
+                     peak=MFMA_PEAK_F16 / 1e12, unit='TFLOP/s', frac=round(kind[1] / t / MFMA_PEAK_F16, 4),
+                     flops=kind[1], flops_algorithmic=kind[3] if len(kind) > 3 else kind[1],
+                     hbm_gbps=round(kind[2] / t / 1e9, 1))
+            if len(kind) > 3:      # attention: the scores are formed again in the backward launches
+                o['achieved_algorithmic'] = round(kind[3] / t / 1e12, 1)
+                o['frac_algorithmic'] = round(kind[3] / t / MFMA_PEAK_F16, 4)
+            ops.append(o)
     ops.sort(key=lambda o: -o['us'])
-    if not ops:        # --profile-steps 0: timing only
-        print(json.dumps({'metric': 'fwd+bwd ms/layer', 'value': round(ms_per_step, 4), 'unit': 'ms',
-                          'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
-                          'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False}))
-        return
     dom = ops[0]
     total_us = sum(o['us'] for o in ops)
     fused = [o for o in ops if o['bound'] == 'hbm']
     gemms = [o for o in ops if o['bound'] == 'mfma']
+    fused_s = sum(o['us'] for o in fused) * 1e-6
+    gemm_s = sum(o['us'] for o in gemms) * 1e-6
     if args.per_op:
         for o in ops:
             print(json.dumps(o), file=sys.stderr)
@@ -671,18 +809,29 @@ def main():
                         and not args.option else None),
             'launch_us': dom['us'], 'launches_per_step': 1,
         },
+        # GPU time of a step without and with the per-launch events, steps back to back behind a spin kernel;
+        # their difference per launch is what was taken off every entry of `ops`
+        'gpu_us_per_step': round(gpu_us_per_step, 1), 'gpu_us_per_step_with_events': round(statistics.median(inst), 1),
         'op_time_us': round(total_us, 1), 'event_us_per_launch': round(event_us, 2),
-        'fused_ops': {'us': round(sum(o['us'] for o in fused), 1),
-                      'gbps': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / 1e9, 1),
-                      'frac_of_hbm_peak': round(sum(o['bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4),
-                      'bytes': "the reference operators' tensors, each read once and written once",
-                      'moved_gbps': round(sum(o['moved_bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / 1e9, 1),
-                      'moved_frac_of_hbm_peak': round(sum(o['moved_bytes'] for o in fused) / (sum(o['us'] for o in fused) * 1e-6) / HBM_PEAK, 4)},
-        'contractions': {'us': round(sum(o['us'] for o in gemms), 1),
-                         'tflops': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / 1e12, 1),
-                         'frac_of_mfma_peak': round(sum(o['flops'] for o in gemms) / (sum(o['us'] for o in gemms) * 1e-6) / MFMA_PEAK_F16, 4)},
-        'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac', 'moved_gbps') if k in o} for o in ops],
+        'passes': passes,
+        'fused_ops': {'us': round(fused_s * 1e6, 1),
+                      'gbps': round(sum(o['bytes'] for o in fused) / fused_s / 1e9, 1),
+                      'frac_of_hbm_peak': round(sum(o['bytes'] for o in fused) / fused_s / HBM_PEAK, 4),
+                      'bytes': 'what the launches move: each big tensor once, residual dropout masks as bits',
+                      'effective_gbps_ref_bytes': round(sum(o['ref_bytes'] for o in fused) / fused_s / 1e9, 1)},
+        # flops: the 18 products of the layer (attention without the scores formed a second time in the
+        # backward launches); executed_tflops counts those as well
+        'contractions': {'us': round(gemm_s * 1e6, 1),
+                         'tflops': round(sum(o['flops_algorithmic'] for o in gemms) / gemm_s / 1e12, 1),
+                         'frac_of_mfma_peak': round(sum(o['flops_algorithmic'] for o in gemms) / gemm_s / MFMA_PEAK_F16, 4),
+                         'executed_tflops': round(sum(o['flops'] for o in gemms) / gemm_s / 1e12, 1)},
+        'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac', 'effective_gbps_ref_bytes',
+                                   'achieved_algorithmic', 'frac_algorithmic') if k in o} for o in ops],
     }
+    del enc, X, DY, step
+    torch.cuda.empty_cache()
+    if headline and args.layouts == 'mi355x' and not args.option and not args.no_other_workloads:
+        out['other_workloads'] = other_workloads(args)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(out))

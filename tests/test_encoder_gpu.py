@@ -13,6 +13,15 @@ from tests.test_golden import load_encoder_fixture
 pytestmark = pytest.mark.gpu
 
 SEED = 0xC0FFEE
+# Share of ReLU gates (pre-activations that fp16 rounds across 0) that may differ between the device
+# and the fp64 oracle forward pass: 6e-5 to 7e-5 measured at every BASELINE workload, twice that allowed
+# (plus, for the small shapes, four standard deviations of a count at that rate).
+GATE_FLIPS_MAX = 1.5e-4
+
+
+def _gate_flips_allowed(n):
+    return GATE_FLIPS_MAX * n + 4 * np.sqrt(GATE_FLIPS_MAX * n) + 1
+LAST = {}          # figures of the latest run_layer / run_layer_default call (the gate flips it saw)
 
 
 def _layouts(which):
@@ -95,7 +104,8 @@ def run_layer(B, L, H, E, which, p, act, seed_data=0, w_std=0.05, step=0, params
     want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate, attn_mask=attn_mask)
     if gate is not None:
         flips = (gate != (want['LIN1'] > 0)).mean()
-        assert flips < 1e-3, f'{flips:.2e} of the ReLU gates differ from the oracle forward'
+        LAST['gate_flips'] = flips
+        assert flips * gate.size <= _gate_flips_allowed(gate.size), f'{flips:.2e} of the ReLU gates differ from the oracle forward'
     return want, got
 
 
@@ -171,7 +181,8 @@ def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=
     want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate, attn_mask=attn_mask)
     if gate is not None:
         flips = (gate != ((want['LIN1'] > 0) * masks['DROP2MASK'])).mean()
-        assert flips < 1e-3, f'{flips:.2e} of the ReLU gates differ from the oracle forward'
+        LAST['gate_flips'] = flips
+        assert flips * gate.size <= _gate_flips_allowed(gate.size), f'{flips:.2e} of the ReLU gates differ from the oracle forward'
     return want, got
 
 
@@ -241,10 +252,10 @@ CHECK = ['KKQQVV', 'WKKWQQWVV', 'BETA', 'ALPHA', 'ATTN_DROP', 'GAMMA', 'ATT', 'S
 
 
 def _compare(want, got, tol=1e-2, names=CHECK, outliers=None):
+    # one bound for every tensor, the column sums over all tokens (DS*, DB*, DBO, DLINB*, DBKQV) included:
+    # measured at the BASELINE workloads they sit at 1e-3 to 3e-3 of it
     for name in names:
-        # reductions over B*L tokens of fp16-rounded intermediates get a looser bound
-        t = 3 * tol if name in ('DS1', 'DB1', 'DS2', 'DB2', 'DBO', 'DLINB1', 'DLINB2', 'DBKQV') else tol
-        assert_close(got[name], want[name], tol=t, name=name, outliers=(outliers or {}).get(name, 0.0))
+        assert_close(got[name], want[name], tol=tol, name=name, outliers=(outliers or {}).get(name, 0.0))
 
 
 @pytest.mark.parametrize('which', ['mi355x', 'bert-b8-l512-h16-e1024', 'bert-b96-l128-h16-e1024'])
