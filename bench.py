@@ -25,6 +25,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK = 8.0e12        # B/s, MI355X HBM3E
 MFMA_PEAK_F16 = 2.5e15   # FLOP/s, MI355X dense fp16
+PEAK_MHZ = 2400.0        # the engine clock that peak is quoted at
 V100_MS = 6.71           # reference README.md:23, V100-SXM2, same layer and sizes
 
 CONFIGS = {
@@ -746,6 +747,16 @@ def main():
         step()
         for n, ms in enc.profile():
             per_op.setdefault(n, []).append(ms)
+    # The shader clock the GPU held during each launch (a one-lane kernel in front of every launch samples the
+    # clock counters; a pass of its own, durations are not taken from it): the matrix-core peak scales with it.
+    enc._handle.profile_enable(2)
+    clocks = {}
+    for _ in range(min(5, args.profile_steps)):
+        spin(2 * 2 * lead_ms)
+        step()
+        step()
+        for n, mhz in enc._handle.profile_read_clocks():
+            clocks.setdefault(n, []).append(mhz)
     enc._handle.profile_enable(False)
     work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
                             relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
@@ -770,11 +781,17 @@ def main():
                             peak=HBM_PEAK / 1e9, unit='GB/s', frac=round(kind[1] / t / HBM_PEAK, 4),
                             bytes=kind[1], ref_bytes=ref_bytes,
                             effective_gbps_ref_bytes=round(ref_bytes / t / 1e9, 1)))
+            if clocks.get(n):
+                ops[-1]['mhz'] = round(statistics.median(clocks[n]))
         else:
             o = dict(op=n, bound='mfma', us=round(t * 1e6, 2), achieved=round(kind[1] / t / 1e12, 1),
                      peak=MFMA_PEAK_F16 / 1e12, unit='TFLOP/s', frac=round(kind[1] / t / MFMA_PEAK_F16, 4),
                      flops=kind[1], flops_algorithmic=kind[3] if len(kind) > 3 else kind[1],
                      hbm_gbps=round(kind[2] / t / 1e9, 1))
+            if clocks.get(n):
+                # fraction of what the matrix cores could do at the clock they ran at (peak is quoted at 2400 MHz)
+                o['mhz'] = round(statistics.median(clocks[n]))
+                o['frac_at_clock'] = round(kind[1] / t / (MFMA_PEAK_F16 * o['mhz'] / PEAK_MHZ), 4)
             if len(kind) > 3:      # attention: the scores are formed again in the backward launches
                 o['achieved_algorithmic'] = round(kind[3] / t / 1e12, 1)
                 o['frac_algorithmic'] = round(kind[3] / t / MFMA_PEAK_F16, 4)
@@ -826,7 +843,8 @@ def main():
                          'frac_of_mfma_peak': round(sum(o['flops_algorithmic'] for o in gemms) / gemm_s / MFMA_PEAK_F16, 4),
                          'executed_tflops': round(sum(o['flops'] for o in gemms) / gemm_s / 1e12, 1)},
         'ops': [{k: o[k] for k in ('op', 'bound', 'us', 'achieved', 'unit', 'frac', 'effective_gbps_ref_bytes',
-                                   'achieved_algorithmic', 'frac_algorithmic') if k in o} for o in ops],
+                                   'achieved_algorithmic', 'frac_algorithmic', 'mhz', 'frac_at_clock') if k in o}
+                for o in ops],
     }
     del enc, X, DY, step
     torch.cuda.empty_cache()

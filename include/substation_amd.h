@@ -279,6 +279,13 @@ int sub_encoder_backward(void* handle, void* const* ptrs, int n);
  * end of each pass; a launch is timed from its event to the next one. */
 int sub_profile_enable(void* handle, int on);
 int sub_profile_read(void* handle, int cap, const char** names, float* ms);
+/* on = 2 in sub_profile_enable: a one-lane kernel in front of every launch also samples the GPU's
+ * shader clock counter and its constant-rate wall clock (no counterpart in the reference).
+ * sub_profile_read_clocks returns, for the same launches as sub_profile_read, the shader clock in MHz
+ * the GPU held from one sample to the next: the matrix-core peak a launch could have reached scales
+ * with it.  The extra kernels lengthen a step by a few microseconds per launch; take durations from a
+ * run with on = 1. */
+int sub_profile_read_clocks(void* handle, int cap, const char** names, float* mhz);
 
 /* ---- single operators (the units pytorch_module/benchmark.py times) -------- */
 /* Sizes come from the handle's configuration; every tensor takes its own layout
@@ -395,8 +402,12 @@ int sub_op_ln_backward(void* handle, int extended, const void* in, const char* l
                        const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias, void* dout_bias);
 /* sub_op_ln_backward for callers that cannot allocate device memory -- code under a
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
- * counterpart in the reference.  Same arguments, same kernels and bit-identical
- * results; the fp32 partial rows of the column sums (which sub_op_ln_backward keeps
+ * counterpart in the reference.  Same arguments; for rows of up to 1024 features the
+ * same kernels and bit-identical results.  Rows of 1032 to 4096 features run as the
+ * separate operators here, where sub_op_ln_backward may take its one-launch form:
+ * the scaled gradient is bit-identical, the other outputs add the same terms in
+ * another order and agree to fp16 rounding.  The fp32 partial rows of the column
+ * sums (which sub_op_ln_backward keeps
  * in a buffer the handle allocates on first use) live in a 4 MiB array that is part
  * of the library's device image, one copy per GPU for the life of the process.
  * Nothing is allocated or freed.  A call whose partial rows would need more than

@@ -69,6 +69,7 @@ SIGNATURES = {
     'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_profile_enable': (_I, [_VP, _I]),
     'sub_profile_read': (_I, [_VP, _I, ctypes.POINTER(_CP), ctypes.POINTER(_F)]),
+    'sub_profile_read_clocks': (_I, [_VP, _I, ctypes.POINTER(_CP), ctypes.POINTER(_F)]),
     'sub_op_softmax': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _U32]),
     'sub_op_softmax_masked': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _F, _F, _F, _U32]),
     'sub_set_attention_mask': (_I, [_VP, _VP, _CP]),
@@ -220,7 +221,15 @@ class Handle:
         return bool(out.value)
 
     def profile_enable(self, on=True):
-        check(self.lib.sub_profile_enable(self.ptr, 1 if on else 0), 'sub_profile_enable')
+        """on: False / True, or 2 for per-launch timing plus clock samples (profile_read_clocks)."""
+        check(self.lib.sub_profile_enable(self.ptr, int(on)), 'sub_profile_enable')
+
+    def profile_read_clocks(self, cap=64):
+        """(launch name, shader clock in MHz during it) for the launches profile_read lists."""
+        names = (ctypes.c_char_p * cap)()
+        mhz = (ctypes.c_float * cap)()
+        n = check(self.lib.sub_profile_read_clocks(self.ptr, cap, names, mhz), 'sub_profile_read_clocks')
+        return [(names[i].decode(), float(mhz[i])) for i in range(min(n, cap))]
 
     def profile_read(self, cap=64):
         names = (ctypes.c_char_p * cap)()

@@ -168,6 +168,20 @@ enum G { G_QKV_BIAS, G_DXQKV_RESID, G_LIN1_BAD, G_DXLIN2_BDRLB, G_QKV, G_QKT, G_
 // one (the next launch's, or the marker that closes a pass: name == nullptr).
 struct ProfEntry { const char* name; hipEvent_t a; };
 
+// sub_profile_enable(handle, 2): besides the event, a one-lane kernel in front of every launch stores the
+// shader clock counter (s_memtime) and the constant-rate wall clock (s_memrealtime); the ratio of their
+// differences between two samples is the shader clock the GPU held during the launch between them.
+// The shader clock counter is one per XCD and the eight do not agree, so every sample is taken on each
+// XCD (sixteen one-lane workgroups, dealt round-robin over the XCDs; each stores into the slot of the XCD
+// it finds itself on) and differences are formed per XCD.
+constexpr int kMaxClockSamples = 256;
+constexpr int kClockXcds = 8;
+__global__ void k_clock_sample(unsigned long long* slot) {
+    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kClockXcds - 1);     // XCC_ID, bits 3:0
+    slot[2 * xcc] = __builtin_readcyclecounter();
+    slot[2 * xcc + 1] = wall_clock64();
+}
+
 struct Handle {
     bool configured = false;
     Sizes sz;
@@ -192,6 +206,8 @@ struct Handle {
     float* gws = nullptr;         // split-k partials of the small-output contractions
     size_t gws_floats = 0, gws_need = 0;
     bool profiling = false;
+    bool profile_clocks = false;      // profiling with clock samples (sub_profile_enable(handle, 2))
+    unsigned long long* clock_buf = nullptr;   // kMaxClockSamples pairs (shader clock counter, wall clock)
     uint32_t* step_dev = nullptr;     // optional device-side dropout step (HIP-graph replays)
     const void* attn_mask = nullptr;  // optional additive [J,K] attention mask (caller-owned)
     Layout l_attn_mask;
@@ -226,6 +242,7 @@ struct Handle {
         if (ws) (void)hipFree(ws);
         if (gws) (void)hipFree(gws);
         if (mask_plan) (void)hipFree(mask_plan);
+        if (clock_buf) (void)hipFree(clock_buf);
         for (auto& e : prof) (void)hipEventDestroy(e.a);
         if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
     }
@@ -278,6 +295,8 @@ struct ProfScope {
         ProfEntry& e = h.prof[h.prof_used++];
         e.name = name;
         hip_check(hipEventRecord(e.a, h.stream), "hipEventRecord");
+        if (h.profile_clocks && h.prof_used <= (size_t)kMaxClockSamples)
+            hipLaunchKernelGGL(k_clock_sample, dim3(2 * kClockXcds), dim3(1), 0, h.stream, h.clock_buf + 2 * kClockXcds * (h.prof_used - 1));
         used = true;
     }
     // nothing was launched: the entry goes (its event stays in the stream, harmless)
@@ -1421,7 +1440,47 @@ int sub_attention_in_registers(void* handle, int* planned) {
 }
 
 int sub_profile_enable(void* handle, int on) {
-    return guarded([&] { Handle& h = as_handle(handle); h.profiling = on != 0; h.prof_used = 0; });
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        h.profiling = on != 0; h.prof_used = 0;
+        h.profile_clocks = on == 2;
+        if (h.profile_clocks && !h.clock_buf)
+            hip_check(hipMalloc((void**)&h.clock_buf, sizeof(unsigned long long) * 2 * kClockXcds * kMaxClockSamples), "hipMalloc(clock samples)");
+        if (h.profile_clocks)       // a slot no workgroup wrote reads as zero and is left out
+            hip_check(hipMemset(h.clock_buf, 0, sizeof(unsigned long long) * 2 * kClockXcds * kMaxClockSamples), "hipMemset(clock samples)");
+    });
+}
+
+int sub_profile_read_clocks(void* handle, int cap, const char** names, float* mhz) {
+    int count = 0;
+    int rc = guarded([&] {
+        Handle& h = as_handle(handle);
+        if (!h.profile_clocks || !h.clock_buf) fail("sub_profile_read_clocks: enable profiling with mode 2 first");
+        hip_check(hipStreamSynchronize(h.stream), "hipStreamSynchronize");
+        std::vector<unsigned long long> v(2 * kClockXcds * kMaxClockSamples);
+        hip_check(hipMemcpy(v.data(), h.clock_buf, v.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost), "hipMemcpy");
+        int dev = 0, wall_khz = 0;
+        hip_check(hipGetDevice(&dev), "hipGetDevice");
+        hip_check(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, dev), "hipDeviceGetAttribute");
+        for (size_t i = 0; i + 1 < h.prof_used && i + 1 < (size_t)kMaxClockSamples; ++i) {
+            if (!h.prof[i].name) continue;
+            if (count < cap) {
+                // the mean over the XCDs that both samples reached
+                double sum = 0.0; int n = 0;
+                for (int x = 0; x < kClockXcds; ++x) {
+                    const unsigned long long* a = &v[2 * (kClockXcds * i + x)];
+                    const unsigned long long* b = &v[2 * (kClockXcds * (i + 1) + x)];
+                    if (a[1] == 0 || b[1] <= a[1] || b[0] <= a[0]) continue;
+                    sum += (double)(b[0] - a[0]) / (double)(b[1] - a[1]);
+                    ++n;
+                }
+                if (names) names[count] = h.prof[i].name;
+                if (mhz) mhz[count] = n ? (float)(sum / n * wall_khz * 1e-3) : 0.f;
+            }
+            ++count;
+        }
+    });
+    return rc == 0 ? count : rc;
 }
 
 int sub_profile_read(void* handle, int cap, const char** names, float* ms) {

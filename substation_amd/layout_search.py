@@ -11,9 +11,14 @@ candidate configuration is only a new handle: the whole layer is run under it
 with per-operator timing on and the measured times are entered in the same
 kind of table (operator x layouts of its tensors -> seconds, minimum over
 measurements).  The minimisation is a coordinate descent over that table with
-three kinds of moves (one tensor; all same-shaped tensors of one operator; all
-same-shaped tensors of the layer), measuring only configurations whose
-operators are not all in the table yet.  Configurations that would send a
+four kinds of moves (all same-shaped tensors of the layer; those together with
+the weights of the operators that touch them, every combination of their layouts
+as one coordinate; all same-shaped tensors of one operator; one tensor), measuring
+only configurations whose operators are not all in the table yet.  The second
+kind is what lets the descent leave the family of layouts it was started in
+(feature-major activations, as in the reference's shipped configurations, against
+token-major ones): the fused paths switch on for a whole group of tensors or
+not at all.  Configurations that would send a
 contraction to the scalar fallback kernel are discarded without being run.
 
 Output: a layouts pickle in the schema of config_selection/optimize.py:443-493
@@ -162,14 +167,16 @@ class LayerTimer:
 # --------------------------------------------------------------------------- #
 
 class LayoutSearch:
-    """Coordinate descent on the measured operator-time table.
+    """Coordinate descent on the measured operator-time table (the place of the shortest-path
+    search of config_selection/optimize.py:13-493).
 
     ``timer`` needs ``measure(layouts) -> {operator: seconds}`` and
     ``usable(layouts) -> bool``."""
 
     def __init__(self, timer, start, tie_io=True, fixed=(), min_gain=0.002, log=None, out=sys.stdout,
-                 budget_s=None):
+                 budget_s=None, max_compound=4096):
         self.timer, self.tie_io, self.min_gain = timer, tie_io, min_gain
+        self.max_compound = max_compound     # largest number of settings one compound coordinate may have
         self.fixed = set(fixed)
         self.current = _lay.validate(_og.with_layouts(start, {}))
         self.table = {}          # (operator, layouts of its tensors) -> seconds, min over measurements
@@ -279,6 +286,35 @@ class LayoutSearch:
             gm = group_moves(f'class {ds}', members)
             if gm:
                 yield gm
+        # 1b. a class together with the weights of the operators that touch it, every combination of
+        # their layouts as one coordinate.  What switches a fused path on or off is a property of such
+        # a group -- the attention kernels with the scores in registers need the projections, their
+        # gradients, WKQV, BKQV and WO to agree on where heads and head size lie; the activation
+        # epilogues need the [B,J,U] tensors and LINW1 / LINW2 to agree -- and no path of single-coordinate
+        # improvements leads from one such family of layouts to another: half-way configurations cannot be
+        # expressed as GEMMs at all or fall to strided kernels.
+        for ds, members in classes.items():
+            members = [m for m in members if len(_og.candidate_layouts(m)) > 1]
+            params = []
+            for _, _, tensors in _og.OPERATORS:
+                if any(m in tensors for m in members):
+                    params += [n for n in tensors if n in _lay.PARAM_NAMES and n not in params
+                               and n not in self.fixed and len(_og.candidate_layouts(n)) > 1]
+            if not members or not params:
+                continue
+            count = len(list(itertools.permutations(_lay.CANONICAL[members[0]].replace('Q', ''))))
+            for n in params:
+                count *= len(_og.candidate_layouts(n))
+            if count > self.max_compound:
+                continue
+            base = _lay.CANONICAL[members[0]].replace('Q', '')
+            alts = []
+            for p in itertools.permutations(base):
+                p = ''.join(p)
+                act = {m: ('Q' + p if 'Q' in _lay.CANONICAL[m] else p) for m in members}
+                for combo in itertools.product(*[_og.candidate_layouts(n) for n in params]):
+                    alts.append({**act, **dict(zip(params, combo))})
+            yield f'class {ds} with ' + ' '.join(params), alts
         # 2. same-shaped tensors of one operator
         for op, _, tensors in _og.OPERATORS:
             per = {}
@@ -315,6 +351,8 @@ class LayoutSearch:
                     return self.current
                 best, best_cost = None, cur_cost
                 for raw in alts:
+                    if self.out_of_time():
+                        break
                     ch = self._expand(raw)
                     if ch is None:
                         continue

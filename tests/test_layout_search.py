@@ -120,3 +120,52 @@ def test_search_on_device_returns_layouts_that_keep_parity(tmp_path):
     assert og.tensor_layouts(again) == og.tensor_layouts(best)
     want, got = run_layer(*dims, again, 0.1, 'relu', seed_data=21)
     _compare(want, got)
+
+
+class _CoupledTimer(_SyntheticTimer):
+    """A table with a fused path that a whole group of tensors switches on, as the attention kernels
+    with the scores in registers do on the device: the projections, the attention output and their
+    gradients must have the head size innermost and the tokens outermost, and the weights that
+    produce and consume them must order heads and head size the same way.  Configurations in which
+    activations and weights disagree on that order cannot be expressed as GEMMs (not usable), so no
+    sequence of single-coordinate or single-class moves leads from the reference's family of layouts
+    (head size outermost) to the other one."""
+    GROUP = ('KKQQVV', 'WKKWQQWVV', 'GAMMA', 'DGAMMA', 'DKKQQVV')
+
+    @staticmethod
+    def _hp(layout):
+        return layout.index('H') < layout.index('P')
+
+    def usable(self, layouts):
+        t = og.tensor_layouts(layouts)
+        orders = {self._hp(t[n]) for n in self.GROUP + ('WKQV', 'BKQV', 'WO')}
+        return len(orders) == 1 and super().usable(layouts)
+
+    def measure(self, layouts):
+        times = super().measure(layouts)
+        t = og.tensor_layouts(layouts)
+        fused = all(t[n].endswith('BJHP') for n in self.GROUP) and t['WKQV'] == 'QHPI' and t['WO'] == 'IHP'
+        for op in ('attention', 'attention-bwd-dQ', 'attention-bwd-dKdV'):
+            times[op] = 1e-6 if fused else 20e-6
+        return times
+
+
+def test_descent_leaves_the_family_of_layouts_it_was_started_in():
+    """Started from the reference's shipped configuration (feature-major, head size outermost) the search
+    must end where it ends when started from the MI355X default: within 3 % of that time, with the
+    group's fused path switched on."""
+    preferred = {n: l for n, l in og.tensor_layouts(L.mi355x_layouts()).items()}
+    ends = {}
+    for label, start in (('default', L.mi355x_layouts()), ('reference', L.reference_layouts('bert-b8-l512-h16-e1024'))):
+        timer = _CoupledTimer(preferred)
+        s = ls.LayoutSearch(timer, start, out=io.StringIO())
+        best = s.run(sweeps=4)
+        ends[label] = s.cost(best)
+        t = og.tensor_layouts(best)
+        assert all(t[n].endswith('BJHP') for n in _CoupledTimer.GROUP), (label, {n: t[n] for n in _CoupledTimer.GROUP})
+    assert ends['reference'] <= 1.03 * ends['default'], ends
+    # without the compound coordinates the same search stays in the reference's family
+    timer = _CoupledTimer(preferred)
+    s = ls.LayoutSearch(timer, L.reference_layouts('bert-b8-l512-h16-e1024'), out=io.StringIO(), max_compound=0)
+    stuck = s.cost(s.run(sweeps=4))
+    assert stuck > 1.03 * ends['default']
