@@ -66,7 +66,26 @@ GEMM_OPS = ('QKV-fused', 'QKT', 'gamma', 'out', 'lin1', 'lin2', 'dXlin2', 'dWlin
             'dWout', 'dXout', 'dX1gamma', 'dX2gamma', 'dX1QKT', 'dX2QKT', 'dXQKV-fused', 'dWQKV-fused')
 
 
-def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_unread=True):
+#: the orders the library runs a feature-major configuration in (SUB_OPT_PRIVATE_LAYOUTS): weights that are
+#: copied across the boundary when the configuration names another order
+OWN_WEIGHT_ORDERS = {'WKQV': 'QHPI', 'BKQV': 'QHP', 'WO': 'IHP', 'LINW1': 'UI', 'LINW2': 'IU'}
+
+
+def staged_elements(layouts, B, L, H, E):
+    """Elements copied across the boundary per pass when the library runs a configuration in its own orders:
+    (input or output [B,J,I] tensors, weights) -- 0, 0 for a configuration whose activations are all token-major."""
+    acts = [layouts['input'][1], layouts['output'][1]] + [l for _, l in layouts['forward_interm']] \
+        + [l for _, l in layouts['backward_interm']]
+    own = {'BJI', 'BJU', 'HBJK', 'QBJHP', 'BJHP', 'BJ'}
+    if all(l in own for l in acts):
+        return 0, 0
+    U, P = 4 * E, E // H
+    numel = {'WKQV': 3 * E * E, 'BKQV': 3 * E, 'WO': E * E, 'LINW1': E * U, 'LINW2': E * U}
+    w = sum(numel[n] for n, l in layouts['params'] if n in OWN_WEIGHT_ORDERS and l != OWN_WEIGHT_ORDERS[n])
+    return B * L * E, w
+
+
+def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_unread=True, staged=(0, 0)):
     """Per operator: ('hbm', bytes) or ('mfma', flops, bytes).  Bytes = each big
     tensor read once + written once in fp16; flops = 2*batch*M*N*K.
     relu_from_output: the ReLU layer as it runs by default -- bad writes only its
@@ -101,6 +120,13 @@ def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_
         # and two score-sized tensors in, one out)
         'QKT+softmax': ('hbm', (3 * hbjk + 2 * bji) * 2), 'dX1gamma+bs': ('hbm', (3 * hbjk + 2 * bji) * 2),
     }
+    # copies across the boundary of a configuration that runs in the library's own orders: read + write
+    sa, sw = staged
+    w['relayout-in'] = ('hbm', 4 * (sa + sw))
+    w['relayout-out'] = ('hbm', 4 * sa)
+    w['relayout-in-bwd'] = ('hbm', 4 * sa)
+    w['relayout-in-again'] = ('hbm', 4 * (sa + sw))
+    w['relayout-out-bwd'] = ('hbm', 4 * (sa + sw))
     tok = B * L
     proj = (2 * tok * 3 * E * E, 2 * (tok * E + 3 * E * E + 3 * tok * E))
     attn = (2 * H * B * L * L * P, 2 * (2 * tok * E + hbjk))
@@ -758,17 +784,18 @@ def main():
         for n, mhz in enc._handle.profile_read_clocks():
             clocks.setdefault(n, []).append(mhz)
     enc._handle.profile_enable(False)
+    staged = staged_elements(enc.layouts, cfg['B'], cfg['L'], cfg['H'], cfg['E']) if '11=0' not in args.option else (0, 0)
     work = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
                             relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
                             packed_masks='9=0' not in args.option and cfg['E'] % 8 == 0,
-                            skip_unread='10=0' not in args.option)
+                            skip_unread='10=0' not in args.option, staged=staged)
     # Memory-bound launches: `achieved` and `frac` are the bytes the launch moves (each big tensor it reads
     # or writes once, the residual dropout masks as bits, outputs nothing reads not written) per second; what
     # the reference's operators would have moved for the same result (masks as fp16 tensors, every named
     # output written) is reported beside it as effective_gbps_ref_bytes.
     work_ref = algorithmic_work(cfg['B'], cfg['L'], cfg['H'], cfg['E'],
                                 relu_from_output=cfg['act'] == 'relu' and '6=0' not in args.option,
-                                packed_masks=False, skip_unread=False)
+                                packed_masks=False, skip_unread=False, staged=staged)
     raw_us = {n: statistics.mean(ts) * 1e3 for n, ts in per_op.items()}
     event_us = (statistics.median(inst) - gpu_us_per_step) / max(1, len(raw_us))
     ops = []

@@ -255,6 +255,23 @@ int sub_set_attention_mask(void* handle, const void* attn_mask, const char* layo
  * E=1024; outputs and gradients are bit-identical.  Set it to 0 (debug capture
  * does) when those tensors are wanted. */
 #define SUB_OPT_SKIP_UNREAD 10
+/* SUB_OPT_PRIVATE_LAYOUTS (default 1): when an activation of the configuration is not in the dimension
+ * order the fused paths of this library need (token-major rows with the feature dim contiguous: input,
+ * output and [B,J,I] tensors BJI, [B,J,U] tensors BJU, scores HBJK, projections QBJHP, attention output
+ * BJHP) -- the reference's shipped configurations are feature-major, chosen for V100
+ * (pytorch_module/layouts-bert-*.pickle) -- encoder_forward / encoder_backward run the whole layer in those
+ * orders: every intermediate lies in the library's order inside the caller's buffer (same number of
+ * elements), and the tensors that cross the boundary in another order (input, output, their gradients,
+ * weights, weight gradients; weights WKQV QHPI, BKQV QHP, WO IHP, LINW1 UI, LINW2 IU) are copied into it
+ * and back by a tiled transposing kernel (entries `relayout-in`, `relayout-out`, `relayout-in-bwd`,
+ * `relayout-out-bwd` of the per-launch timing).
+ * Outputs and gradients are the same to rounding; saved intermediates are NOT in the configured order
+ * (sub_tensor_layout tells the order in use).  The staged copies (input, output, two gradients, the
+ * weights and their gradients that differ) are allocated by the first calls.  A configuration whose
+ * activations are all in the library's orders runs as it is, whatever its weight orders.  0: every
+ * tensor in the configured order, through strided kernels where it must be (what debug capture and
+ * a layout search need).  The operator entry points sub_op_* always take the layouts they are given. */
+#define SUB_OPT_PRIVATE_LAYOUTS 11
 /* *planned = 1 when, with the handle's sizes, layouts and options as they are
  * now, self-attention runs with the scores in registers
  * (given 16-byte aligned tensors).  No counterpart in the reference. */
@@ -263,6 +280,10 @@ int sub_set_option(void* handle, int option, int value);
 /* The present value of an option (a caller that sized LIN1 and DROP2MASK down,
  * see SUB_OPT_RELU_FROM_OUTPUT, checks it before every call). */
 int sub_get_option(void* handle, int option, int* value);
+/* The dimension order in which encoder_forward / encoder_backward hold a tensor of the configuration
+ * ("X", "SB2" or a name of the three lists) inside its buffer: the configured one, or the library's own
+ * under SUB_OPT_PRIVATE_LAYOUTS.  out receives a NUL-terminated string of at most 8 letters. */
+int sub_tensor_layout(void* handle, const char* name, char out[16]);
 
 /* Array forms of the two calls above: ptrs holds the same pointers in the same
  * order, without the handle (n must be 37 resp. 64). */
@@ -426,6 +447,11 @@ int sub_op_ln_backward_static(void* handle, int extended, const void* in, const 
                               const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
                               const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias,
                               void* dout_bias);
+/* dst (order l_dst) = src (order l_src): the same tensor in another dimension order (any two permutations
+ * of the same dims; 128-bit accesses on both sides through 64 x 64 tiles in LDS when the sizes of the two
+ * contiguous dims are multiples of 8).  No counterpart in the reference, whose kernels are generated per
+ * layout; here it carries tensors across the boundary of SUB_OPT_PRIVATE_LAYOUTS.  src and dst must not overlap. */
+int sub_op_relayout(void* handle, const void* src, const char* l_src, void* dst, const char* l_dst);
 /* block_bei.cuh:58-106 */
 int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void* dresid1,
                const char* l_dresid1, void* dx, const char* l_dx);

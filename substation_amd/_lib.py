@@ -24,6 +24,7 @@ OPT_FINISH_IN_PAIR = 7
 OPT_SIDE_JOBS = 8
 OPT_PACKED_MASKS = 9
 OPT_SKIP_UNREAD = 10
+OPT_PRIVATE_LAYOUTS = 11
 FUSE_REQUIRED = 2
 
 
@@ -64,6 +65,7 @@ SIGNATURES = {
     'sub_set_option': (_I, [_VP, _I, _I]),
     'sub_ops_defer': (_I, [_VP, _I]),
     'sub_get_option': (_I, [_VP, ctypes.c_int, ctypes.POINTER(ctypes.c_int)]),
+    'sub_tensor_layout': (_I, [_VP, ctypes.c_char_p, ctypes.c_char_p]),
     'sub_attention_in_registers': (_I, [_VP, ctypes.POINTER(_I)]),
     'sub_encoder_forward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
     'sub_encoder_backward': (_I, [_VP, ctypes.POINTER(_VP), _I]),
@@ -91,6 +93,7 @@ SIGNATURES = {
     'sub_op_aib': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
     'sub_op_baib': (_I, [_VP, _VP, _CP, _VP, _CP]),
     'sub_op_bei': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
+    'sub_op_relayout': (_I, [_VP, _VP, _CP, _VP, _CP]),
     'sub_op_ln_backward': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP,
                                 _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
     'sub_op_ln_backward_static': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP,
@@ -219,6 +222,13 @@ class Handle:
         out = _I(0)
         check(self.lib.sub_attention_in_registers(self.ptr, ctypes.byref(out)), 'sub_attention_in_registers')
         return bool(out.value)
+
+    def tensor_layout(self, name):
+        """The dimension order in which the layer calls hold tensor ``name`` inside its buffer: the
+        configured one, or the library's own under OPT_PRIVATE_LAYOUTS."""
+        out = ctypes.create_string_buffer(16)
+        check(self.lib.sub_tensor_layout(self.ptr, name.encode(), out), 'sub_tensor_layout')
+        return out.value.decode()
 
     def profile_enable(self, on=True):
         """on: False / True, or 2 for per-launch timing plus clock samples (profile_read_clocks)."""

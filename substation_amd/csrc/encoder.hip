@@ -7,6 +7,7 @@
 
 #include <cmath>
 #include <map>
+#include <algorithm>
 #include <mutex>
 #include <string>
 #include <vector>
@@ -171,15 +172,15 @@ struct ProfEntry { const char* name; hipEvent_t a; };
 // sub_profile_enable(handle, 2): besides the event, a one-lane kernel in front of every launch stores the
 // shader clock counter (s_memtime) and the constant-rate wall clock (s_memrealtime); the ratio of their
 // differences between two samples is the shader clock the GPU held during the launch between them.
-// The shader clock counter is one per XCD and the eight do not agree, so every sample is taken on each
-// XCD (sixteen one-lane workgroups, dealt round-robin over the XCDs; each stores into the slot of the XCD
-// it finds itself on) and differences are formed per XCD.
+// The shader clock counter is one per XCD and the eight do not agree, so every sample is taken by a
+// number of one-lane workgroups (dealt round-robin over the XCDs), each storing its own pair; two
+// samples are then compared pair by pair, and only pairs from the same XCD give a ratio that a clock can
+// have (the counters of different XCDs lie far apart).
 constexpr int kMaxClockSamples = 256;
-constexpr int kClockXcds = 8;
+constexpr int kClockSlots = 32;
 __global__ void k_clock_sample(unsigned long long* slot) {
-    const unsigned xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kClockXcds - 1);     // XCC_ID, bits 3:0
-    slot[2 * xcc] = __builtin_readcyclecounter();
-    slot[2 * xcc + 1] = wall_clock64();
+    slot[2 * blockIdx.x] = __builtin_readcyclecounter();
+    slot[2 * blockIdx.x + 1] = wall_clock64();
 }
 
 struct Handle {
@@ -192,6 +193,18 @@ struct Handle {
     hipStream_t stream = nullptr;
     Layout lX, lY;
     Layout lp[SUB_N_PARAMS], lf[SUB_N_FWD], lb[SUB_N_BWD];
+    // The dimension orders the caller configured (the orders above are what the launches use: the same, or,
+    // under SUB_OPT_PRIVATE_LAYOUTS, the library's own -- see plan_layouts).
+    Layout xX, xY;
+    Layout xp[SUB_N_PARAMS], xf[SUB_N_FWD], xb[SUB_N_BWD];
+    bool private_layouts = true;      // SUB_OPT_PRIVATE_LAYOUTS
+    bool staging = false;             // the launches run in the library's own orders
+    bool stage_x = false, stage_y = false, stage_p[SUB_N_PARAMS] = {};
+    // staged copies in the library's orders: input, output, their gradients, weights and weight gradients
+    half_t* sX = nullptr; half_t* sY = nullptr; half_t* sDY = nullptr; half_t* sDX = nullptr;
+    half_t* sW[SUB_N_PARAMS] = {}; half_t* sDW[SUB_N_PARAMS] = {};
+    // what the last forward call made sX / sW from (the backward call after it reuses them for the same pointers)
+    const void* staged_x_from = nullptr; const void* staged_w_from[SUB_N_PARAMS] = {};
     int pos_p[SUB_N_PARAMS], pos_f[SUB_N_FWD], pos_b[SUB_N_BWD];   // internal id -> caller position
     Layout lKK, lQQ, lDKK, lDQQ, lWsub, lBsub;
     GemmPlan gemm[G_COUNT];
@@ -243,6 +256,8 @@ struct Handle {
         if (gws) (void)hipFree(gws);
         if (mask_plan) (void)hipFree(mask_plan);
         if (clock_buf) (void)hipFree(clock_buf);
+        for (half_t* q : {sX, sY, sDY, sDX}) if (q) (void)hipFree(q);
+        for (int i = 0; i < SUB_N_PARAMS; ++i) { if (sW[i]) (void)hipFree(sW[i]); if (sDW[i]) (void)hipFree(sDW[i]); }
         for (auto& e : prof) (void)hipEventDestroy(e.a);
         if (swapped) (void)hipThreadExchangeStreamCaptureMode(&mode);
     }
@@ -296,7 +311,7 @@ struct ProfScope {
         e.name = name;
         hip_check(hipEventRecord(e.a, h.stream), "hipEventRecord");
         if (h.profile_clocks && h.prof_used <= (size_t)kMaxClockSamples)
-            hipLaunchKernelGGL(k_clock_sample, dim3(2 * kClockXcds), dim3(1), 0, h.stream, h.clock_buf + 2 * kClockXcds * (h.prof_used - 1));
+            hipLaunchKernelGGL(k_clock_sample, dim3(kClockSlots), dim3(1), 0, h.stream, h.clock_buf + 2 * kClockSlots * (h.prof_used - 1));
         used = true;
     }
     // nothing was launched: the entry goes (its event stays in the stream, harmless)
@@ -386,6 +401,9 @@ void plan_gemm(Handle& h, int id, const Layout& a, const Layout& b, const Layout
     h.gemm[id].alpha = alpha;
 }
 
+void plan_layouts(Handle& h, bool own);
+void drop_staged(Handle& h);
+
 void configure(Handle& h, const sub_config* c) {
     if (!c) fail("sub_configure: null config");
     if (c->abi_version != SUB_ABI_VERSION) fail("sub_configure: ABI version mismatch");
@@ -403,6 +421,7 @@ void configure(Handle& h, const sub_config* c) {
         hip_check(hipFree(h.mask_plan), "hipFree(mask plan)");
     }
     h.mask_plan = nullptr; h.mask_plan_bytes = 0; h.mask_plan_built = false; h.attn_mask = nullptr;
+    drop_staged(h);
     Sizes sz;
     sz.n[dB] = c->batch; sz.n[dJ] = c->seq; sz.n[dK] = c->seq; sz.n[dH] = c->heads;
     sz.n[dP] = c->embed / c->heads; sz.n[dI] = c->embed;
@@ -412,12 +431,60 @@ void configure(Handle& h, const sub_config* c) {
     h.p_softmax = c->p_softmax; h.p_resid1 = c->p_resid1; h.p_act = c->p_act; h.p_resid2 = c->p_resid2;
     h.eps = c->ln_eps > 0.f ? c->ln_eps : 1e-5f;
     h.seed = c->seed; h.step = 0;
-    h.lX = make_layout(c->input_layout, sz);
-    h.lY = make_layout(c->output_layout, sz);
-    if (!same_dims(h.lX, "BJI") || !same_dims(h.lY, "BJI")) fail("input/output layout must be a permutation of BJI");
-    bind_tensors(kParams, c->param_names, c->param_layouts, sz, h.lp, h.pos_p, "params");
-    bind_tensors(kFwd, c->fwd_names, c->fwd_layouts, sz, h.lf, h.pos_f, "forward_interm");
-    bind_tensors(kBwd, c->bwd_names, c->bwd_layouts, sz, h.lb, h.pos_b, "backward_interm");
+    h.xX = make_layout(c->input_layout, sz);
+    h.xY = make_layout(c->output_layout, sz);
+    if (!same_dims(h.xX, "BJI") || !same_dims(h.xY, "BJI")) fail("input/output layout must be a permutation of BJI");
+    bind_tensors(kParams, c->param_names, c->param_layouts, sz, h.xp, h.pos_p, "params");
+    bind_tensors(kFwd, c->fwd_names, c->fwd_layouts, sz, h.xf, h.pos_f, "forward_interm");
+    bind_tensors(kBwd, c->bwd_names, c->bwd_layouts, sz, h.xb, h.pos_b, "backward_interm");
+    // the caller's orders must be usable as they are (debug capture and SUB_OPT_PRIVATE_LAYOUTS = 0 run in them)
+    plan_layouts(h, false);
+    if (h.private_layouts) plan_layouts(h, true);
+    h.configured = true;
+}
+
+// The dimension orders the launches run in, and everything that follows from them (contraction plans,
+// scratch sizes).  own = false: the caller's.  own = true (SUB_OPT_PRIVATE_LAYOUTS): when an activation of the
+// caller's configuration is not in the order the fused paths of this library need -- token-major rows with the
+// feature dim contiguous; the reference's shipped configurations are feature-major -- every intermediate
+// lives in the library's own order inside the caller's buffer (same number of elements), and the tensors that
+// cross the boundary (input, output, their gradients, weights, weight gradients) are copied into that order and
+// back by k_relayout.  A configuration whose activations are all in the library's orders runs as it is, with
+// its own weight orders.
+void plan_layouts(Handle& h, bool own) {
+    const Sizes& sz = h.sz;
+    static const char* const kOwnP[SUB_N_PARAMS] = {"QHPI", "QHP", "IHP", "I", "I", "I", "U", "UI", "I", "I", "I", "IU"};
+    static const char* const kOwnF[SUB_N_FWD] = {
+        "QBJHP", "QBJHP", "HBJK", "HBJK", "HBJK", "HBJK", "BJHP", "BJI", "BJI", "BJI", "BJU", "BJU", "BJU",
+        "BJI", "BJI", "BJI", "BJ", "BJI", "BJU", "BJI", "BJI", "BJ", "BJI"};
+    static const char* const kOwnB[SUB_N_BWD] = {
+        "BJI", "BJI", "BJI", "BJU", "BJU", "BJI", "BJI", "BJI", "BJI", "BJI", "BJHP", "HBJK", "HBJK", "QBJHP"};
+    bool differs = false;
+    if (own) {
+        differs = h.xX.str() != "BJI" || h.xY.str() != "BJI";
+        for (int i = 0; i < SUB_N_FWD; ++i) differs = differs || h.xf[i].str() != kOwnF[i];
+        for (int i = 0; i < SUB_N_BWD; ++i) differs = differs || h.xb[i].str() != kOwnB[i];
+    }
+    h.staging = own && differs;
+    h.stage_x = h.stage_y = false;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) h.stage_p[i] = false;
+    h.staged_x_from = nullptr;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) h.staged_w_from[i] = nullptr;
+    if (h.staging) {
+        h.lX = make_layout("BJI", sz); h.lY = make_layout("BJI", sz);
+        h.stage_x = h.xX.str() != "BJI"; h.stage_y = h.xY.str() != "BJI";
+        for (int i = 0; i < SUB_N_PARAMS; ++i) {
+            h.lp[i] = make_layout(kOwnP[i], sz);
+            h.stage_p[i] = h.xp[i].str() != kOwnP[i];
+        }
+        for (int i = 0; i < SUB_N_FWD; ++i) h.lf[i] = make_layout(kOwnF[i], sz);
+        for (int i = 0; i < SUB_N_BWD; ++i) h.lb[i] = make_layout(kOwnB[i], sz);
+    } else {
+        h.lX = h.xX; h.lY = h.xY;
+        for (int i = 0; i < SUB_N_PARAMS; ++i) h.lp[i] = h.xp[i];
+        for (int i = 0; i < SUB_N_FWD; ++i) h.lf[i] = h.xf[i];
+        for (int i = 0; i < SUB_N_BWD; ++i) h.lb[i] = h.xb[i];
+    }
 
     // Sub-tensors of the Q-stacked tensors (pytorch_module/encoder.py:318-362).
     Layout kq = drop_front(h.lf[KKQQVV], dQ);
@@ -513,7 +580,6 @@ void configure(Handle& h, const sub_config* c) {
     }
     // The fp32 scratch of the column reductions is allocated by the first
     // operator that needs it, so that configuring needs no GPU.
-    h.configured = true;
 }
 
 // ---------------------------------------------------------------------------
@@ -923,10 +989,66 @@ __global__ void k_step_increment(uint32_t* step) {
     if (threadIdx.x == 0) step[0] = step[0] + 1u;
 }
 
-void forward(Handle& h, const FwdPtrs& t) {
+// A staged copy in the library's own order (SUB_OPT_PRIVATE_LAYOUTS), allocated on first use.
+half_t* staged(Handle& h, half_t*& slot, int64_t numel, const char* what) {
+    if (!slot) {
+        refuse_capture(h, what);
+        hip_check(hipMalloc((void**)&slot, (size_t)numel * sizeof(half_t)), what);
+    }
+    return slot;
+}
+
+void drop_staged(Handle& h) {
+    bool any = h.sX || h.sY || h.sDY || h.sDX;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) any = any || h.sW[i] || h.sDW[i];
+    if (!any) return;
+    refuse_capture(h, "sub_configure");
+    for (half_t** q : {&h.sX, &h.sY, &h.sDY, &h.sDX}) if (*q) { hip_check(hipFree(*q), "hipFree(staged tensor)"); *q = nullptr; }
+    for (int i = 0; i < SUB_N_PARAMS; ++i) {
+        if (h.sW[i]) { hip_check(hipFree(h.sW[i]), "hipFree(staged weight)"); h.sW[i] = nullptr; }
+        if (h.sDW[i]) { hip_check(hipFree(h.sDW[i]), "hipFree(staged weight gradient)"); h.sDW[i] = nullptr; }
+    }
+}
+
+// The input and the weights in the library's orders: copied when `fresh`, or when the copies at hand were made
+// from other pointers than these (a backward call handed other tensors than its forward call).
+void stage_inputs(Handle& h, const void* X, void* const* W, const void*& Xs, void** Ws, bool fresh, const char* name) {
+    Xs = X;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) Ws[i] = W[i];
+    bool any = h.stage_x;
+    for (int i = 0; i < SUB_N_PARAMS; ++i) any = any || h.stage_p[i];
+    if (!any) return;
+    ProfScope ps(h, name);
+    bool launched = false;
+    if (h.stage_x) {
+        Xs = staged(h, h.sX, h.lX.numel, "hipMalloc(staged input)");
+        if (fresh || h.staged_x_from != X) {
+            launch_relayout(h.xX, h.lX, (const half_t*)X, h.sX, h.stream);
+            h.staged_x_from = X; launched = true;
+        }
+    }
+    for (int i = 0; i < SUB_N_PARAMS; ++i) {
+        if (!h.stage_p[i]) continue;
+        Ws[i] = staged(h, h.sW[i], h.lp[i].numel, "hipMalloc(staged weight)");
+        if (fresh || h.staged_w_from[i] != W[i]) {
+            launch_relayout(h.xp[i], h.lp[i], (const half_t*)W[i], h.sW[i], h.stream);
+            h.staged_w_from[i] = W[i]; launched = true;
+        }
+    }
+    if (!launched) ps.cancel();
+}
+
+void forward(Handle& h, const FwdPtrs& t0) {
     if (!h.configured) fail("encoder_forward: handle is not configured");
     h.prof_used = 0;
     h.prof_forward = 0;
+    FwdPtrs t = t0;
+    if (h.staging) {
+        const void* xs = nullptr;
+        stage_inputs(h, t0.X, t0.W, xs, t.W, true, "relayout-in");
+        t.X = const_cast<void*>(xs);
+        if (h.stage_y) t.Y = staged(h, h.sY, h.lY.numel, "hipMalloc(staged output)");
+    }
     void* const* W = t.W; void* const* F = t.F;
     AttnArgs at;
     const bool fused_attention = attention_fused(h, F, at);
@@ -1016,6 +1138,10 @@ void forward(Handle& h, const FwdPtrs& t) {
                  F[LIN2], h.lf[LIN2], F[DROP3MASK], h.lf[DROP3MASK], F[LN2DIFF], h.lf[LN2DIFF],
                  F[LN2], h.lf[LN2], t.Y, h.lY, F[LN2STD], h.lf[LN2STD], h.p_resid2, SUB_SITE_RESID2, packed_masks(h), !h.skip_unread);
     }
+    if (h.staging && h.stage_y) {
+        ProfScope ps(h, "relayout-out");
+        launch_relayout(h.lY, h.xY, (const half_t*)t.Y, (half_t*)t0.Y, h.stream);
+    }
     prof_mark_end(h);
     if (h.step_dev) {
         hipLaunchKernelGGL(k_step_increment, dim3(1), dim3(64), 0, h.stream, h.step_dev);
@@ -1026,11 +1152,25 @@ void forward(Handle& h, const FwdPtrs& t) {
     h.prof_forward = h.prof_used;
 }
 
-void backward(Handle& h, const BwdPtrs& t) {
+void backward(Handle& h, const BwdPtrs& t0) {
     if (!h.configured) fail("encoder_backward: handle is not configured");
     // the first backward call after a forward call keeps that call's entries in front of its own
     h.prof_used = h.prof_forward;
     h.prof_forward = 0;
+    BwdPtrs t = t0;
+    if (h.staging) {
+        const void* xs = nullptr;
+        stage_inputs(h, t0.X, t0.W, xs, t.W, false, "relayout-in-again");
+        t.X = const_cast<void*>(xs);
+        if (h.stage_y) {
+            ProfScope ps(h, "relayout-in-bwd");
+            t.DY = staged(h, h.sDY, h.lY.numel, "hipMalloc(staged output gradient)");
+            launch_relayout(h.xY, h.lY, (const half_t*)t0.DY, h.sDY, h.stream);
+        }
+        if (h.stage_x) t.DX = staged(h, h.sDX, h.lX.numel, "hipMalloc(staged input gradient)");
+        for (int i = 0; i < SUB_N_PARAMS; ++i)
+            if (h.stage_p[i]) t.DW[i] = staged(h, h.sDW[i], h.lp[i].numel, "hipMalloc(staged weight gradient)");
+    }
     // The five bias / scale gradients are only consumed by the caller: their
     // reductions leave fp32 partials in separate scratch regions and one launch
     // at the end of the pass finishes them all (or workgroups of the last pair of
@@ -1241,6 +1381,16 @@ void backward(Handle& h, const BwdPtrs& t) {
         ProfScope ps(h, "colfinish");
         launch_colfinish(h.deferred, h.stream);
     }
+    if (h.staging) {
+        bool any = h.stage_x;
+        for (int i = 0; i < SUB_N_PARAMS; ++i) any = any || h.stage_p[i];
+        if (any) {
+            ProfScope ps(h, "relayout-out-bwd");
+            if (h.stage_x) launch_relayout(h.lX, h.xX, (const half_t*)t.DX, (half_t*)t0.DX, h.stream);
+            for (int i = 0; i < SUB_N_PARAMS; ++i)
+                if (h.stage_p[i]) launch_relayout(h.lp[i], h.xp[i], (const half_t*)t.DW[i], (half_t*)t0.DW[i], h.stream);
+        }
+    }
     prof_mark_end(h);
 }
 
@@ -1406,6 +1556,7 @@ int sub_get_option(void* handle, int option, int* value) {
         else if (option == SUB_OPT_SIDE_JOBS) *value = h.side_jobs;
         else if (option == SUB_OPT_PACKED_MASKS) *value = h.packed_masks;
         else if (option == SUB_OPT_SKIP_UNREAD) *value = h.skip_unread;
+        else if (option == SUB_OPT_PRIVATE_LAYOUTS) *value = h.private_layouts;
         else fail("sub_get_option: unknown option");
     });
 }
@@ -1422,11 +1573,31 @@ int sub_set_option(void* handle, int option, int value) {
         else if (option == SUB_OPT_SIDE_JOBS) h.side_jobs = value & 3;
         else if (option == SUB_OPT_PACKED_MASKS) h.packed_masks = value != 0;
         else if (option == SUB_OPT_SKIP_UNREAD) h.skip_unread = value != 0;
+        else if (option == SUB_OPT_PRIVATE_LAYOUTS) {
+            h.private_layouts = value != 0;
+            if (h.configured) plan_layouts(h, h.private_layouts);
+        }
         else if (option == SUB_OPT_FUSE_ATTENTION) {
             if (value < 0 || value > SUB_FUSE_REQUIRED) fail("sub_set_option: SUB_OPT_FUSE_ATTENTION takes 0, 1 or 2");
             h.fuse_attention = value;
         }
         else fail("sub_set_option: unknown option");
+    });
+}
+
+int sub_tensor_layout(void* handle, const char* name, char out[16]) {
+    return guarded([&] {
+        Handle& h = as_handle(handle);
+        need_cfg(h);
+        if (!name || !out) fail("sub_tensor_layout: null argument");
+        std::string l;
+        if (!std::strcmp(name, "X")) l = h.lX.str();
+        else if (!std::strcmp(name, "SB2")) l = h.lY.str();
+        for (int i = 0; i < SUB_N_PARAMS && l.empty(); ++i) if (!std::strcmp(name, kParams[i].name)) l = h.lp[i].str();
+        for (int i = 0; i < SUB_N_FWD && l.empty(); ++i) if (!std::strcmp(name, kFwd[i].name)) l = h.lf[i].str();
+        for (int i = 0; i < SUB_N_BWD && l.empty(); ++i) if (!std::strcmp(name, kBwd[i].name)) l = h.lb[i].str();
+        if (l.empty()) fail(std::string("sub_tensor_layout: unknown tensor name ") + name);
+        std::snprintf(out, 16, "%s", l.c_str());
     });
 }
 
@@ -1445,9 +1616,9 @@ int sub_profile_enable(void* handle, int on) {
         h.profiling = on != 0; h.prof_used = 0;
         h.profile_clocks = on == 2;
         if (h.profile_clocks && !h.clock_buf)
-            hip_check(hipMalloc((void**)&h.clock_buf, sizeof(unsigned long long) * 2 * kClockXcds * kMaxClockSamples), "hipMalloc(clock samples)");
+            hip_check(hipMalloc((void**)&h.clock_buf, sizeof(unsigned long long) * 2 * kClockSlots * kMaxClockSamples), "hipMalloc(clock samples)");
         if (h.profile_clocks)       // a slot no workgroup wrote reads as zero and is left out
-            hip_check(hipMemset(h.clock_buf, 0, sizeof(unsigned long long) * 2 * kClockXcds * kMaxClockSamples), "hipMemset(clock samples)");
+            hip_check(hipMemset(h.clock_buf, 0, sizeof(unsigned long long) * 2 * kClockSlots * kMaxClockSamples), "hipMemset(clock samples)");
     });
 }
 
@@ -1457,7 +1628,7 @@ int sub_profile_read_clocks(void* handle, int cap, const char** names, float* mh
         Handle& h = as_handle(handle);
         if (!h.profile_clocks || !h.clock_buf) fail("sub_profile_read_clocks: enable profiling with mode 2 first");
         hip_check(hipStreamSynchronize(h.stream), "hipStreamSynchronize");
-        std::vector<unsigned long long> v(2 * kClockXcds * kMaxClockSamples);
+        std::vector<unsigned long long> v(2 * kClockSlots * kMaxClockSamples);
         hip_check(hipMemcpy(v.data(), h.clock_buf, v.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost), "hipMemcpy");
         int dev = 0, wall_khz = 0;
         hip_check(hipGetDevice(&dev), "hipGetDevice");
@@ -1465,17 +1636,22 @@ int sub_profile_read_clocks(void* handle, int cap, const char** names, float* mh
         for (size_t i = 0; i + 1 < h.prof_used && i + 1 < (size_t)kMaxClockSamples; ++i) {
             if (!h.prof[i].name) continue;
             if (count < cap) {
-                // the mean over the XCDs that both samples reached
-                double sum = 0.0; int n = 0;
-                for (int x = 0; x < kClockXcds; ++x) {
-                    const unsigned long long* a = &v[2 * (kClockXcds * i + x)];
-                    const unsigned long long* b = &v[2 * (kClockXcds * (i + 1) + x)];
-                    if (a[1] == 0 || b[1] <= a[1] || b[0] <= a[0]) continue;
-                    sum += (double)(b[0] - a[0]) / (double)(b[1] - a[1]);
-                    ++n;
+                // every pair of (slot of this sample, slot of the next) whose ratio is a possible clock
+                std::vector<double> r;
+                for (int x = 0; x < kClockSlots; ++x) {
+                    const unsigned long long* a = &v[2 * (kClockSlots * i + x)];
+                    for (int y = 0; y < kClockSlots; ++y) {
+                        const unsigned long long* b = &v[2 * (kClockSlots * (i + 1) + y)];
+                        if (b[1] <= a[1] || b[0] <= a[0]) continue;
+                        const double f = (double)(b[0] - a[0]) / (double)(b[1] - a[1]) * wall_khz * 1e-3;
+                        if (f > 300.0 && f < 3000.0) r.push_back(f);
+                    }
                 }
+                std::sort(r.begin(), r.end());
+                const int n = (int)r.size();
+                const double sum = n ? r[n / 2] * n : 0.0;        // the median
                 if (names) names[count] = h.prof[i].name;
-                if (mhz) mhz[count] = n ? (float)(sum / n * wall_khz * 1e-3) : 0.f;
+                if (mhz) mhz[count] = n ? (float)(sum / n) : 0.f;
             }
             ++count;
         }
@@ -1804,6 +1980,15 @@ int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void*
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);
         op_bei(h, dxatt, L(h, l_dxatt), dresid1, L(h, l_dresid1), dx, L(h, l_dx));
+    });
+}
+
+int sub_op_relayout(void* handle, const void* src, const char* l_src, void* dst, const char* l_dst) {
+    return guarded([&] {
+        Handle& h = as_handle(handle); need_cfg(h);
+        if (!src || !dst) fail("sub_op_relayout: null tensor pointer");
+        ProfScope ps(h, "relayout");
+        launch_relayout(L(h, l_src), L(h, l_dst), (const half_t*)src, (half_t*)dst, h.stream);
     });
 }
 

@@ -195,6 +195,10 @@ void launch_mha_mask_plan(AttnArgs& a, void* plan, bool rebuild, hipStream_t st)
 void launch_mha_backward_dq(const AttnArgs& a, int head_size, hipStream_t st);
 void launch_mha_backward_dkv(const AttnArgs& a, int head_size, hipStream_t st);
 
+// --- dimension order --------------------------------------------------------
+// dst (dense, order ld) = src (dense, order ls): the same logical tensor in another dimension order.
+void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half_t* dst, hipStream_t st);
+
 // --- tensor contraction ------------------------------------------------------
 // Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
 // that broadcasts along M or N, or a whole tensor (a residual).

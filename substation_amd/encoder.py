@@ -99,6 +99,7 @@ class Encoder(torch.nn.Module):
             self._handle.set_option(_lib.OPT_RELU_FROM_OUTPUT, 0)
             self._handle.set_option(_lib.OPT_PACKED_MASKS, 0)
             self._handle.set_option(_lib.OPT_SKIP_UNREAD, 0)
+            self._handle.set_option(_lib.OPT_PRIVATE_LAYOUTS, 0)
         # compact_attention: when self-attention runs with the scores in registers,
         # four of the six score-sized tensors ([H,B,J,K]) are never touched and the
         # other two only hold 8 resp. K/8 bytes per score row; allocate just that

@@ -93,6 +93,9 @@ class LayerTimer:
                                     activation=self.activation, seed=self.seed,
                                     intermediate_size=self.intermediate_size)
         handle = self._lib.Handle(cfg)
+        # every tensor in the order under test (by default the library would run a configuration with
+        # feature-major activations in its own orders and copy at the boundary)
+        handle.set_option(self._lib.OPT_PRIVATE_LAYOUTS, 0)
         handle.set_stream(self.torch.cuda.current_stream().cuda_stream)
         if profiling:
             handle.profile_enable(True)

@@ -165,6 +165,10 @@ class Ops:
         _lib.check(self.lib.sub_op_bei(self._pre(), _p(dxatt), _s(l_dxatt), _p(dresid1),
                                        _s(l_dresid1), _p(dx), _s(l_dx)), 'bei')
 
+    def relayout(self, src, l_src, dst, l_dst):
+        """dst (order l_dst) = src (order l_src): the same tensor in another dimension order."""
+        _lib.check(self.lib.sub_op_relayout(self._pre(), _p(src), _s(l_src), _p(dst), _s(l_dst)), 'relayout')
+
     def einsum_bad(self, a, l_a, b, l_b, bias, l_bias, lin, out, l_out, bits, p=0.0, site=2):
         """out = dropout(act(einsum(a, b) + bias)) in one launch where the product qualifies
         (then True; False: nothing was launched).  ``bits``: a uint8 tensor of numel(out) / 8

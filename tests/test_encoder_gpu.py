@@ -175,7 +175,10 @@ def run_layer_default(B, L, H, E, p, seed_data=0, w_std=0.05, step=0, attn_mask=
     gate = None
     if act == 'relu':
         names = [n for n, _ in lay['forward_interm']]
-        drop2 = from_layout(enc._workspace['forward_interm'][names.index('DROP2')], 'BJU', t['DROP2'])
+        # (the order the library holds it in: the configured one unless it runs in its own orders)
+        held = enc._handle.tensor_layout('DROP2')
+        drop2 = from_layout(enc._workspace['forward_interm'][names.index('DROP2')].reshape(-1).view(
+            [sz[d] for d in held]), 'BJU', held)
         gate = (drop2 > 0).astype(np.float64)
         assert (drop2[masks['DROP2MASK'] == 0] == 0).all(), 'DROP2 is not zero where the seeded mask drops'
     want = ref.run_named(params_np, X_np, DY_np, masks, act, relu_gate=gate, attn_mask=attn_mask)
@@ -223,6 +226,21 @@ def test_bench_path_matches_the_oracle(dims, which):
     BASELINE configs[2] (B=8 L=512) and configs[3] (B=96 L=128) with the layouts the
     benchmark uses.  Output, DX and the 12 gradients to 1e-2."""
     want, got = run_layer_default(*dims, 0.1, seed_data=17, w_std=0.02, act='relu', which=which)
+    _compare(want, got, names=OUTPUTS)
+
+
+@pytest.mark.parametrize('which,dims,act', [('bert-b8-l512-h16-e1024', (2, 128, 2, 128), 'relu'),
+                                            ('bert-b96-l128-h16-e1024', (4, 128, 4, 256), 'gelu'),
+                                            ('bert-b8-l512-h16-e1024', (8, 512, 16, 1024), 'relu')])
+def test_feature_major_configurations_run_in_the_library_own_orders(which, dims, act):
+    """Under the reference's shipped configurations (feature-major activations) the layer as shipped runs in
+    the library's own orders and copies input, output, gradients, weights and weight gradients across
+    the boundary (SUB_OPT_PRIVATE_LAYOUTS): the fused launches of the default configuration must appear,
+    and output, DX and the 12 gradients -- all in the configured orders -- must match the oracle."""
+    launches = []
+    want, got = run_layer_default(*dims, 0.1, seed_data=41, w_std=0.02, act=act, which=which, launches=launches)
+    # (the weights always cross; input and output only where the configuration has them feature-major)
+    assert 'relayout-in' in launches and 'relayout-out-bwd' in launches and 'attention' in launches, launches
     _compare(want, got, names=OUTPUTS)
 
 
@@ -517,6 +535,7 @@ def test_fused_epilogues_match_unfused(which, dims, act):
         enc = Encoder('unused', B, L, H, E, lay, torch.float16, 0.1, 0.1, 0.1, 0.1, enable_debug=debug,
                       seed=SEED, activation=act).cuda()
         enc._handle.set_option(4, 0)      # the attention kernels are compared separately (rounding differs)
+        enc._handle.set_option(11, 0)     # every tensor in the configured order in both runs (the same kernels)
         enc.set_rng(SEED, 0)
         with torch.no_grad():
             for p in enc.parameters():

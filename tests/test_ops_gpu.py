@@ -397,3 +397,23 @@ def test_ln_backward_one_launch_or_separate(B, L, H, E, extended):
         if extended:
             assert_close(dlb.float().cpu().numpy(), w[3], name='DLINEAR_BIAS')
             assert_close(dob.float().cpu().numpy(), ref.op_baob(from_layout(o2, 'BJI', lay)), name='DOUT_BIAS')
+
+
+@pytest.mark.parametrize('dims', [(2, 64, 2, 128), (3, 40, 3, 120), (2, 5, 1, 20), (8, 512, 16, 1024)])
+def test_relayout_is_a_permutation_of_the_same_tensor(dims):
+    """sub_op_relayout against a permuted copy, bit for bit: tiled transposes (the contiguous dim changes),
+    vector copies (it stays), the scalar path (sizes that are not multiples of 8), five dims."""
+    B, L, H, E = dims
+    o = _ops(B, L, H, E)
+    g = torch.Generator(device='cuda').manual_seed(11)
+    cases = [('BJI', 'IBJ'), ('IBJ', 'BJI'), ('JBI', 'BJI'), ('BJU', 'UBJ'), ('QPHBJ', 'QBJHP'), ('QBJHP', 'QPHBJ'),
+             ('QPHI', 'QHPI'), ('IPH', 'IHP'), ('UI', 'IU'), ('HBJK', 'KJBH')]
+    if B * L * E > 1 << 20:
+        cases = cases[:5]
+    for l_src, l_dst in cases:
+        src = o.empty(l_src).normal_(0.0, 1.0, generator=g)
+        dst = o.empty(l_dst).fill_(float('nan'))
+        o.relayout(src, l_src, dst, l_dst)
+        torch.cuda.synchronize()
+        want = src.permute([l_src.index(d) for d in l_dst]).contiguous()
+        assert torch.equal(dst, want), (dims, l_src, l_dst)

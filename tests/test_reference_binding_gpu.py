@@ -91,7 +91,14 @@ def test_positional_exports_through_the_reference_binding(which):
                                        ('DROP2MASK', (B, S, U), 2), ('DROP3MASK', (B, S, E), 3))}
     names = [n for n, _ in lay['forward_interm']]
     layouts_f = dict(lay['forward_interm'])
-    drop2 = from_layout(fwd[names.index('DROP2')], 'BJU', layouts_f['DROP2'])
+    # (the intermediates lie in the order sub_tensor_layout names: the configured one, or, for a configuration
+    # with feature-major activations, the library's own)
+    held = ctypes.create_string_buffer(16)
+    lib.sub_tensor_layout.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_char_p]
+    assert lib.sub_tensor_layout(handle, b'DROP2', held) == 0, lib.sub_last_error()
+    held = held.value.decode()
+    assert held == ('BJU' if which != 'mi355x' else layouts_f['DROP2'])
+    drop2 = from_layout(fwd[names.index('DROP2')].reshape(-1).view([sizes[d] for d in held]), 'BJU', held)
     assert (drop2[masks['DROP2MASK'] == 0] == 0).all()
     # by default the residual dropout masks travel as one bit per element, canonical order, in
     # the first B*J*I/8 bytes of their buffers (SUB_OPT_PACKED_MASKS)
