@@ -146,6 +146,7 @@ def algorithmic_work(B, L, H, E, relu_from_output=True, packed_masks=True, skip_
     w['attention-bwd-dKdV'] = ('mfma', 4 * attn[0], 2 * 6 * bji + hbjk // 8, 2 * attn[0])
     # two products in one launch
     w['dXlin1+dWlin1'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
+    w['dWlin1+dWlin2'] = ('mfma', 2 * ffn[0], 2 * ffn[1])
     w['dXQKV-fused+dWQKV-fused'] = ('mfma', 2 * proj[0], 2 * proj[1])
     w['dXout+dWout'] = ('mfma', 2 * outp[0], 2 * outp[1])
     # the last launch of the backward pass with dWout's tiles in the places it leaves free

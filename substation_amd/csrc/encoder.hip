@@ -650,6 +650,17 @@ bool pair_takes_third(Handle& h, int id1, const void* A1, const void* B1, void* 
                                  (half_t*)C2, GemmEpilogue{}, h.gws, h.gws_floats, third);
 }
 
+// Would run_gemm_pair run these two products as one launch?
+bool pair_ok(Handle& h, int id1, const void* A1, const void* B1, void* C1, const void* addend1, int id2,
+             const void* A2, const void* B2, void* C2) {
+    if (!h.pair_products) return false;
+    const GemmPlan& p1 = h.gemm[id1];
+    const GemmPlan& p2 = h.gemm[id2];
+    ensure_gws(h, h.gws_need);
+    return gemm_pair_ok(p1.shape, (const half_t*)A1, (const half_t*)B1, (half_t*)C1, addend_epilogue(p1, addend1),
+                        p2.shape, (const half_t*)A2, (const half_t*)B2, (half_t*)C2, GemmEpilogue{}, h.gws, h.gws_floats);
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 void op_softmax(Handle& h, const void* beta, const Layout& lb, void* alpha, const Layout& la,
@@ -1249,7 +1260,14 @@ void backward(Handle& h, const BwdPtrs& t0) {
     } else {
         run_gemm(h, G_DXLIN2, D[DLIN2], W[LINW2], D[DDROP2], "dXlin2");
     }
-    run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
+    // With many tokens the data gradient of linear1 has too many tiles to share a launch with the weight
+    // gradient next to it; the two weight gradients of the feed-forward block -- one tile per CU each, their
+    // contraction as long as the token count -- then run as a pair of their own on 256 x 128 tiles (a quarter
+    // less operand traffic from L2 than alone on 128 x 128 tiles), dWlin2 waiting for dWlin1's operands.
+    const bool pair_weights = !pair_ok(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], nullptr, G_DWLIN1, D[DLIN1], F[SB1],
+                                       DW[LINW1]) &&
+                              pair_ok(h, G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], nullptr, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2]);
+    if (!pair_weights) run_gemm(h, G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2");
     if (!fuse_bdrlb) {
         ProfScope ps(h, "bdrlb");
         if (relu_from_output(h))
@@ -1258,8 +1276,14 @@ void backward(Handle& h, const BwdPtrs& t0) {
             op_bdrlb(h, D[DDROP2], h.lb[DDROP2], F[DROP2MASK], h.lf[DROP2MASK], F[LIN1], h.lf[LIN1],
                      D[DLIN1], h.lb[DLIN1], DW[LINB1]);
     }
-    run_gemm_pair(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1", nullptr,
-                  G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1", "dXlin1+dWlin1");
+    if (pair_weights) {
+        run_gemm(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1");
+        run_gemm_pair(h, G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1", nullptr,
+                      G_DWLIN2, D[DLIN2], F[DROP2], DW[LINW2], "dWlin2", "dWlin1+dWlin2");
+    } else {
+        run_gemm_pair(h, G_DXLIN1, D[DLIN1], W[LINW1], D[DLIN1_LINW1], "dXlin1", nullptr,
+                      G_DWLIN1, D[DLIN1], F[SB1], DW[LINW1], "dWlin1", "dXlin1+dWlin1");
+    }
     fused = false;
     if (h.fuse_ln_backward) {
         ProfScope ps(h, "ebsb+blnrd2+baob");

@@ -1344,6 +1344,15 @@ bool gemm_pair_takes_third(const GemmShape& s1, const half_t* A1, const half_t* 
     return pair_select(sh, c, ws, ws_floats, &third, sel) && sel.n3 > 0;
 }
 
+bool gemm_pair_ok(const GemmShape& s1, const half_t* A1, const half_t* B1, half_t* C1, const GemmEpilogue& ep1,
+                  const GemmShape& s2, const half_t* A2, const half_t* B2, half_t* C2, const GemmEpilogue& ep2,
+                  float* ws, size_t ws_floats) {
+    const GemmShape* sh[2] = {&s1, &s2};
+    const Canon c[2] = {canonicalise(s1, A1, B1, C1, 1.f, ep1), canonicalise(s2, A2, B2, C2, 1.f, ep2)};
+    PairSel sel;
+    return pair_select(sh, c, ws, ws_floats, nullptr, sel);
+}
+
 // Two independent products in one launch (see k_gemm_pair).  Returns false, having
 // launched nothing, unless both are products the register-staged kernel would take
 // as whole 128x128 tiles with about one tile per CU, in an operand orientation

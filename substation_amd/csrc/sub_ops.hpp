@@ -271,6 +271,10 @@ bool launch_gemm_pair(const GemmShape& g1, const half_t* A1, const half_t* B1, h
                       const GemmEpilogue& ep1, const GemmShape& g2, const half_t* A2, const half_t* B2,
                       half_t* C2, float alpha2, const GemmEpilogue& ep2, hipStream_t st, float* ws = nullptr,
                       size_t ws_floats = 0, FinishJobs* tail = nullptr, PairThird* third = nullptr);
+// Would launch_gemm_pair take these two products as one launch?
+bool gemm_pair_ok(const GemmShape& g1, const half_t* A1, const half_t* B1, half_t* C1, const GemmEpilogue& ep1,
+                  const GemmShape& g2, const half_t* A2, const half_t* B2, half_t* C2, const GemmEpilogue& ep2,
+                  float* ws, size_t ws_floats);
 // Would launch_gemm_pair with these two products take `third` along?
 bool gemm_pair_takes_third(const GemmShape& g1, const half_t* A1, const half_t* B1, half_t* C1,
                            const GemmEpilogue& ep1, const GemmShape& g2, const half_t* A2, const half_t* B2,

@@ -37,6 +37,8 @@ OPERATORS = [
     ('dXlin2+bdrlb', 'bwd', ('DLIN2', 'LINW2', 'DROP2', 'LIN1', 'DLIN1')),    # GELU: LIN1 and keep bits, not DROP2
     ('bdrlb', 'bwd', ('DDROP2', 'DROP2MASK', 'LIN1', 'DROP2', 'DLIN1')),      # ReLU: the gate is read off DROP2
     ('dXlin1+dWlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1', 'SB1')),
+    # many tokens: the two weight gradients of the feed-forward block as a pair, dXlin1 alone
+    ('dWlin1+dWlin2', 'bwd', ('DLIN1', 'SB1', 'LINW1', 'DLIN2', 'DROP2', 'LINW2')),
     ('dXlin1', 'bwd', ('DLIN1', 'LINW1', 'DLIN1_LINW1')),
     ('dWlin1', 'bwd', ('DLIN1', 'SB1', 'LINW1')),
     ('ebsb+blnrd2+baob', 'bwd', ('LN1', 'DRESID2', 'DLIN1_LINW1', 'DLIN2', 'DLN1', 'LN1STD', 'LN1DIFF',
@@ -78,8 +80,8 @@ ALTERNATIVES = [
     ('dXQKV-fused+dWQKV-fused+dWout', 'dXQKV-fused+dWQKV-fused', 'dXQKV-fused', 'dWQKV-fused', 'bei',
      'dXout+dWout', 'dXout', 'dWout', 'colfinish'),
     ('lin1+bad', 'lin1', 'bad'),
-    ('dXlin2+bdrlb', 'dXlin2', 'bdrlb'),
-    ('dXlin1+dWlin1', 'dXlin1', 'dWlin1'),
+    # (dWlin2 waits for dWlin1 when the two run as a pair)
+    ('dXlin2+bdrlb', 'dXlin2', 'bdrlb', 'dXlin1+dWlin1', 'dWlin1+dWlin2', 'dXlin1', 'dWlin1', 'dWlin2'),
     ('attention', 'QKT+softmax', 'QKT', 'softmax', 'gamma'),
     ('attention-bwd-dQ', 'attention-bwd-dKdV', 'dX2gamma', 'dX1gamma+bs', 'dX1gamma', 'bs', 'dX1QKT', 'dX2QKT',
      'baib'),
