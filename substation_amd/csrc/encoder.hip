@@ -1030,23 +1030,25 @@ void stage_inputs(Handle& h, const void* X, void* const* W, const void*& Xs, voi
     for (int i = 0; i < SUB_N_PARAMS; ++i) any = any || h.stage_p[i];
     if (!any) return;
     ProfScope ps(h, name);
-    bool launched = false;
+    RelayoutJob jobs[1 + SUB_N_PARAMS];
+    int n = 0;
     if (h.stage_x) {
         Xs = staged(h, h.sX, h.lX.numel, "hipMalloc(staged input)");
         if (fresh || h.staged_x_from != X) {
-            launch_relayout(h.xX, h.lX, (const half_t*)X, h.sX, h.stream);
-            h.staged_x_from = X; launched = true;
+            jobs[n++] = RelayoutJob{h.xX, h.lX, (const half_t*)X, h.sX};
+            h.staged_x_from = X;
         }
     }
     for (int i = 0; i < SUB_N_PARAMS; ++i) {
         if (!h.stage_p[i]) continue;
         Ws[i] = staged(h, h.sW[i], h.lp[i].numel, "hipMalloc(staged weight)");
         if (fresh || h.staged_w_from[i] != W[i]) {
-            launch_relayout(h.xp[i], h.lp[i], (const half_t*)W[i], h.sW[i], h.stream);
-            h.staged_w_from[i] = W[i]; launched = true;
+            jobs[n++] = RelayoutJob{h.xp[i], h.lp[i], (const half_t*)W[i], h.sW[i]};
+            h.staged_w_from[i] = W[i];
         }
     }
-    if (!launched) ps.cancel();
+    if (n) launch_relayout_batch(jobs, n, h.stream);     // one launch for all of them
+    else ps.cancel();
 }
 
 void forward(Handle& h, const FwdPtrs& t0) {
@@ -1410,9 +1412,12 @@ void backward(Handle& h, const BwdPtrs& t0) {
         for (int i = 0; i < SUB_N_PARAMS; ++i) any = any || h.stage_p[i];
         if (any) {
             ProfScope ps(h, "relayout-out-bwd");
-            if (h.stage_x) launch_relayout(h.lX, h.xX, (const half_t*)t.DX, (half_t*)t0.DX, h.stream);
+            RelayoutJob jobs[1 + SUB_N_PARAMS];
+            int n = 0;
+            if (h.stage_x) jobs[n++] = RelayoutJob{h.lX, h.xX, (const half_t*)t.DX, (half_t*)t0.DX};
             for (int i = 0; i < SUB_N_PARAMS; ++i)
-                if (h.stage_p[i]) launch_relayout(h.lp[i], h.xp[i], (const half_t*)t.DW[i], (half_t*)t0.DW[i], h.stream);
+                if (h.stage_p[i]) jobs[n++] = RelayoutJob{h.lp[i], h.xp[i], (const half_t*)t.DW[i], (half_t*)t0.DW[i]};
+            launch_relayout_batch(jobs, n, h.stream);
         }
     }
     prof_mark_end(h);

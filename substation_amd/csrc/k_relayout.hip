@@ -29,10 +29,8 @@ struct RelayoutArgs {
 
 constexpr int TILE = 64, PITCH = TILE + 2;      // halves; the odd word pitch spreads a column over the banks
 
-__global__ __launch_bounds__(256) void k_relayout_tiled(RelayoutArgs a) {
-    __shared__ half_t tile[TILE * PITCH];
+__device__ __forceinline__ void relayout_tiled(const RelayoutArgs& a, unsigned b, half_t* tile) {
     const int t0 = (a.n[0] + TILE - 1) / TILE, t1 = (a.n[1] + TILE - 1) / TILE;
-    unsigned b = blockIdx.x;
     const int i0 = (int)(b % t0) * TILE; b /= t0;
     const int i1 = (int)(b % t1) * TILE; b /= t1;
     long so = 0, dofs = 0;
@@ -66,8 +64,10 @@ __global__ __launch_bounds__(256) void k_relayout_tiled(RelayoutArgs a) {
 }
 
 // dim 0 contiguous on both sides: one 8-pack per thread, offsets from the other dims' strides
-__global__ __launch_bounds__(256) void k_relayout_vector(RelayoutArgs a, long packs) {
-    long q = (long)blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void relayout_vector(const RelayoutArgs& a, unsigned block) {
+    long packs = a.n[0] / 8;
+    for (int d = 1; d < a.rank; ++d) packs *= a.n[d];
+    long q = (long)block * 256 + threadIdx.x;
     if (q >= packs) return;
     const int p0 = a.n[0] / 8;
     long so = (q % p0) * 8, dofs = so;
@@ -79,8 +79,10 @@ __global__ __launch_bounds__(256) void k_relayout_vector(RelayoutArgs a, long pa
     *reinterpret_cast<h8*>(a.dst + dofs) = *reinterpret_cast<const h8*>(a.src + so);
 }
 
-__global__ __launch_bounds__(256) void k_relayout_scalar(RelayoutArgs a, long total) {
-    long q = (long)blockIdx.x * 256 + threadIdx.x;
+__device__ __forceinline__ void relayout_scalar(const RelayoutArgs& a, unsigned block) {
+    long total = 1;
+    for (int d = 0; d < a.rank; ++d) total *= a.n[d];
+    long q = (long)block * 256 + threadIdx.x;
     if (q >= total) return;
     long so = 0, dofs = 0;
     for (int d = 0; d < a.rank; ++d) {
@@ -90,12 +92,30 @@ __global__ __launch_bounds__(256) void k_relayout_scalar(RelayoutArgs a, long to
     a.dst[dofs] = a.src[so];
 }
 
-}  // namespace
+// Several tensors in one launch: workgroups first[j] .. first[j+1]-1 copy tensor j.
+constexpr int kMaxJobs = 8;
+enum { MODE_TILED = 0, MODE_VECTOR = 1, MODE_SCALAR = 2 };
+struct RelayoutBatch {
+    RelayoutArgs a[kMaxJobs];
+    int mode[kMaxJobs];
+    unsigned first[kMaxJobs + 1];
+    int n;
+};
 
-void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half_t* dst, hipStream_t st) {
+__global__ __launch_bounds__(256) void k_relayout(RelayoutBatch b) {
+    __shared__ half_t tile[TILE * PITCH];
+    int j = 0;
+    while (j + 1 < b.n && blockIdx.x >= b.first[j + 1]) ++j;
+    const unsigned block = blockIdx.x - b.first[j];
+    if (b.mode[j] == MODE_TILED) relayout_tiled(b.a[j], block, tile);
+    else if (b.mode[j] == MODE_VECTOR) relayout_vector(b.a[j], block);
+    else relayout_scalar(b.a[j], block);
+}
+
+// How tensor (ls -> ld) is copied and by how many workgroups.
+unsigned plan_relayout(const Layout& ls, const Layout& ld, const half_t* src, half_t* dst, RelayoutArgs& a, int& mode) {
     if (ls.rank != ld.rank || ls.numel != ld.numel) fail("relayout: the two layouts do not name the same tensor");
     if (ls.rank > kMaxRank) fail("relayout: more than five dimensions");
-    if (ls.numel == 0) return;
     int cs = -1, cd = -1;           // the logical dims with unit stride (the innermost of extent > 1, else the last)
     for (int i = 0; i < ls.rank; ++i) {
         if (!ld.has[ls.dims[i]] || ld.size[ls.dims[i]] != ls.size[ls.dims[i]])
@@ -103,7 +123,6 @@ void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half
         if (ls.stride[ls.dims[i]] == 1) cs = ls.dims[i];
         if (ld.stride[ld.dims[i]] == 1) cd = ld.dims[i];
     }
-    RelayoutArgs a;
     a.src = src; a.dst = dst; a.rank = ls.rank;
     int order[kMaxRank], k = 0;
     order[k++] = cs;
@@ -117,29 +136,50 @@ void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half
     const bool aligned = ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0;
     bool vec = aligned && a.n[0] % 8 == 0;
     for (int i = 1; i < a.rank; ++i) vec = vec && a.ss[i] % 8 == 0;
+    long blocks;
     if (cd == cs) {
         for (int i = 1; i < a.rank; ++i) vec = vec && a.sd[i] % 8 == 0;
-        if (vec) {
-            const long packs = ls.numel / 8;
-            hipLaunchKernelGGL(k_relayout_vector, dim3((unsigned)((packs + 255) / 256)), dim3(256), 0, st, a, packs);
-            check_launch("relayout (vector)");
-            return;
-        }
+        mode = vec ? MODE_VECTOR : MODE_SCALAR;
+        blocks = ((vec ? ls.numel / 8 : ls.numel) + 255) / 256;
     } else {
         vec = vec && a.n[1] % 8 == 0 && a.sd[0] % 8 == 0;
         for (int i = 2; i < a.rank; ++i) vec = vec && a.sd[i] % 8 == 0;
+        mode = vec ? MODE_TILED : MODE_SCALAR;
         if (vec) {
-            long blocks = (long)((a.n[0] + TILE - 1) / TILE) * ((a.n[1] + TILE - 1) / TILE);
+            blocks = (long)((a.n[0] + TILE - 1) / TILE) * ((a.n[1] + TILE - 1) / TILE);
             for (int i = 2; i < a.rank; ++i) blocks *= a.n[i];
-            if (blocks > 0x7fffffffL) fail("relayout: tensor too large");
-            hipLaunchKernelGGL(k_relayout_tiled, dim3((unsigned)blocks), dim3(256), 0, st, a);
-            check_launch("relayout (tiled)");
-            return;
+        } else {
+            blocks = (ls.numel + 255) / 256;
         }
     }
-    const long total = ls.numel;
-    hipLaunchKernelGGL(k_relayout_scalar, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, a, total);
-    check_launch("relayout (scalar)");
+    if (blocks > 0x3fffffffL) fail("relayout: tensor too large");
+    return (unsigned)blocks;
+}
+
+}  // namespace
+
+void launch_relayout_batch(const RelayoutJob* jobs, int n, hipStream_t st) {
+    int done = 0;
+    while (done < n) {
+        RelayoutBatch b;
+        b.n = 0; b.first[0] = 0;
+        while (done < n && b.n < kMaxJobs) {
+            const RelayoutJob& j = jobs[done++];
+            if (j.ls.numel == 0) continue;
+            const unsigned blocks = plan_relayout(j.ls, j.ld, j.src, j.dst, b.a[b.n], b.mode[b.n]);
+            if ((unsigned long)b.first[b.n] + blocks > 0x7fffffffUL) fail("relayout: too many workgroups in one launch");
+            b.first[b.n + 1] = b.first[b.n] + blocks;
+            ++b.n;
+        }
+        if (b.n == 0) continue;
+        hipLaunchKernelGGL(k_relayout, dim3(b.first[b.n]), dim3(256), 0, st, b);
+        check_launch("relayout");
+    }
+}
+
+void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half_t* dst, hipStream_t st) {
+    RelayoutJob j{ls, ld, src, dst};
+    launch_relayout_batch(&j, 1, st);
 }
 
 }  // namespace sub

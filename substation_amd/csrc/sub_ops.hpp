@@ -198,6 +198,9 @@ void launch_mha_backward_dkv(const AttnArgs& a, int head_size, hipStream_t st);
 // --- dimension order --------------------------------------------------------
 // dst (dense, order ld) = src (dense, order ls): the same logical tensor in another dimension order.
 void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half_t* dst, hipStream_t st);
+// Several tensors in one launch (eight to a launch).
+struct RelayoutJob { Layout ls, ld; const half_t* src; half_t* dst; };
+void launch_relayout_batch(const RelayoutJob* jobs, int n, hipStream_t st);
 
 // --- tensor contraction ------------------------------------------------------
 // Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
