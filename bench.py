@@ -530,6 +530,31 @@ def bench_fused_ops(args):
     print(json.dumps(out))
 
 
+def bench_fetch_probe(args):
+    """What 256 CUs draw from the L2s and from beyond them (sub_probe_fetch): a table on stdout, one line
+    per working set and load form.  The contraction kernels' operand fetch is priced against these rates."""
+    import ctypes
+    import torch
+    from substation_amd import _lib
+    lib = _lib.load()
+    cap = 1 << 30
+    buf = torch.empty(cap, dtype=torch.uint8, device='cuda').fill_(1)
+    torch.cuda.synchronize()
+    us, mhz = ctypes.c_float(), ctypes.c_float()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    print(f'{"working set":>12s}  {"load form":20s} {"workgroups":>10s} {"us":>8s} {"TB/s":>6s} {"GB/s per CU":>11s} {"MHz":>5s} {"bytes/clk per CU":>16s}')
+    rows = [(ws, form, 256) for ws in (1 << 20, 2 << 20, 8 << 20, 32 << 20, 128 << 20, 1 << 30) for form in (1, 0)]
+    rows += [(2 << 20, 1, 64), (2 << 20, 1, 8)]
+    iters = 64
+    for ws, to_lds, wgs in rows:
+        _lib.check(lib.sub_probe_fetch(ctypes.c_void_p(buf.data_ptr()), ws, to_lds, iters, wgs, stream, ctypes.byref(us),
+                                       ctypes.byref(mhz)), 'sub_probe_fetch')
+        nbytes = 65536.0 * iters * wgs
+        print(f'{ws / 2**20:8.0f} MiB  {"asynchronous to LDS" if to_lds else "128-bit to registers":20s} {wgs:10d} {us.value:8.1f} '
+              f'{nbytes / us.value / 1e6:6.2f} {nbytes / us.value / 1e3 / wgs:11.1f} {mhz.value:5.0f} '
+              f'{nbytes / wgs / (us.value * mhz.value):16.1f}')
+
+
 def bench_decoder(cfg, args):
     """Forward + backward of substation_amd.DecoderLayer (substation/transformer.py:288-441), not the headline
     metric: one JSON line of its own."""
@@ -693,6 +718,8 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE readings')
+    ap.add_argument('--fetch-probe', action='store_true',
+                    help='measure what the CUs draw from the L2s and from beyond them (a table, no JSON line)')
     ap.add_argument('--activation', choices=['relu', 'gelu'], default=None,
                     help="the feed-forward activation, instead of the configuration's own (then named in config.workload)")
     ap.add_argument('--decoder', action='store_true',
@@ -709,6 +736,9 @@ def main():
         print('bench.py: no GPU visible', file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
+    if args.fetch_probe:
+        bench_fetch_probe(args)
+        return
     if args.config == 2:
         bench_fused_ops(args)
         return

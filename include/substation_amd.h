@@ -447,6 +447,16 @@ int sub_op_ln_backward_static(void* handle, int extended, const void* in, const 
                               const char* l_g, void* d_ln_in, const char* l_d_ln_in, void* d_drop_in,
                               const char* l_d_drop_in, void* dscale, void* dbias, void* dlinear_bias,
                               void* dout_bias);
+/* Measurement only, no counterpart in the reference and no handle: `workgroups` workgroups of eight waves
+ * (one per CU at 256) each read `iters` chunks of 64 KiB -- the operand bytes of one k-step of a 256 x 256
+ * tile -- from the `working_set` bytes at buf (device memory, a multiple of 64 KiB), with asynchronous loads
+ * into LDS (to_lds != 0) or plain 128-bit loads into registers, every workgroup from a start of its own.
+ * A working set below one XCD's 4 MiB of L2 measures what the L2s deliver to the CUs, a larger one the path
+ * beyond them.  *us = duration of the launch (second of two), *mhz = shader clock during it (median over the
+ * workgroups of cycle counter / wall counter).  Bytes read = workgroups x iters x 65536.  Allocates and frees a
+ * few KiB per call and synchronises the stream. */
+int sub_probe_fetch(const void* buf, size_t working_set, int to_lds, int iters, int workgroups, void* stream,
+                    float* us, float* mhz);
 /* dst (order l_dst) = src (order l_src): the same tensor in another dimension order (any two permutations
  * of the same dims; 128-bit accesses on both sides through 64 x 64 tiles in LDS when the sizes of the two
  * contiguous dims are multiples of 8).  No counterpart in the reference, whose kernels are generated per

@@ -94,6 +94,8 @@ SIGNATURES = {
     'sub_op_baib': (_I, [_VP, _VP, _CP, _VP, _CP]),
     'sub_op_bei': (_I, [_VP, _VP, _CP, _VP, _CP, _VP, _CP]),
     'sub_op_relayout': (_I, [_VP, _VP, _CP, _VP, _CP]),
+    'sub_probe_fetch': (_I, [_VP, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, _VP, ctypes.POINTER(ctypes.c_float),
+                        ctypes.POINTER(ctypes.c_float)]),
     'sub_op_ln_backward': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP,
                                 _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _VP, _VP, _VP]),
     'sub_op_ln_backward_static': (_I, [_VP, ctypes.c_int, _VP, _CP, _VP, _VP, _CP, _VP, _CP, _VP, _CP, _VP, _CP, _VP,

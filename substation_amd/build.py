@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, 'csrc')
 OBJ = os.path.join(CSRC, 'build')
 LIB_DIR = os.path.join(HERE, 'lib')
 LIB = os.path.join(LIB_DIR, 'libsubstation_amd.so')
-SOURCES = ['encoder.hip', 'k_rows.hip', 'k_elem.hip', 'k_cols.hip', 'k_lnbwd.hip', 'k_attn.hip', 'k_mha.hip', 'k_relayout.hip', 'k_gemm.hip']
+SOURCES = ['encoder.hip', 'k_rows.hip', 'k_elem.hip', 'k_cols.hip', 'k_lnbwd.hip', 'k_attn.hip', 'k_mha.hip', 'k_relayout.hip', 'k_probe.hip', 'k_gemm.hip']
 FLAGS = ['--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-Wall', '-Wno-unused-function',
          # packed-fp32 VALU forms are switched off for every kernel of this library
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']

@@ -2012,6 +2012,44 @@ int sub_op_bei(void* handle, const void* dxatt, const char* l_dxatt, const void*
     });
 }
 
+int sub_probe_fetch(const void* buf, size_t working_set, int to_lds, int iters, int workgroups, void* stream,
+                    float* us, float* mhz) {
+    return guarded([&] {
+        hipStream_t st = (hipStream_t)stream;
+        unsigned long long* stamps = nullptr;
+        int* sink = nullptr;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        hip_check(hipMalloc(&stamps, sizeof(unsigned long long) * 4 * (size_t)(workgroups > 0 ? workgroups : 1)), "hipMalloc");
+        hip_check(hipMalloc(&sink, 4096), "hipMalloc");
+        hip_check(hipEventCreate(&e0), "hipEventCreate");
+        hip_check(hipEventCreate(&e1), "hipEventCreate");
+        auto release = [&] { (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); (void)hipFree(stamps); (void)hipFree(sink); };
+        try {
+            float ms = 0.f;
+            for (int rep = 0; rep < 2; ++rep) {       // the second launch is the one measured
+                hip_check(hipEventRecord(e0, st), "hipEventRecord");
+                launch_fetch_probe(buf, working_set, to_lds != 0, iters, workgroups, stamps, sink, st);
+                hip_check(hipEventRecord(e1, st), "hipEventRecord");
+                hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
+                hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+            }
+            std::vector<unsigned long long> v(4 * (size_t)workgroups);
+            hip_check(hipMemcpy(v.data(), stamps, v.size() * sizeof(unsigned long long), hipMemcpyDeviceToHost), "hipMemcpy");
+            int dev = 0, wall_khz = 0;
+            hip_check(hipGetDevice(&dev), "hipGetDevice");
+            hip_check(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, dev), "hipDeviceGetAttribute");
+            std::vector<double> f;
+            for (int b = 0; b < workgroups; ++b)
+                if (v[4 * b + 3] > v[4 * b + 1] && v[4 * b + 2] > v[4 * b])
+                    f.push_back((double)(v[4 * b + 2] - v[4 * b]) / (double)(v[4 * b + 3] - v[4 * b + 1]) * wall_khz * 1e-3);
+            std::sort(f.begin(), f.end());
+            if (us) *us = ms * 1e3f;
+            if (mhz) *mhz = f.empty() ? 0.f : (float)f[f.size() / 2];
+        } catch (...) { release(); throw; }
+        release();
+    });
+}
+
 int sub_op_relayout(void* handle, const void* src, const char* l_src, void* dst, const char* l_dst) {
     return guarded([&] {
         Handle& h = as_handle(handle); need_cfg(h);

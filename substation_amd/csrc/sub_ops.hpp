@@ -202,6 +202,13 @@ void launch_relayout(const Layout& ls, const Layout& ld, const half_t* src, half
 struct RelayoutJob { Layout ls, ld; const half_t* src; half_t* dst; };
 void launch_relayout_batch(const RelayoutJob* jobs, int n, hipStream_t st);
 
+// --- measurement --------------------------------------------------------------
+// `workgroups` workgroups of eight waves each read `iters` chunks of 64 KiB from a working set of
+// `working_set` bytes at buf (into LDS with asynchronous loads, or into registers); every workgroup leaves
+// (cycle counter, wall counter) at its start and end in stamps[4 * workgroup ..].
+void launch_fetch_probe(const void* buf, size_t working_set, bool to_lds, int iters, int workgroups,
+                        unsigned long long* stamps, int* sink, hipStream_t st);
+
 // --- tensor contraction ------------------------------------------------------
 // Optional addend of the output: C = fp16(fp16(alpha * A.B) + addend), a bias
 // that broadcasts along M or N, or a whole tensor (a residual).
