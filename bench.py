@@ -545,14 +545,18 @@ def bench_fetch_probe(args):
     print(f'{"working set":>12s}  {"load form":20s} {"workgroups":>10s} {"us":>8s} {"TB/s":>6s} {"GB/s per CU":>11s} {"MHz":>5s} {"bytes/clk per CU":>16s}')
     rows = [(ws, form, 256) for ws in (1 << 20, 2 << 20, 8 << 20, 32 << 20, 128 << 20, 1 << 30) for form in (1, 0)]
     rows += [(2 << 20, 1, 64), (2 << 20, 1, 8)]
-    iters = 64
-    for ws, to_lds, wgs in rows:
-        _lib.check(lib.sub_probe_fetch(ctypes.c_void_p(buf.data_ptr()), ws, to_lds, iters, wgs, stream, ctypes.byref(us),
+    # copy and fill of tensor-sized regions, every chunk once, at several occupancies (workgroups x iterations = chunks)
+    rows += [(ws, form, wgs) for ws in (8 << 20, 64 << 20, 512 << 20) for form in (2, 3) for wgs in (128, 256, 1024)
+             if wgs <= ws // 65536 and (wgs == 128) == (ws == 8 << 20)]
+    names = {0: '128-bit to registers', 1: 'asynchronous to LDS', 2: 'copy (read + write)', 3: 'fill (write)'}
+    for ws, form, wgs in rows:
+        iters = 64 if form < 2 else max(1, ws // 65536 // wgs)
+        _lib.check(lib.sub_probe_fetch(ctypes.c_void_p(buf.data_ptr()), ws, form, iters, wgs, stream, ctypes.byref(us),
                                        ctypes.byref(mhz)), 'sub_probe_fetch')
-        nbytes = 65536.0 * iters * wgs
-        print(f'{ws / 2**20:8.0f} MiB  {"asynchronous to LDS" if to_lds else "128-bit to registers":20s} {wgs:10d} {us.value:8.1f} '
-              f'{nbytes / us.value / 1e6:6.2f} {nbytes / us.value / 1e3 / wgs:11.1f} {mhz.value:5.0f} '
-              f'{nbytes / wgs / (us.value * mhz.value):16.1f}')
+        nbytes = 65536.0 * iters * wgs * (2 if form == 2 else 1)
+        print(f'{ws / 2**20:8.0f} MiB  {names[form]:20s} {wgs:10d} {us.value:8.1f} '
+              f'{nbytes / us.value / 1e6:6.2f} {nbytes / us.value / 1e3 / min(wgs, 256):11.1f} {mhz.value:5.0f} '
+              f'{nbytes / min(wgs, 256) / (us.value * mhz.value):16.1f}')
 
 
 def bench_decoder(cfg, args):

@@ -450,11 +450,15 @@ int sub_op_ln_backward_static(void* handle, int extended, const void* in, const 
 /* Measurement only, no counterpart in the reference and no handle: `workgroups` workgroups of eight waves
  * (one per CU at 256) each read `iters` chunks of 64 KiB -- the operand bytes of one k-step of a 256 x 256
  * tile -- from the `working_set` bytes at buf (device memory, a multiple of 64 KiB), with asynchronous loads
- * into LDS (to_lds != 0) or plain 128-bit loads into registers, every workgroup from a start of its own.
- * A working set below one XCD's 4 MiB of L2 measures what the L2s deliver to the CUs, a larger one the path
- * beyond them.  *us = duration of the launch (second of two), *mhz = shader clock during it (median over the
- * workgroups of cycle counter / wall counter).  Bytes read = workgroups x iters x 65536.  Allocates and frees a
- * few KiB per call and synchronises the stream. */
+ * into LDS (to_lds = 1) or plain 128-bit loads into registers (to_lds = 0), every workgroup from a start of
+ * its own.  A working set below one XCD's 4 MiB of L2 measures what the L2s deliver to the CUs, a larger one
+ * the path beyond them.  to_lds = 2: a copy instead -- every chunk read is also written, to the `working_set`
+ * bytes behind the first (buf holds 2 x working_set; nontemporal accesses, as the fused operators use them for
+ * tensors on their last read or written for a later pass); to_lds = 3: only those writes (a fill).  In these
+ * two forms workgroup w takes chunks w, w + workgroups, ...: with workgroups x iters = working_set / 65536 every
+ * chunk is touched once.  *us = duration of the launch (second of two), *mhz = shader clock during it (median
+ * over the workgroups of cycle counter / wall counter).  Bytes read (and/or written) = workgroups x iters x
+ * 65536.  Allocates and frees a few KiB per call and synchronises the stream. */
 int sub_probe_fetch(const void* buf, size_t working_set, int to_lds, int iters, int workgroups, void* stream,
                     float* us, float* mhz);
 /* dst (order l_dst) = src (order l_src): the same tensor in another dimension order (any two permutations

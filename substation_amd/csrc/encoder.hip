@@ -2028,7 +2028,7 @@ int sub_probe_fetch(const void* buf, size_t working_set, int to_lds, int iters, 
             float ms = 0.f;
             for (int rep = 0; rep < 2; ++rep) {       // the second launch is the one measured
                 hip_check(hipEventRecord(e0, st), "hipEventRecord");
-                launch_fetch_probe(buf, working_set, to_lds != 0, iters, workgroups, stamps, sink, st);
+                launch_fetch_probe(buf, working_set, to_lds, iters, workgroups, stamps, sink, st);
                 hip_check(hipEventRecord(e1, st), "hipEventRecord");
                 hip_check(hipEventSynchronize(e1), "hipEventSynchronize");
                 hip_check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");

@@ -204,9 +204,10 @@ void launch_relayout_batch(const RelayoutJob* jobs, int n, hipStream_t st);
 
 // --- measurement --------------------------------------------------------------
 // `workgroups` workgroups of eight waves each read `iters` chunks of 64 KiB from a working set of
-// `working_set` bytes at buf (into LDS with asynchronous loads, or into registers); every workgroup leaves
+// `working_set` bytes at buf (form 0: into registers, 1: into LDS with asynchronous loads), copy them into the
+// `working_set` bytes behind (form 2) or only write those (form 3); every workgroup leaves
 // (cycle counter, wall counter) at its start and end in stamps[4 * workgroup ..].
-void launch_fetch_probe(const void* buf, size_t working_set, bool to_lds, int iters, int workgroups,
+void launch_fetch_probe(const void* buf, size_t working_set, int form, int iters, int workgroups,
                         unsigned long long* stamps, int* sink, hipStream_t st);
 
 // --- tensor contraction ------------------------------------------------------
