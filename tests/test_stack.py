@@ -123,6 +123,14 @@ def test_checkpoint_moves_between_layout_configurations():
     ya, yb = a(xa), b(xb)
     from_b = [lay_b['output'][1].index(d) for d in 'BJI']
     assert_close(yb.detach().permute(from_b).float().cpu().numpy(), ya.detach().float().cpu().numpy(), tol=1e-2, name='Y')
+    # and back: the same output gradient through both stacks (under the reference's configuration every layer
+    # runs in the library's own orders and copies what crosses its boundary)
+    DY = torch.randn(2, 128, 128, generator=g).half()
+    ya.backward(DY.cuda())
+    to_b_out = ['BJI'.index(d) for d in lay_b['output'][1]]
+    yb.backward(DY.permute(to_b_out).contiguous().cuda())
+    from_b_in = [lay_b['input'][1].index(d) for d in 'BJI']
+    assert_close(xb.grad.permute(from_b_in).float().cpu().numpy(), xa.grad.float().cpu().numpy(), tol=1e-2, name='DX')
 
 
 @pytest.mark.gpu
