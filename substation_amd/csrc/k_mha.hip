@@ -480,8 +480,12 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
 // backward, dQ.  grid = H * B * (J / 128); wave = 32 queries.
 // ---------------------------------------------------------------------------
 template <int P, bool MASKED>
-__global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
+__global__ __launch_bounds__(256, (P == 128 && !MASKED) ? 2 : 1) void k_mha_bwd_dq(AttnArgs a) {
     using G = Geo<P>;
+    // Head size 128: with the key and value fragments of a whole tile in registers a tile ahead the kernel
+    // needs 300 registers per lane and runs one wave per SIMD; read two k-slices ahead of their use instead,
+    // it fits 256 and two waves share a SIMD.
+    constexpr bool JIT = P == 128 && !MASKED;
     __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
     __shared__ __attribute__((aligned(16))) half_t vt[RING][G::TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
@@ -526,8 +530,10 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         if (hi == 0) a.dsum[row] = dsum;
     }
     __syncthreads();
-    row_frags_lds<P>(kt[0], l32, hi, fk);
-    row_frags_lds<P>(vt[0], l32, hi, fv);
+    if constexpr (!JIT) {
+        row_frags_lds<P>(kt[0], l32, hi, fk);
+        row_frags_lds<P>(vt[0], l32, hi, fv);
+    }
 
     f16v dq[G::NPT];
 #pragma unroll
@@ -553,17 +559,34 @@ __global__ __launch_bounds__(256) void k_mha_bwd_dq(AttnArgs a) {
         for (int v = 0; v < 16; ++v) { s[v] = 0.f; dp[v] = 0.f; }
         if (from_mask) start_from_mask(mk, s);
         if (MASKED && i + 1 < n && entry_class(e1, wave) != BLOCK_CLEAR) load_mask<true>(a, j, entry_tile(e1) * 32, hi, mk);
+        if constexpr (JIT) {
+            h8 ck[2], cv[2];
+            ck[0] = *reinterpret_cast<const h8*>(kt[cur] + G::at(l32, hi));
+            cv[0] = *reinterpret_cast<const h8*>(vt[cur] + G::at(l32, hi));
 #pragma unroll
-        for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
+            for (int ks = 0; ks < G::NKS; ++ks) {
+                if (ks + 1 < G::NKS) {
+                    ck[(ks + 1) & 1] = *reinterpret_cast<const h8*>(kt[cur] + G::at(l32, 2 * (ks + 1) + hi));
+                    cv[(ks + 1) & 1] = *reinterpret_cast<const h8*>(vt[cur] + G::at(l32, 2 * (ks + 1) + hi));
+                }
+                s = __builtin_amdgcn_mfma_f32_32x32x16_f16(ck[ks & 1], fq[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(cv[ks & 1], fdo[ks], dp, 0, 0, 0);
+            }
+        } else {
 #pragma unroll
-        for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fv[ks], fdo[ks], dp, 0, 0, 0);
+            for (int ks = 0; ks < G::NKS; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_f16(fk[ks], fq[ks], s, 0, 0, 0);
+#pragma unroll
+            for (int ks = 0; ks < G::NKS; ++ks) dp = __builtin_amdgcn_mfma_f32_32x32x16_f16(fv[ks], fdo[ks], dp, 0, 0, 0);
+        }
         h8 ka[2][G::NPT];
 #pragma unroll
         for (int st = 0; st < 2; ++st)
 #pragma unroll
             for (int pt = 0; pt < G::NPT; ++pt) ka[st][pt] = tr_frag<P>(kt[cur], pt * 32, st, lane);
-        row_frags_lds<P>(kt[nxt], l32, hi, fk);
-        row_frags_lds<P>(vt[nxt], l32, hi, fv);
+        if constexpr (!JIT) {
+            row_frags_lds<P>(kt[nxt], l32, hi, fk);
+            row_frags_lds<P>(vt[nxt], l32, hi, fv);
+        }
         const uint32_t nib = word >> (hi * 4);
         // stage by stage over the 16 scores of the lane, so that consecutive
         // instructions do not depend on one another
