@@ -480,12 +480,12 @@ __global__ __launch_bounds__(256) void k_mha_fwd(AttnArgs a, PhiloxKey key_) {
 // backward, dQ.  grid = H * B * (J / 128); wave = 32 queries.
 // ---------------------------------------------------------------------------
 template <int P, bool MASKED>
-__global__ __launch_bounds__(256, (P == 128 && !MASKED) ? 2 : 1) void k_mha_bwd_dq(AttnArgs a) {
+__global__ __launch_bounds__(256, !MASKED ? (P == 128 ? 2 : 3) : 1) void k_mha_bwd_dq(AttnArgs a) {
     using G = Geo<P>;
     // Head size 128: with the key and value fragments of a whole tile in registers a tile ahead the kernel
     // needs 300 registers per lane and runs one wave per SIMD; read two k-slices ahead of their use instead,
     // it fits 256 and two waves share a SIMD.
-    constexpr bool JIT = P == 128 && !MASKED;
+    constexpr bool JIT = !MASKED;
     __shared__ __attribute__((aligned(16))) half_t kt[RING][G::TILE];
     __shared__ __attribute__((aligned(16))) half_t vt[RING][G::TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, hi = lane >> 5;
