@@ -5,7 +5,13 @@
 A step is one forward + one backward pass of a single encoder layer over one
 batch of synthetic input (the protocol of pytorch_module/run_encoder.py:345-383).
 The default workload is BERT-large B=8 L=512 H=16 E=1024 fp16 with the four
-dropouts at p=0.1.  Prints ONE JSON line: ms per layer, the per-launch
+dropouts at p=0.1.  The timed region -- W untimed steps, then K steps between
+two synchronisations on the host clock -- is run twice: as the process finds
+the device (`cold_start_ms_per_step`) and again behind 150 ms of the same
+steps (`value`: a device left idle for a few tens of milliseconds is slow for
+the next 10-20 ms of work, and the figure to compare with the reference's
+medians over 1000 iterations is the steady one; --preheat-ms 0 makes `value`
+the cold figure).  Prints ONE JSON line: ms per layer, the per-launch
 roofline measured live with HIP events on the launch stream, and the CPU
 baseline (the NumPy oracle on the bench workload and on the reference's own
 CPU-sized case).  --config 2 times the fused operators on their own (softmax
@@ -607,28 +613,51 @@ def make_step(enc, X, DY):
     return step
 
 
-def spin(ms, _state={}):
-    """Keeps the current stream busy for about `ms` milliseconds with a spin kernel (what the
-    reference's gpuwait/wait_kernel.cu is for): the host issues the launches that follow while it
-    runs, so they execute back to back whatever the host's issue rate.  The kernel counts clock
-    ticks and ends by itself; its rate is measured once."""
+def lead_steps(ms_per_step):
+    """How many steps to issue in front of a measured one so that the host is a whole step ahead of
+    the GPU when the measured step begins (the host issues a step in roughly half the time the GPU
+    takes for it; fewer for long steps)."""
+    return max(3, min(10, int(6.0 / max(ms_per_step, 0.05)) + 1))
+
+
+def preheat(step, ms_per_step, ms=150.0):
+    """Runs the step itself for about `ms` milliseconds.  After an idle period of a few tens of
+    milliseconds the device is slow for the next ten to twenty milliseconds of work (0.55 ms per
+    step falling to 0.49 at the bench workload, measured; a spin kernel does not prevent it, real
+    memory traffic does): whatever is to be compared with steady-state figures -- the reference's are
+    medians of 1000 iterations after 100 warm-ups, pytorch_module/run_encoder.py:34-38 -- is measured
+    behind this."""
     import torch
-    if 'ticks_per_ms' not in _state:
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda._sleep(1000)
-        torch.cuda.synchronize()
-        e0.record(); torch.cuda._sleep(1_000_000); e1.record()
-        torch.cuda.synchronize()
-        _state['ticks_per_ms'] = 1_000_000 / max(e0.elapsed_time(e1), 1e-3)
-    torch.cuda._sleep(int(min(ms, 200.0) * _state['ticks_per_ms']))
+    n = int(ms / max(ms_per_step, 0.05)) + 1
+    for _ in range(n):
+        step()
+    torch.cuda.synchronize()
+    return n
 
 
-def gpu_step_us(step, n, lead_ms):
-    """GPU time of one step in microseconds: n steps issued behind a spin kernel of about n * lead_ms,
-    from an event in front of the first to one behind the last."""
+def timed_steps(step, steps, warmup):
+    """The timed region: `warmup` untimed steps, then `steps` steps between two synchronisations on
+    the host clock; ms per step."""
+    import torch
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def gpu_step_us(step, n, lead):
+    """GPU time of one step in microseconds: n steps behind `lead` steps of the same workload (which
+    keep the device at its working clocks and give the host its lead, so that the figure does not
+    depend on how fast this host issues launches), from an event in front of the first to one
+    behind the last."""
     import torch
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    spin(n * lead_ms)
+    for _ in range(lead):
+        step()
     e0.record()
     for _ in range(n):
         step()
@@ -637,28 +666,33 @@ def gpu_step_us(step, n, lead_ms):
     return e0.elapsed_time(e1) * 1e3 / n
 
 
-def pass_times(enc, X, DY, n, lead_ms):
+def pass_times(enc, X, DY, n, lead):
     """Forward and backward pass timed apart, as pytorch_module/run_encoder.py:359-383 does: an event
-    before the forward call, one between the passes, one after the backward call, n steps; median,
-    min, max and standard deviation of each pass in ms (the three events of a step cost a few
-    microseconds, which stay in the figures)."""
+    before the forward call, one between the passes, one after the backward call, n steps in a row
+    behind `lead` untimed ones; median, min, max and standard deviation of each pass in ms (the
+    three events of a step cost a few microseconds, which stay in the figures)."""
     import torch
     params = list(enc.parameters())
-    done = []
-    for first in range(0, n, 10):              # ten steps at a time behind one spin kernel
-        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(min(10, n - first))]
-        spin(len(evs) * lead_ms)
-        for a, b, c in evs:
-            X.grad = None
-            for q in params:
-                q.grad = None
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(n)]
+
+    def one(a=None, b=None, c=None):
+        X.grad = None
+        for q in params:
+            q.grad = None
+        if a is not None:
             a.record()
-            Y = enc(X)
+        Y = enc(X)
+        if b is not None:
             b.record()
-            Y.backward(DY)
+        Y.backward(DY)
+        if c is not None:
             c.record()
-        torch.cuda.synchronize()
-        done += [(a.elapsed_time(b), b.elapsed_time(c)) for a, b, c in evs]
+    for _ in range(lead):
+        one()
+    for a, b, c in evs:
+        one(a, b, c)
+    torch.cuda.synchronize()
+    done = [(a.elapsed_time(b), b.elapsed_time(c)) for a, b, c in evs]
     out = {}
     for name, ts in (('forward', [d[0] for d in done]), ('backward', [d[1] for d in done])):
         out[name] = {'median_ms': round(statistics.median(ts), 4), 'min_ms': round(min(ts), 4),
@@ -670,28 +704,25 @@ def pass_times(enc, X, DY, n, lead_ms):
 def other_workloads(args):
     """The BASELINE workloads the headline figure does not cover, each for a fraction of a second of GPU
     time: configs[3] and configs[4] as ms per layer (the headline's protocol -- warm-ups, then steps
-    between two synchronisations on the host clock -- and the GPU's own time per step behind a spin
-    kernel), configs[1] as the fused operators standing alone on buffers larger than the memory-side cache."""
+    between two synchronisations on the host clock, behind the same preheating -- and the GPU's own time per
+    step), configs[1] as the fused operators standing alone on buffers larger than the memory-side cache."""
     import torch
     out = {}
     for cid, steps, warmup in ((4, 20, 5), (5, 6, 2)):
         cfg = dict(CONFIGS[cid])
         enc, X, DY = make_encoder(cfg, args.layouts)
         step = make_step(enc, X, DY)
-        for _ in range(warmup):
-            step()
+        step()                                   # (allocations)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        ms = (time.perf_counter() - t0) * 1e3 / steps
-        gpu_ms = gpu_step_us(step, min(steps, 10), 1.2 * ms) * 1e-3
+        pre = preheat(step, 1.3 if cid == 4 else 11.0)           # building the layer left the device idle
+        ms = timed_steps(step, steps, warmup)
+        gpu_ms = gpu_step_us(step, min(steps, 10), lead_steps(ms)) * 1e-3
         U, P = 4 * cfg['E'], cfg['E'] // cfg['H']
         flops = 3 * (2 * cfg['B'] * cfg['L'] * (4 * cfg['E'] ** 2 + 2 * cfg['E'] * U)
                      + 4 * cfg['B'] * cfg['H'] * cfg['L'] ** 2 * P)
         out['configs[%d]' % (cid - 1)] = {'workload': cfg['name'], 'ms_per_layer': round(ms, 4),
                                           'gpu_ms_per_layer': round(gpu_ms, 4), 'steps': steps, 'warmup': warmup,
+                                          'preheat_steps': pre,
                                           'tflops': round(flops / (gpu_ms * 1e-3) / 1e12, 1),
                                           'frac_of_mfma_peak': round(flops / (gpu_ms * 1e-3) / MFMA_PEAK_F16, 4)}
         del enc, X, DY, step
@@ -722,6 +753,10 @@ def main():
     ap.add_argument('--copy-calibration', action='store_true',
                     help='also run 5 device copies of 256 MiB (known traffic) for scaling rocprofv3 '
                          'FETCH_SIZE / WRITE_SIZE readings')
+    ap.add_argument('--preheat-ms', type=float, default=None,
+                    help='milliseconds of the workload itself run before the timed region is repeated for `value` '
+                         '(default 150; 0: `value` is the cold-start figure; with --profile-steps 0 the default is 0 and '
+                         'the one timed region runs behind the preheating)')
     ap.add_argument('--fetch-probe', action='store_true',
                     help='measure what the CUs draw from the L2s and from beyond them (a table, no JSON line)')
     ap.add_argument('--activation', choices=['relu', 'gelu'], default=None,
@@ -759,14 +794,25 @@ def main():
         enc._handle.set_option(int(k), int(v))
     step = make_step(enc, X, DY)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    # The timed region twice: as the process finds the device (idle since the module was built), and again
+    # behind 150 ms of the same steps.  The second is `value`: the steady state, which is what the reference's
+    # published figures are; the first is kept beside it as cold_start_ms_per_step.
+    # (Timing-only runs, --profile-steps 0, are what the profiler is pointed at: one timed region, behind the
+    # preheating when --preheat-ms is given.)
+    timing_only = args.profile_steps <= 0
+    preheat_ms = args.preheat_ms if args.preheat_ms is not None else (0.0 if timing_only else 150.0)
+    preheat_steps = 0
+    if timing_only:
+        if preheat_ms > 0:
+            step()
+            torch.cuda.synchronize()
+            preheat_steps = preheat(step, 0.55 * cfg['B'] * cfg['L'] / 4096 * (cfg['E'] / 1024) ** 2, preheat_ms)
+        cold_ms = ms_per_step = timed_steps(step, args.steps, args.warmup)
+    else:
+        cold_ms = ms_per_step = timed_steps(step, args.steps, args.warmup)
+        if preheat_ms > 0:
+            preheat_steps = preheat(step, cold_ms, preheat_ms)
+            ms_per_step = timed_steps(step, args.steps, args.warmup)
 
     if args.copy_calibration:
         a = torch.empty(128 << 20, dtype=torch.float16, device='cuda').normal_()
@@ -778,24 +824,24 @@ def main():
 
     if args.profile_steps <= 0:        # timing only
         print(json.dumps({'metric': 'fwd+bwd ms/layer', 'value': round(ms_per_step, 4), 'unit': 'ms',
-                          'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+                          'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'preheat_steps': preheat_steps,
                           'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False}))
         return
 
-    # Everything below is timed on the GPU's own clock (HIP events on the launch stream) behind a spin
-    # kernel, so that the host has issued the launches before they run: a figure does not depend on how
-    # fast this host issues them.
-    lead_ms = 1.5 * max(ms_per_step, 0.4)
+    # Everything below is timed on the GPU's own clock (HIP events on the launch stream) behind a few steps
+    # of the same workload, so that the host has issued the launches before they run and the device is at its
+    # working clocks: a figure does not depend on how fast this host issues them.
+    lead = lead_steps(ms_per_step)
     # Forward and backward pass apart, an event between them (pytorch_module/run_encoder.py:359-383).
-    passes = pass_times(enc, X, DY, max(10, min(args.steps, 50)), lead_ms)
+    passes = pass_times(enc, X, DY, max(10, min(args.steps, 50)), lead)
     # The cost of the library's per-launch events, calibrated directly: the same steps back to back with
     # and without them, in turns; the difference per launch is taken off every entry below.
     n_cal = 10
     plain, inst = [], []
     for _ in range(3):
-        plain.append(gpu_step_us(step, n_cal, lead_ms))
+        plain.append(gpu_step_us(step, n_cal, lead))
         enc._handle.profile_enable(True)
-        inst.append(gpu_step_us(step, n_cal, 2 * lead_ms))
+        inst.append(gpu_step_us(step, n_cal, lead))
         enc._handle.profile_enable(False)
     gpu_us_per_step = statistics.median(plain)
     # Per-launch durations: an event in front of every launch and one at the end of each pass, a launch
@@ -803,9 +849,8 @@ def main():
     enc._handle.profile_enable(True)
     per_op = {}
     for _ in range(args.profile_steps):
-        spin(2 * 2 * lead_ms)
-        step()
-        step()
+        for _ in range(lead + 1):          # the last one is read
+            step()
         for n, ms in enc.profile():
             per_op.setdefault(n, []).append(ms)
     # The shader clock the GPU held during each launch (a one-lane kernel in front of every launch samples the
@@ -813,9 +858,8 @@ def main():
     enc._handle.profile_enable(2)
     clocks = {}
     for _ in range(min(5, args.profile_steps)):
-        spin(2 * 2 * lead_ms)
-        step()
-        step()
+        for _ in range(lead + 1):
+            step()
         for n, mhz in enc._handle.profile_read_clocks():
             clocks.setdefault(n, []).append(mhz)
     enc._handle.profile_enable(False)
@@ -878,6 +922,8 @@ def main():
         'value': round(ms_per_step, 4), 'unit': 'ms', 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4), 'higher_is_better': False,
         'scaling': 'weak', 'vs_baseline': round(ms_per_step / V100_MS, 4) if headline else None,
+        # the same timed region as the process found the device, before `preheat_steps` steps of the workload
+        'cold_start_ms_per_step': round(cold_ms, 4), 'preheat_steps': preheat_steps,
         'dtype': 'fp16', 'data': 'synthetic',
         'config': {'workload': cfg['name'], 'layouts': args.layouts,
                    'baseline': 'reference README.md:23: 6.71 ms on V100-SXM2 (other hardware)'},
@@ -888,7 +934,7 @@ def main():
                         and not args.option else None),
             'launch_us': dom['us'], 'launches_per_step': 1,
         },
-        # GPU time of a step without and with the per-launch events, steps back to back behind a spin kernel;
+        # GPU time of a step without and with the per-launch events, steps back to back;
         # their difference per launch is what was taken off every entry of `ops`
         'gpu_us_per_step': round(gpu_us_per_step, 1), 'gpu_us_per_step_with_events': round(statistics.median(inst), 1),
         'op_time_us': round(total_us, 1), 'event_us_per_launch': round(event_us, 2),
