@@ -1223,8 +1223,13 @@ void launch_mfma(const GemmArgs& a, bool akc, bool bkc, long batch, bool dma, hi
     dim3 grid((unsigned)nblocks + a.side_blocks);
     const bool full = a.M % (64 * TM) == 0 && a.N % (64 * TN) == 0 && a.K1 % BK == 0;
     if (DMA_OK && full && dma && a.splits == 1) { launch_dma<TM, TN>(a, akc, bkc, grid, st); return; }
-    if (full) launch_mfma2<TM, TN, true>(a, akc, bkc, grid, st);
-    else launch_mfma2<TM, TN, false>(a, akc, bkc, grid, st);
+    if constexpr (TM * TN >= 16) {
+        // 256 x 256 tiles exist in the asynchronous kernel only; pick_tile chooses them for whole tiles alone
+        fail("gemm: 256x256 tiles need whole tiles and an unsplit contraction");
+    } else {
+        if (full) launch_mfma2<TM, TN, true>(a, akc, bkc, grid, st);
+        else launch_mfma2<TM, TN, false>(a, akc, bkc, grid, st);
+    }
     if (a.splits > 1) {
         long n = batch * (long)a.M * (a.N / 4);
         hipLaunchKernelGGL(k_gemm_splitk_reduce, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a, batch);
